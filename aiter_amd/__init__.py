@@ -1,0 +1,39 @@
+"""MI355X-native FP8 block-scale path behind the reference's Python entry points.
+
+    y, s = aiter_amd.get_hip_quant(aiter_amd.QuantType.per_1x128)(x, quant_dtype=aiter_amd.dtypes.fp8)
+    out  = aiter_amd.gemm_a8w8_blockscale(y, wq, s, w_scale, dtype=torch.bfloat16)
+    aiter_amd.rmsnorm2d_fwd_with_dynamicquant(out8, x, yscale, weight, eps, 0, group_size=128)
+
+Everything computes in ``libaiter_fp8bs.so`` (hand-written HIP for gfx950, C ABI declared in
+``include/aiter_fp8bs.h``).  There is no other backend and no CPU fallback.
+"""
+
+from . import dtypes
+from .enums import QuantType
+from .gemm_op_a8w8 import gemm_a8w8_blockscale, gemm_a8w8_blockscale_ck, gemm_kernel_names
+from .quant import dynamic_per_token_scaled_quant, get_hip_quant, per_group_quant_hip
+from .rmsnorm import (
+    add_rmsnorm,
+    add_rmsnorm_quant,
+    rmsnorm,
+    rmsnorm2d_fwd_with_add_dynamicquant,
+    rmsnorm2d_fwd_with_dynamicquant,
+    rmsnorm_quant,
+)
+
+__all__ = [
+    "dtypes",
+    "QuantType",
+    "get_hip_quant",
+    "per_group_quant_hip",
+    "dynamic_per_token_scaled_quant",
+    "gemm_a8w8_blockscale",
+    "gemm_a8w8_blockscale_ck",
+    "gemm_kernel_names",
+    "rmsnorm",
+    "rmsnorm_quant",
+    "add_rmsnorm",
+    "add_rmsnorm_quant",
+    "rmsnorm2d_fwd_with_dynamicquant",
+    "rmsnorm2d_fwd_with_add_dynamicquant",
+]

@@ -1,0 +1,264 @@
+// Block-scale FP8 GEMM for gfx950:  Out[m,n] = sum_kb dot(XQ[m,kb], WQ[n,kb]) * xs[m,kb] * ws[n/128,kb]
+//
+// Replaces the CK / CK-Tile device ops behind gemm_a8w8_blockscale
+// (csrc/ck_gemm_a8w8_blockscale/include/gemm_a8w8_blockscale_common.cuh:97-176,
+//  ..._cktile_common.cuh:121-140); semantics as in
+// aiter/ops/triton/_triton_kernels/gemm/basic/gemm_a8w8_blockscale.py:160-190:
+// one exact fp8 dot product per 128-wide K block, scaled in fp32 and accumulated in fp32.
+//
+// MFMA mapping.  v_mfma_f32_16x16x128_f8f6f4 consumes one whole 128-wide K block, so one
+// instruction yields exactly the unscaled partial product of a 16x16 output tile for one
+// scale block.  The weight rows play the MFMA "A" role and the activation rows the "B" role:
+// a lane then owns 4 consecutive n for one m, which makes (a) the scale of its 4 accumulators
+// one scalar per lane, xs[m,kb]*ws[nb,kb], and (b) its output 4 consecutive 16-bit values.
+#include "fp8bs_launch.h"
+
+#include <string.h>
+
+namespace fp8bs {
+
+typedef int      i32x8 __attribute__((ext_vector_type(8)));
+typedef int      i32x4 __attribute__((ext_vector_type(4)));
+typedef float    f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ f32x4 mfma_16x16x128_fp8(const i32x8& a, const i32x8& b, const f32x4& c)
+{
+    // cbsz = blgp = 0 selects e4m3 for both operands; zero scale operands select the
+    // unscaled instruction
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
+template <In16 DT>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi)
+{
+    if constexpr(DT == In16::bf16)
+    {
+        __bf16 a = (__bf16)lo, b = (__bf16)hi;
+        return (uint32_t)__builtin_bit_cast(unsigned short, a) |
+               ((uint32_t)__builtin_bit_cast(unsigned short, b) << 16);
+    }
+    else
+    {
+        _Float16 a = (_Float16)lo, b = (_Float16)hi;
+        return (uint32_t)__builtin_bit_cast(unsigned short, a) |
+               ((uint32_t)__builtin_bit_cast(unsigned short, b) << 16);
+    }
+}
+
+struct GemmKernelParams
+{
+    const uint8_t* xq;
+    const uint8_t* wq;
+    const float*   xs;
+    const float*   ws;
+    uint16_t*      out;
+    int32_t        M, N, K;
+    int64_t        lda, ldb;
+    int32_t        kblocks; // K / 128
+};
+
+// LDS tile: rows of 128 bytes (one K block); the 16-byte chunk c of row r lives at chunk
+// c ^ (r & 7) so that the 16 rows a quarter-wave reads with one ds_read_b128 spread over banks.
+__device__ __forceinline__ uint32_t lds_off(uint32_t row, uint32_t chunk)
+{
+    return row * 128u + ((chunk ^ (row & 7u)) << 4);
+}
+
+// ---------------------------------------------------------------- generic tile kernel
+// BM x BN output tile per block (m = activation rows, n = weight rows), WAVES_M x WAVES_N
+// waves, single-buffered LDS.  Handles every shape (ragged M and N); used for small and odd
+// problems and as the always-available fallback.
+template <In16 DT, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_kernel(GemmKernelParams p)
+{
+    constexpr int T  = 64 * WAVES_M * WAVES_N;
+    constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;
+    constexpr int MT = TM / 16, NT = TN / 16;
+    static_assert(TM % 16 == 0 && TN % 16 == 0, "wave tile must be a multiple of 16x16");
+
+    __shared__ __attribute__((aligned(16))) uint8_t sW[BN * 128];
+    __shared__ __attribute__((aligned(16))) uint8_t sX[BM * 128];
+
+    const int t    = threadIdx.x;
+    const int lane = t & 63, wave = t >> 6;
+    const int wm = (wave % WAVES_M) * TM, wn = (wave / WAVES_M) * TN;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int l16 = lane & 15, kg = lane >> 4;
+
+    f32x4 acc[NT][MT];
+#pragma unroll
+    for(int i = 0; i < NT; ++i)
+#pragma unroll
+        for(int j = 0; j < MT; ++j)
+            acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // rows of x_scale this lane needs (one per m tile), clamped for ragged M
+    int mrow[MT];
+#pragma unroll
+    for(int j = 0; j < MT; ++j)
+    {
+        int m   = m0 + wm + j * 16 + l16;
+        mrow[j] = m < p.M ? m : p.M - 1;
+    }
+    int nblk[NT];
+#pragma unroll
+    for(int i = 0; i < NT; ++i)
+    {
+        int n   = n0 + wn + i * 16;
+        n       = n < p.N ? n : p.N - 1;
+        nblk[i] = n >> 7;
+    }
+
+    for(int kb = 0; kb < p.kblocks; ++kb)
+    {
+        // global -> LDS, 16-byte chunks; 8 consecutive lanes cover one 128-byte row segment
+        for(int q = t; q < BN * 8; q += T)
+        {
+            int row = q >> 3, c = q & 7;
+            int n   = n0 + row;
+            n       = n < p.N ? n : p.N - 1;
+            u32x4 d = *(const u32x4*)(p.wq + (size_t)n * p.ldb + (size_t)kb * 128 + c * 16);
+            *(u32x4*)(sW + lds_off(row, c)) = d;
+        }
+        for(int q = t; q < BM * 8; q += T)
+        {
+            int row = q >> 3, c = q & 7;
+            int m   = m0 + row;
+            m       = m < p.M ? m : p.M - 1;
+            u32x4 d = *(const u32x4*)(p.xq + (size_t)m * p.lda + (size_t)kb * 128 + c * 16);
+            *(u32x4*)(sX + lds_off(row, c)) = d;
+        }
+        __syncthreads();
+
+        i32x8 bx[MT];
+#pragma unroll
+        for(int j = 0; j < MT; ++j)
+        {
+            uint32_t row = wm + j * 16 + l16;
+            i32x4    lo  = *(const i32x4*)(sX + lds_off(row, 2 * kg));
+            i32x4    hi  = *(const i32x4*)(sX + lds_off(row, 2 * kg + 1));
+            bx[j]        = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+        float sc[MT];
+#pragma unroll
+        for(int j = 0; j < MT; ++j)
+            sc[j] = p.xs[(size_t)mrow[j] * p.kblocks + kb];
+
+#pragma unroll
+        for(int i = 0; i < NT; ++i)
+        {
+            uint32_t row = wn + i * 16 + l16;
+            i32x4    lo  = *(const i32x4*)(sW + lds_off(row, 2 * kg));
+            i32x4    hi  = *(const i32x4*)(sW + lds_off(row, 2 * kg + 1));
+            i32x8    aw  = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            float    wsc = p.ws[(size_t)nblk[i] * p.kblocks + kb];
+#pragma unroll
+            for(int j = 0; j < MT; ++j)
+            {
+                f32x4 part = mfma_16x16x128_fp8(aw, bx[j], f32x4{0.f, 0.f, 0.f, 0.f});
+                float s    = sc[j] * wsc;
+#pragma unroll
+                for(int r = 0; r < 4; ++r)
+                    acc[i][j][r] = __builtin_fmaf(part[r], s, acc[i][j][r]);
+            }
+        }
+        __syncthreads();
+    }
+
+    // epilogue: lane holds out[m][n .. n+3]
+#pragma unroll
+    for(int j = 0; j < MT; ++j)
+    {
+        int m = m0 + wm + j * 16 + l16;
+        if(m >= p.M)
+            continue;
+#pragma unroll
+        for(int i = 0; i < NT; ++i)
+        {
+            int       n   = n0 + wn + i * 16 + kg * 4;
+            uint16_t* dst = p.out + (size_t)m * p.N + n;
+            if(n + 3 < p.N && (p.N & 3) == 0)
+            {
+                u32x2 v = u32x2{pack2<DT>(acc[i][j][0], acc[i][j][1]),
+                                pack2<DT>(acc[i][j][2], acc[i][j][3])};
+                *(u32x2*)dst = v;
+            }
+            else
+            {
+#pragma unroll
+                for(int r = 0; r < 4; ++r)
+                    if(n + r < p.N)
+                        dst[r] = (uint16_t)(pack2<DT>(acc[i][j][r], 0.f) & 0xffffu);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------- dispatch
+
+template <In16 DT, int BM, int BN, int WAVES_M, int WAVES_N>
+static hipError_t launch_tile(const GemmKernelParams& p, hipStream_t stream)
+{
+    dim3 grid((p.N + BN - 1) / BN, (p.M + BM - 1) / BM);
+    hipLaunchKernelGGL((gemm_tile_kernel<DT, BM, BN, WAVES_M, WAVES_N>), grid,
+                       dim3(64 * WAVES_M * WAVES_N), 0, stream, p);
+    return hipGetLastError();
+}
+
+static const char* const kKernelNames = "tile_16x256,tile_64x128,tile_128x128";
+
+const char* gemm_kernel_names() { return kKernelNames; }
+
+template <In16 DT>
+static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStream_t stream,
+                           const char** why)
+{
+    const char* name = (a.kernel_name && a.kernel_name[0]) ? a.kernel_name : nullptr;
+    if(name == nullptr)
+    {
+        if(a.M <= 16)
+            name = "tile_16x256";
+        else if(a.M <= 64)
+            name = "tile_64x128";
+        else
+            name = "tile_128x128";
+    }
+    if(strcmp(name, "tile_16x256") == 0)
+        return launch_tile<DT, 16, 256, 1, 4>(p, stream);
+    if(strcmp(name, "tile_64x128") == 0)
+        return launch_tile<DT, 64, 128, 2, 2>(p, stream);
+    if(strcmp(name, "tile_128x128") == 0)
+        return launch_tile<DT, 128, 128, 2, 2>(p, stream);
+    *why = "unknown kernelName (see aiter_fp8bs_gemm_kernel_names())";
+    return hipErrorInvalidValue;
+}
+
+hipError_t launch_gemm_blockscale(const GemmArgs& a, hipStream_t stream, const char** why)
+{
+    *why = nullptr;
+    if(a.M == 0 || a.N == 0)
+        return hipSuccess;
+    GemmKernelParams p;
+    p.xq      = a.xq;
+    p.wq      = a.wq;
+    p.xs      = a.xs;
+    p.ws      = a.ws;
+    p.out     = (uint16_t*)a.out;
+    p.M       = (int32_t)a.M;
+    p.N       = (int32_t)a.N;
+    p.K       = (int32_t)a.K;
+    p.lda     = a.lda;
+    p.ldb     = a.ldb;
+    p.kblocks = (int32_t)(a.K / 128);
+    if(a.split_k_log2 > 0)
+    {
+        *why = "splitK > 0 is not available for this kernel";
+        return hipErrorInvalidValue;
+    }
+    return a.out_dtype == In16::bf16 ? dispatch<In16::bf16>(a, p, stream, why)
+                                     : dispatch<In16::fp16>(a, p, stream, why);
+}
+
+} // namespace fp8bs

@@ -1,0 +1,500 @@
+// 1 x G dynamic FP8 group quant, and RMSNorm (optionally with residual add) with or without
+// that quant fused behind it.  gfx950 only.
+//
+// Both kernels are HBM-bound streaming passes: every lane owns 16 consecutive elements of one
+// group (two 16-byte loads of 16-bit floats in, one 16-byte store of fp8 codes out), so a
+// G-element group is held by G/16 neighbouring lanes and its amax is reduced with DPP
+// quad/row permutes -- no LDS, no cross-wave traffic in the quant stage.
+//
+// Reference behaviour replaced: csrc/kernels/quant_kernels.cu:27-167 (group quant kernel) and
+// the absent csrc/kernels/rmsnorm_quant_kernels.cu (contract: csrc/include/rmsnorm_quant.h:9-41).
+// Arithmetic follows the reference's torch definition aiter/ops/quant.py:64-94, not the
+// reference kernel's multiply-by-reciprocal approximation.
+#include "fp8bs_launch.h"
+#include "fp8bs_math.h"
+
+namespace fp8bs {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+// ---------------------------------------------------------------- 16-bit <-> fp32
+
+template <In16 DT>
+__device__ __forceinline__ void unpack8(const u32x4& c, float* v)
+{
+#pragma unroll
+    for(int i = 0; i < 4; ++i)
+    {
+        if constexpr(DT == In16::bf16)
+        {
+            v[2 * i]     = __uint_as_float(c[i] << 16);
+            v[2 * i + 1] = __uint_as_float(c[i] & 0xffff0000u);
+        }
+        else
+        {
+            f16x2 h      = __builtin_bit_cast(f16x2, c[i]);
+            v[2 * i]     = (float)h.x;
+            v[2 * i + 1] = (float)h.y;
+        }
+    }
+}
+
+// round to nearest even to the 16-bit type; returns the raw code
+template <In16 DT>
+__device__ __forceinline__ uint32_t round16(float f)
+{
+    if constexpr(DT == In16::bf16)
+    {
+        __bf16 b = (__bf16)f;
+        return (uint32_t)__builtin_bit_cast(unsigned short, b);
+    }
+    else
+    {
+        _Float16 h = (_Float16)f;
+        return (uint32_t)__builtin_bit_cast(unsigned short, h);
+    }
+}
+
+template <In16 DT>
+__device__ __forceinline__ float widen16(uint32_t code)
+{
+    if constexpr(DT == In16::bf16)
+        return __uint_as_float(code << 16);
+    else
+        return (float)__builtin_bit_cast(_Float16, (unsigned short)code);
+}
+
+// ---------------------------------------------------------------- DPP reductions over a group
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
+}
+
+constexpr int kDppXor1       = 0xB1;  // quad_perm [1,0,3,2]
+constexpr int kDppXor2       = 0x4E;  // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // lane i <- lane 7-i inside each 8 lanes
+constexpr int kDppRowMirror  = 0x140; // lane i <- lane 15-i inside each 16 lanes
+
+// all-reduce max over LPG (1,2,4,8,16) adjacent lanes; every lane ends with the group's value
+template <int LPG>
+__device__ __forceinline__ float group_max_f32(float v)
+{
+    if constexpr(LPG >= 2)
+        v = fmaxf(v, __uint_as_float(dpp_u32<kDppXor1>(__float_as_uint(v))));
+    if constexpr(LPG >= 4)
+        v = fmaxf(v, __uint_as_float(dpp_u32<kDppXor2>(__float_as_uint(v))));
+    if constexpr(LPG >= 8)
+        v = fmaxf(v, __uint_as_float(dpp_u32<kDppHalfMirror>(__float_as_uint(v))));
+    if constexpr(LPG >= 16)
+        v = fmaxf(v, __uint_as_float(dpp_u32<kDppRowMirror>(__float_as_uint(v))));
+    return v;
+}
+
+template <int LPG>
+__device__ __forceinline__ uint32_t group_max_u32(uint32_t v)
+{
+    if constexpr(LPG >= 2)
+        v = max(v, dpp_u32<kDppXor1>(v));
+    if constexpr(LPG >= 4)
+        v = max(v, dpp_u32<kDppXor2>(v));
+    if constexpr(LPG >= 8)
+        v = max(v, dpp_u32<kDppHalfMirror>(v));
+    if constexpr(LPG >= 16)
+        v = max(v, dpp_u32<kDppRowMirror>(v));
+    return v;
+}
+
+// ---------------------------------------------------------------- the quant stage
+// v[16]: this lane's 16 consecutive elements of its group (already widened to fp32).
+// codes: their 16 e4m3fn codes in memory order.  scale: the group's scale (same in all lanes).
+
+// Rare path: group holds NaN/inf, is all zero, or its amax is so small or large that the
+// scale or its reciprocal leaves the normal range.  Everything is done with IEEE divisions and
+// the software conversion.  NaN/inf follow what the host division does in the torch reference:
+// a NaN element keeps its own sign, other elements of a NaN group get the (positive) NaN of
+// the scale; inf/inf is the default NaN, which has the sign bit set on x86.
+template <int LPG>
+__device__ __noinline__ void quant16_slow(const float (&v)[16], u32x4& codes, float& scale)
+{
+    uint32_t mm = 0;
+#pragma unroll
+    for(int i = 0; i < 16; ++i)
+        mm = max(mm, __float_as_uint(v[i]) & 0x7fffffffu);
+    mm = group_max_u32<LPG>(mm); // as integers: NaN > inf > every finite magnitude
+
+    float s;
+    if(mm > 0x7f800000u)
+        s = __uint_as_float(mm | 0x00400000u);
+    else
+    {
+        s = __uint_as_float(mm) / 448.0f;
+        if(s == 0.0f)
+            s = 1.0f;
+    }
+    uint32_t out[4] = {0, 0, 0, 0};
+#pragma unroll
+    for(int i = 0; i < 16; ++i)
+    {
+        uint32_t xb = __float_as_uint(v[i]);
+        uint32_t xa = xb & 0x7fffffffu;
+        uint32_t sg = (xb >> 24) & 0x80u;
+        uint32_t c;
+        if(mm > 0x7f800000u)
+            c = (xa > 0x7f800000u) ? (sg | 0x7fu) : 0x7fu;
+        else if(mm == 0x7f800000u)
+            c = (xa == 0x7f800000u) ? 0xffu : sg;
+        else
+            c = f32_to_e4m3fn_sw(v[i] / s);
+        out[i >> 2] |= c << (8 * (i & 3));
+    }
+    codes = u32x4{out[0], out[1], out[2], out[3]};
+    scale = s;
+}
+
+template <int LPG>
+__device__ __forceinline__ void quant16(const float (&v)[16], u32x4& codes, float& scale)
+{
+    float m  = 0.0f;
+    bool  un = false;
+#pragma unroll
+    for(int i = 0; i < 16; i += 2)
+    {
+        m = fmaxf(fmaxf(m, fabsf(v[i])), fabsf(v[i + 1]));
+        un |= __builtin_isunordered(v[i], v[i + 1]);
+    }
+    // a NaN would be dropped by fmaxf: send the group to the slow path through an infinite amax
+    m = un ? __builtin_inff() : m;
+    m = group_max_f32<LPG>(m);
+
+    if(amax_allows_fast_path(__float_as_uint(m)))
+    {
+        const float s = m / 448.0f; // IEEE division
+        const float r = 1.0f / s;   // IEEE division: the correctly rounded reciprocal
+        uint32_t out[4];
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+        {
+            int w = 0;
+            w = __builtin_amdgcn_cvt_pk_fp8_f32(div_by_scale(v[4 * j], s, r),
+                                                div_by_scale(v[4 * j + 1], s, r), w, false);
+            w = __builtin_amdgcn_cvt_pk_fp8_f32(div_by_scale(v[4 * j + 2], s, r),
+                                                div_by_scale(v[4 * j + 3], s, r), w, true);
+            out[j] = (uint32_t)w;
+        }
+        codes = u32x4{out[0], out[1], out[2], out[3]};
+        scale = s;
+    }
+    else
+    {
+        quant16_slow<LPG>(v, codes, scale);
+    }
+}
+
+// ---------------------------------------------------------------- standalone group quant
+
+struct QuantKernelParams
+{
+    const u32x4*   x;
+    u32x4*         y;
+    float*         scale;
+    uint32_t       rows;
+    uint32_t       groups_per_row;
+    const int32_t* num_rows;
+    int32_t        num_rows_factor;
+    int32_t        transpose_scale;
+};
+
+constexpr int kQuantBlock = 256;
+
+template <In16 DT, int GS, int UNITS>
+__global__ __launch_bounds__(kQuantBlock) void group_quant_kernel(QuantKernelParams p)
+{
+    constexpr int LPG = GS / 16;          // lanes per group
+    constexpr int GPB = kQuantBlock / LPG; // groups per block per unit
+
+    uint32_t rows = p.rows;
+    if(p.num_rows != nullptr)
+    {
+        int64_t lim = (int64_t)(*p.num_rows) * p.num_rows_factor;
+        lim         = lim < 0 ? 0 : lim;
+        rows        = lim < (int64_t)rows ? (uint32_t)lim : rows;
+    }
+    const uint32_t n_groups = rows * p.groups_per_row;
+    const uint32_t lig      = threadIdx.x % LPG;
+    const uint32_t g0       = blockIdx.x * (GPB * UNITS) + threadIdx.x / LPG;
+
+    u32x4 c[UNITS][2];
+#pragma unroll
+    for(int u = 0; u < UNITS; ++u)
+    {
+        const uint32_t g = g0 + u * GPB;
+        if(g < n_groups)
+        {
+            const u32x4* src = p.x + (size_t)g * (GS / 8) + lig * 2;
+            c[u][0]          = __builtin_nontemporal_load(src);
+            c[u][1]          = __builtin_nontemporal_load(src + 1);
+        }
+    }
+#pragma unroll
+    for(int u = 0; u < UNITS; ++u)
+    {
+        const uint32_t g = g0 + u * GPB;
+        if(g < n_groups)
+        {
+            float v[16];
+            unpack8<DT>(c[u][0], v);
+            unpack8<DT>(c[u][1], v + 8);
+            u32x4 codes;
+            float s;
+            quant16<LPG>(v, codes, s);
+            __builtin_nontemporal_store(codes, p.y + (size_t)g * (GS / 16) + lig);
+            if(lig == 0)
+            {
+                size_t idx = g;
+                if(p.transpose_scale)
+                {
+                    uint32_t row = g / p.groups_per_row;
+                    uint32_t col = g - row * p.groups_per_row;
+                    idx          = (size_t)col * rows + row;
+                }
+                p.scale[idx] = s;
+            }
+        }
+    }
+}
+
+template <In16 DT, int GS>
+static hipError_t launch_group_quant_t(const QuantArgs& a, hipStream_t stream)
+{
+    constexpr int UNITS = 2;
+    constexpr int LPG   = GS / 16;
+    constexpr int GPB   = kQuantBlock / LPG * UNITS;
+    QuantKernelParams p;
+    p.x               = (const u32x4*)a.x;
+    p.y               = (u32x4*)a.y;
+    p.scale           = a.scale;
+    p.rows            = (uint32_t)a.rows;
+    p.groups_per_row  = (uint32_t)a.groups_per_row;
+    p.num_rows        = a.num_rows;
+    p.num_rows_factor = a.num_rows_factor;
+    p.transpose_scale = a.transpose_scale ? 1 : 0;
+    const uint64_t n_groups = (uint64_t)a.rows * (uint64_t)a.groups_per_row;
+    if(n_groups == 0)
+        return hipSuccess;
+    const uint32_t grid = (uint32_t)((n_groups + GPB - 1) / GPB);
+    hipLaunchKernelGGL((group_quant_kernel<DT, GS, UNITS>), dim3(grid), dim3(kQuantBlock), 0, stream, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_group_quant(const QuantArgs& a, hipStream_t stream)
+{
+    const bool bf = a.dtype == In16::bf16;
+    switch(a.group)
+    {
+    case 128:
+        return bf ? launch_group_quant_t<In16::bf16, 128>(a, stream)
+                  : launch_group_quant_t<In16::fp16, 128>(a, stream);
+    case 64:
+        return bf ? launch_group_quant_t<In16::bf16, 64>(a, stream)
+                  : launch_group_quant_t<In16::fp16, 64>(a, stream);
+    case 32:
+        return bf ? launch_group_quant_t<In16::bf16, 32>(a, stream)
+                  : launch_group_quant_t<In16::fp16, 32>(a, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+// ---------------------------------------------------------------- RMSNorm (+add) (+quant)
+// One block per row, one lane per 16 consecutive elements (hidden <= 8192 -> <= 512 lanes).
+// The sum of squares is accumulated in fp64 (each 16-bit float square is exact there), so the
+// mean is the correctly rounded one regardless of reduction order up to ~2^-45 relative.
+
+struct NormKernelParams
+{
+    const uint16_t* x;
+    const uint16_t* res_in;
+    uint16_t*       res_out;
+    const uint16_t* weight;
+    uint16_t*       out16;
+    uint8_t*        out8;
+    float*          scale;
+    uint32_t        rows;
+    int32_t         hidden;
+    int64_t         x_stride, res_in_stride, res_out_stride, out_stride;
+    float           eps;
+    int32_t         transpose_scale;
+    int32_t         gemma_norm;
+};
+
+template <In16 DT, bool ADD, int GS /* 0 = no quant */>
+__global__ __launch_bounds__(512) void rmsnorm_kernel(NormKernelParams p)
+{
+    const uint32_t row   = blockIdx.x;
+    const int      t     = threadIdx.x;
+    const int      e0    = t * 16;
+    const bool     act0  = e0 < p.hidden;     // first 8 elements present
+    const bool     act1  = e0 + 8 < p.hidden; // second 8 elements present
+
+    float v[16];
+#pragma unroll
+    for(int i = 0; i < 16; ++i)
+        v[i] = 0.0f;
+
+    if(act0)
+    {
+        const u32x4* src = (const u32x4*)(p.x + (size_t)row * p.x_stride + e0);
+        unpack8<DT>(src[0], v);
+        if(act1)
+            unpack8<DT>(src[1], v + 8);
+        if constexpr(ADD)
+        {
+            float        r[16];
+            const u32x4* rs = (const u32x4*)(p.res_in + (size_t)row * p.res_in_stride + e0);
+            unpack8<DT>(rs[0], r);
+            if(act1)
+                unpack8<DT>(rs[1], r + 8);
+            uint32_t h[16];
+#pragma unroll
+            for(int i = 0; i < 16; ++i)
+            {
+                h[i] = round16<DT>(v[i] + r[i]);
+                v[i] = widen16<DT>(h[i]);
+            }
+            u32x4* ro = (u32x4*)(p.res_out + (size_t)row * p.res_out_stride + e0);
+            ro[0]     = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16),
+                          h[6] | (h[7] << 16)};
+            if(act1)
+                ro[1] = u32x4{h[8] | (h[9] << 16), h[10] | (h[11] << 16), h[12] | (h[13] << 16),
+                              h[14] | (h[15] << 16)};
+        }
+    }
+
+    double ss = 0.0;
+#pragma unroll
+    for(int i = 0; i < 16; ++i)
+        ss = __builtin_fma((double)v[i], (double)v[i], ss);
+#pragma unroll
+    for(int off = 32; off >= 1; off >>= 1)
+        ss += __shfl_xor(ss, off, 64);
+
+    __shared__ double part[8];
+    const int         wave = t >> 6, n_waves = blockDim.x >> 6;
+    if((t & 63) == 0)
+        part[wave] = ss;
+    __syncthreads();
+    double tot = 0.0;
+    for(int w = 0; w < n_waves; ++w)
+        tot += part[w];
+
+    const float mean = (float)(tot / (double)p.hidden);
+    const float rstd = 1.0f / sqrtf(mean + p.eps); // correctly rounded sqrt and division
+
+    if(!act0)
+        return;
+
+    {
+        float        w[16];
+        const u32x4* ws = (const u32x4*)(p.weight + e0);
+        unpack8<DT>(ws[0], w);
+        if(act1)
+            unpack8<DT>(ws[1], w + 8);
+        else
+        {
+#pragma unroll
+            for(int i = 8; i < 16; ++i)
+                w[i] = 0.0f;
+        }
+        uint32_t h[16];
+#pragma unroll
+        for(int i = 0; i < 16; ++i)
+        {
+            float wf = p.gemma_norm ? 1.0f + w[i] : w[i];
+            float tt = v[i] * rstd;
+            float u  = tt * wf;
+            h[i]     = round16<DT>(u);
+            v[i]     = widen16<DT>(h[i]);
+        }
+        if constexpr(GS == 0)
+        {
+            u32x4* o = (u32x4*)(p.out16 + (size_t)row * p.out_stride + e0);
+            o[0]     = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16),
+                         h[6] | (h[7] << 16)};
+            if(act1)
+                o[1] = u32x4{h[8] | (h[9] << 16), h[10] | (h[11] << 16), h[12] | (h[13] << 16),
+                             h[14] | (h[15] << 16)};
+        }
+    }
+
+    if constexpr(GS != 0)
+    {
+        constexpr int LPG = GS / 16;
+        u32x4         codes;
+        float         s;
+        quant16<LPG>(v, codes, s);
+        *(u32x4*)(p.out8 + (size_t)row * p.out_stride + e0) = codes;
+        if(t % LPG == 0)
+        {
+            const uint32_t gpr = (uint32_t)p.hidden / GS;
+            const uint32_t col = (uint32_t)t / LPG;
+            size_t idx = p.transpose_scale ? (size_t)col * p.rows + row : (size_t)row * gpr + col;
+            p.scale[idx] = s;
+        }
+    }
+}
+
+template <In16 DT, bool ADD, int GS>
+static hipError_t launch_rmsnorm_t(const NormKernelParams& p, hipStream_t stream)
+{
+    int lanes   = (p.hidden + 15) / 16;
+    int threads = (lanes + 63) / 64 * 64;
+    hipLaunchKernelGGL((rmsnorm_kernel<DT, ADD, GS>), dim3(p.rows), dim3(threads), 0, stream, p);
+    return hipGetLastError();
+}
+
+template <In16 DT, bool ADD>
+static hipError_t launch_rmsnorm_g(const NormKernelParams& p, int group, hipStream_t stream)
+{
+    switch(group)
+    {
+    case 0: return launch_rmsnorm_t<DT, ADD, 0>(p, stream);
+    case 32: return launch_rmsnorm_t<DT, ADD, 32>(p, stream);
+    case 64: return launch_rmsnorm_t<DT, ADD, 64>(p, stream);
+    case 128: return launch_rmsnorm_t<DT, ADD, 128>(p, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_rmsnorm(const NormArgs& a, hipStream_t stream)
+{
+    if(a.rows == 0)
+        return hipSuccess;
+    NormKernelParams p;
+    p.x               = (const uint16_t*)a.x;
+    p.res_in          = (const uint16_t*)a.residual_in;
+    p.res_out         = (uint16_t*)a.residual_out;
+    p.weight          = (const uint16_t*)a.weight;
+    p.out16           = (uint16_t*)a.out16;
+    p.out8            = a.out8;
+    p.scale           = a.scale;
+    p.rows            = (uint32_t)a.rows;
+    p.hidden          = a.hidden;
+    p.x_stride        = a.x_stride;
+    p.res_in_stride   = a.res_in_stride;
+    p.res_out_stride  = a.res_out_stride;
+    p.out_stride      = a.out_stride;
+    p.eps             = a.eps;
+    p.transpose_scale = a.transpose_scale ? 1 : 0;
+    p.gemma_norm      = a.gemma_norm ? 1 : 0;
+    const int  group  = a.out8 ? a.group : 0;
+    const bool add    = a.residual_in != nullptr;
+    if(a.dtype == In16::bf16)
+        return add ? launch_rmsnorm_g<In16::bf16, true>(p, group, stream)
+                   : launch_rmsnorm_g<In16::bf16, false>(p, group, stream);
+    return add ? launch_rmsnorm_g<In16::fp16, true>(p, group, stream)
+               : launch_rmsnorm_g<In16::fp16, false>(p, group, stream);
+}
+
+} // namespace fp8bs

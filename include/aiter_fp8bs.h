@@ -1,0 +1,151 @@
+/*
+ * C ABI of libaiter_fp8bs.so: the gfx950 (MI355X) implementation of the DeepSeek-style FP8
+ * block-scale path -- 1x128 dynamic FP8 group quant, RMSNorm (+residual add) fused with that
+ * quant, and the 1x128 / 128x128 block-scale FP8 GEMM with bf16/fp16 output.
+ *
+ * Calling convention (the reference's ctypes flavour, aiter/jit/core.py:1306-1323 and
+ * :1595-1612): every tensor is a BORROWED descriptor (`aiter_tensor_t*`, the caller owns the
+ * memory and keeps it alive until the stream has run the work); `Optional[Tensor]` is NULL;
+ * `int` is int64_t, `bool` is int, `float` is float, `str` is const char*; the caller's HIP
+ * stream is the last argument.  Functions only enqueue work on that stream: they never
+ * synchronise and never allocate device memory, so they can be captured into a HIP graph.
+ * Return value: 0 on success, -1 on failure with the message available from
+ * aiter_get_last_error() (thread local).  No C++ exception crosses this boundary.
+ *
+ * Descriptor layout follows csrc/include/aiter_tensor.h:8-17 (160 bytes) and the dtype codes
+ * follow csrc/include/aiter_enum.h:34-51 of the reference, so that the reference's own ctypes
+ * marshalling (aiter/utility/aiter_types.py:68-87, aiter/utility/dtypes.py:101-129) can be
+ * pointed at this library unchanged.
+ */
+#ifndef AITER_FP8BS_H
+#define AITER_FP8BS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* csrc/include/aiter_enum.h:34-51 */
+typedef enum
+{
+    AITER_DTYPE_fp8 = 0, /* OCP e4m3fn on gfx950 */
+    AITER_DTYPE_fp8_e8m0,
+    AITER_DTYPE_fp16,
+    AITER_DTYPE_bf16,
+    AITER_DTYPE_fp32,
+    AITER_DTYPE_i4x2,
+    AITER_DTYPE_fp4x2,
+    AITER_DTYPE_u32,
+    AITER_DTYPE_i32,
+    AITER_DTYPE_i16,
+    AITER_DTYPE_i8,
+    AITER_DTYPE_u8,
+    AITER_DTYPE_i64,
+    AITER_DTYPE_u64
+} AiterDtype;
+
+/* csrc/include/aiter_tensor.h:8-17 */
+typedef struct aiter_tensor_t
+{
+    void*   ptr;        /* device pointer */
+    size_t  numel_;     /* number of elements */
+    int     ndim;       /* 0..8 */
+    int64_t shape[8];
+    int64_t strides[8]; /* in elements */
+    int     dtype_;     /* AiterDtype */
+    int     device_id;  /* GPU ordinal, -1 = host memory */
+} aiter_tensor_t;
+
+/* hipStream_t without pulling the HIP headers into C callers */
+typedef void* aiter_stream_t;
+
+/* ---- error / version plumbing: csrc/include/aiter_ctypes_error.h:59-70 ---- */
+int         aiter_ctypes_abi_version(void); /* == 2 */
+const char* aiter_get_last_error(void);     /* NULL when no error is pending */
+void        aiter_clear_last_error(void);
+
+/*
+ * 1 x G dynamic group quant (G = input.shape[-1] in {32, 64, 128}).
+ * Replaces aiter::dynamic_per_token_scaled_quant, csrc/include/quant.h:18-24 (group branch of
+ * csrc/kernels/quant_kernels.cu:738-804) as bound by aiter/ops/quant.py:754-763.
+ *   out      fp8 [..., K] contiguous                (K = out.shape[-1], K % G == 0)
+ *   input    bf16|fp16, the same memory viewed [-1, G], contiguous
+ *   scales   fp32, numel == input.numel / G; written row-major [rows, K/G], or
+ *            [K/G, rows] when shuffle_scale != 0   (rows = numel(out) / K)
+ *   scale_ub must be NULL (unused by the group branch of the reference)
+ *   num_rows optional int32[1] on the device: only the first num_rows[0]*num_rows_factor rows
+ *            are quantised, the rest of out/scales is left untouched
+ * Arithmetic follows the reference's torch definition (aiter/ops/quant.py:64-94), bit for bit:
+ * scale = amax/448 (exact zero -> 1), code = e4m3fn_rne(x / scale), both IEEE fp32 divisions.
+ */
+int dynamic_per_token_scaled_quant(aiter_tensor_t* out, aiter_tensor_t* input,
+                                   aiter_tensor_t* scales, aiter_tensor_t* scale_ub,
+                                   int shuffle_scale, aiter_tensor_t* num_rows,
+                                   int64_t num_rows_factor, aiter_stream_t stream);
+
+/*
+ * RMSNorm -> bf16|fp16.  Replaces aiter::rmsnorm, csrc/include/rmsnorm_quant.h:37-41
+ * (binding aiter/ops/rmsnorm.py:625-632).
+ *   out, input [rows, hidden] same 16-bit dtype, last dim contiguous; weight [hidden] same dtype
+ *   out = round16( (x * rstd) * w ), rstd = 1/sqrt(mean(x^2) + epsilon), fp32 arithmetic;
+ *   gemma_norm != 0 uses (1 + w).
+ */
+int rmsnorm(aiter_tensor_t* out, aiter_tensor_t* input, aiter_tensor_t* weight, float epsilon,
+            int gemma_norm, aiter_stream_t stream);
+
+/*
+ * RMSNorm fused with the 1 x group_size FP8 quant of its (16-bit rounded) result.
+ * Replaces aiter::rmsnorm_quant, csrc/include/rmsnorm_quant.h:28-35 (binding
+ * aiter/ops/rmsnorm.py:612-622; caller aiter/ops/rmsnorm.py:506-532).
+ *   out fp8 [rows, hidden]; scale fp32 [rows, hidden/group_size] (or transposed when
+ *   shuffle_scale != 0); group_size in {32, 64, 128}; hidden % group_size == 0; hidden <= 8192.
+ * The result is bit-identical to rmsnorm() followed by dynamic_per_token_scaled_quant().
+ */
+int rmsnorm_quant(aiter_tensor_t* out, aiter_tensor_t* input, aiter_tensor_t* scale,
+                  aiter_tensor_t* weight, float epsilon, int64_t group_size, int shuffle_scale,
+                  int gemma_norm, aiter_stream_t stream);
+
+/*
+ * Residual-add variants: residual_out = round16(input + residual_in), then as above on
+ * residual_out.  Replace aiter::add_rmsnorm / aiter::add_rmsnorm_quant,
+ * csrc/include/rmsnorm_quant.h:9-26 (bindings aiter/ops/rmsnorm.py:585-609).
+ */
+int add_rmsnorm(aiter_tensor_t* out, aiter_tensor_t* input, aiter_tensor_t* residual_in,
+                aiter_tensor_t* residual_out, aiter_tensor_t* weight, float epsilon,
+                int gemma_norm, aiter_stream_t stream);
+
+int add_rmsnorm_quant(aiter_tensor_t* out, aiter_tensor_t* input, aiter_tensor_t* residual_in,
+                      aiter_tensor_t* residual_out, aiter_tensor_t* scale,
+                      aiter_tensor_t* weight, float epsilon, int64_t group_size,
+                      int shuffle_scale, int gemma_norm, aiter_stream_t stream);
+
+/*
+ * Block-scale FP8 GEMM.  Replaces gemm_a8w8_blockscale,
+ * csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale.cu:82-114 (binding
+ * aiter/ops/gemm_op_a8w8.py:285-298).
+ *   XQ      fp8 [M, K], row stride honoured (last dim contiguous)
+ *   WQ      fp8 [N, K], row stride honoured (last dim contiguous)
+ *   x_scale fp32 [M, K/128] contiguous
+ *   w_scale fp32 [ceil(N/128), K/128] contiguous
+ *   Out     bf16|fp16 [M, N] contiguous
+ *   Out[m,n] = round16( sum_kb  dot(XQ[m, kb], WQ[n, kb]) * x_scale[m,kb] * w_scale[n/128,kb] )
+ *   with exact fp8 products, fp32 accumulation and one final rounding.  K % 128 == 0.
+ *   splitK: log2 of the number of K partitions (0..4); -1 lets the library choose.
+ *   kernelName: optional tile-kernel name (see aiter_fp8bs_gemm_kernel_names); "" or NULL lets
+ *   the library choose.
+ */
+int gemm_a8w8_blockscale(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t* x_scale,
+                         aiter_tensor_t* w_scale, aiter_tensor_t* Out, int64_t splitK,
+                         const char* kernelName, aiter_stream_t stream);
+
+/* Comma-separated list of the tile kernels gemm_a8w8_blockscale can be asked for by name
+ * (the counterpart of the reference's generated kernel zoo,
+ * csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale_instance.py:73-117). */
+const char* aiter_fp8bs_gemm_kernel_names(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AITER_FP8BS_H */

@@ -1,0 +1,163 @@
+"""GPU parity: block-scale FP8 GEMM through the C-ABI vs the fp32/fp64 oracles."""
+
+import numpy as np
+import pytest
+import torch
+
+import aiter_amd
+from aiter_amd import dtypes
+from oracle import c_oracle as co
+from oracle import torch_ref as tr
+from tests.helpers import codes8, codes16, guarded_empty
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+RTOL = ATOL = 1e-2  # aiter/test_common.py:482-483, op_tests/test_gemm_a8w8_blockscale.py:118
+
+
+def make_problem(m, n, k, seed=0, outliers=0.0):
+    x = tr.make_activation(m, k, seed=seed, outlier_frac=outliers)
+    w = tr.make_weight(n, k, seed=seed + 1)
+    xq, xs = tr.per_1x128_quant(x)
+    wq, ws = tr.weight_per_128x128_quant(w)
+    return xq, wq, xs, ws
+
+
+def run_gpu(xq, wq, xs, ws, dtype=torch.bfloat16, kernel=None, splitK=0):
+    a = [t.to(DEV) for t in (xq, wq, xs, ws)]
+    if kernel is None:
+        out = aiter_amd.gemm_a8w8_blockscale(*a, dtype=dtype)
+    else:
+        out = torch.empty(xq.shape[0], wq.shape[0], dtype=dtype, device=DEV)
+        aiter_amd.gemm_a8w8_blockscale_ck(*a, out, splitK=splitK, kernelName=kernel)
+    torch.cuda.synchronize()
+    return out
+
+
+def assert_close_to_f64(out, xq, wq, xs, ws, what=""):
+    ref = tr.gemm_a8w8_blockscale_ref_f64(xq, wq, xs, ws)
+    o = out.cpu().double()
+    err = (o - ref).abs()
+    bound = ATOL + RTOL * ref.abs()
+    bad = (err > bound).sum().item()
+    assert bad == 0, f"{what}: {bad} of {o.numel()} outside rtol=atol=1e-2, max abs err {err.max().item():.4g}"
+    # much tighter in practice: bf16 rounding (2^-9 relative) plus fp32 accumulation noise
+    rel = err.max().item() / max(ref.abs().max().item(), 1e-30)
+    assert rel < 6e-3, f"{what}: max error / max |ref| = {rel:.3g}"
+
+
+def test_config1_plumbing():
+    # BASELINE config 1: [32,1024] x [512,1024]^T, seed 0
+    xq, wq, xs, ws = make_problem(32, 512, 1024, seed=0)
+    out = run_gpu(xq, wq, xs, ws)
+    assert out.shape == (32, 512) and out.dtype == torch.bfloat16
+    ref32 = tr.gemm_a8w8_blockscale_ref(xq, wq, xs, ws)
+    assert tr.check_allclose_ratio(out.cpu(), ref32, RTOL, ATOL) == 0.0
+    assert_close_to_f64(out, xq, wq, xs, ws, "config1")
+    o64, ob = co.gemm_blockscale(codes8(xq), codes8(wq), xs.numpy(), ws.numpy())
+    # against the scalar C oracle: nearly all bf16 codes identical, never more than one ulp apart
+    d = np.abs(codes16(out).astype(np.int32) - ob.astype(np.int32))
+    assert d.max() <= 1 and (d != 0).mean() < 0.02
+
+
+@pytest.mark.parametrize("kernel", [None, "tile_16x256", "tile_64x128", "tile_128x128"])
+@pytest.mark.parametrize(
+    "m,n,k",
+    [(1, 128, 128), (1, 2112, 512), (16, 256, 1024), (17, 384, 256), (64, 2112, 1024), (130, 520, 384), (257, 1000, 256)],
+)
+def test_shapes_and_tiles(kernel, m, n, k):
+    xq, wq, xs, ws = make_problem(m, n, k, seed=m + n + k)
+    out = run_gpu(xq, wq, xs, ws, kernel=kernel)
+    assert_close_to_f64(out, xq, wq, xs, ws, f"{kernel} {m}x{n}x{k}")
+
+
+def test_one_hot_isolates_single_scale_product():
+    # x has a single non-zero element (m0,k0), w a single non-zero element (n0,k0):
+    # out[m0,n0] must be exactly bf16(x*w*xs*ws) and everything else exactly zero.
+    m, n, k = 48, 384, 512
+    xq = torch.zeros(m, k, dtype=torch.uint8)
+    wq = torch.zeros(n, k, dtype=torch.uint8)
+    g = torch.Generator().manual_seed(0)
+    xs = torch.rand(m, k // 128, generator=g) + 0.5
+    ws = torch.rand((n + 127) // 128, k // 128, generator=g) + 0.5
+    cases = [(0, 0, 0), (47, 383, 511), (17, 200, 300), (31, 129, 127), (5, 255, 128)]
+    for m0, n0, k0 in cases:
+        xq.zero_(); wq.zero_()
+        xq[m0, k0] = 0x40  # 2.0
+        wq[n0, k0] = 0xB4  # -1.25 ... sign + exponent 6, mantissa 4 -> -(1.5)*2^-1 = -0.75
+        out = run_gpu(xq.view(dtypes.fp8), wq.view(dtypes.fp8), xs, ws).cpu().float()
+        a = torch.tensor([0x40], dtype=torch.uint8).view(dtypes.fp8).float().item()
+        b = torch.tensor([0xB4], dtype=torch.uint8).view(dtypes.fp8).float().item()
+        expect = np.float32(a * b) * (xs[m0, k0 // 128].numpy() * ws[n0 // 128, k0 // 128].numpy())
+        assert out[m0, n0].item() == torch.tensor(float(expect)).bfloat16().float().item(), (m0, n0, k0)
+        out[m0, n0] = 0
+        assert torch.count_nonzero(out) == 0, (m0, n0, k0)
+
+
+def test_identity_scales_reduce_to_plain_fp8_gemm():
+    m, n, k = 64, 256, 512
+    g = torch.Generator().manual_seed(3)
+    xq = torch.randint(0, 256, (m, k), generator=g, dtype=torch.int32).to(torch.uint8)
+    wq = torch.randint(0, 256, (n, k), generator=g, dtype=torch.int32).to(torch.uint8)
+    xq[(xq & 0x7F) == 0x7F] = 0x10  # no NaN codes
+    wq[(wq & 0x7F) == 0x7F] = 0x10
+    xq[(xq & 0x78) > 0x50] &= 0x8F  # keep magnitudes small so fp32 sums stay exact-ish
+    wq[(wq & 0x78) > 0x50] &= 0x8F
+    xs = torch.ones(m, k // 128)
+    ws = torch.ones(n // 128, k // 128)
+    out = run_gpu(xq.view(dtypes.fp8), wq.view(dtypes.fp8), xs, ws).cpu().float()
+    ref = (xq.view(dtypes.fp8).double() @ wq.view(dtypes.fp8).double().T)
+    assert torch.allclose(out.double(), ref, rtol=2**-8, atol=1e-6)
+
+
+def test_linear_in_x_scale():
+    # doubling x_scale (exact in fp32) doubles every output bit-exactly (power-of-two scaling)
+    xq, wq, xs, ws = make_problem(40, 384, 768, seed=5)
+    a = run_gpu(xq, wq, xs, ws).cpu().float()
+    b = run_gpu(xq, wq, xs * 2, ws).cpu().float()
+    assert torch.equal(a * 2, b)
+
+
+def test_fp16_output():
+    xq, wq, xs, ws = make_problem(33, 256, 512, seed=8)
+    out = run_gpu(xq, wq, xs, ws, dtype=torch.float16)
+    assert out.dtype == torch.float16
+    ref = tr.gemm_a8w8_blockscale_ref_f64(xq, wq, xs, ws)
+    assert torch.allclose(out.cpu().double(), ref, rtol=RTOL, atol=ATOL)
+
+
+def test_strided_operands_and_guard_bands():
+    m, n, k = 24, 300, 512
+    xq, wq, xs, ws = make_problem(m, n, k, seed=12)
+    xbig = torch.zeros(m, k + 256, dtype=torch.uint8, device=DEV)
+    wbig = torch.zeros(n, k + 128, dtype=torch.uint8, device=DEV)
+    xbig[:, :k] = xq.view(torch.uint8).to(DEV)
+    wbig[:, :k] = wq.view(torch.uint8).to(DEV)
+    out, chk = guarded_empty((m, n), torch.bfloat16, DEV)
+    aiter_amd.gemm_a8w8_blockscale_ck(
+        xbig[:, :k].view(dtypes.fp8), wbig[:, :k].view(dtypes.fp8), xs.to(DEV), ws.to(DEV), out
+    )
+    torch.cuda.synchronize()
+    chk()
+    assert_close_to_f64(out, xq, wq, xs, ws, "strided")
+
+
+@pytest.mark.parametrize("m", [1, 16, 64])
+@pytest.mark.parametrize("n,k", [(7168, 2048), (24576, 1536), (2112, 7168)])
+def test_decode_shapes(m, n, k):
+    # BASELINE config 3
+    xq, wq, xs, ws = make_problem(m, n, k, seed=m + n)
+    out = run_gpu(xq, wq, xs, ws)
+    ref32 = tr.gemm_a8w8_blockscale_ref(xq, wq, xs, ws)
+    assert tr.check_allclose_ratio(out.cpu(), ref32, RTOL, ATOL) == 0.0
+    assert_close_to_f64(out, xq, wq, xs, ws, f"decode {m}x{n}x{k}")
+
+
+def test_fused_config_shape_sampled_rows():
+    # BASELINE config 5 GEMM: [2048,7168] x [4096,7168]^T; 64 sampled rows vs fp32 torch
+    m, n, k = 2048, 4096, 7168
+    xq, wq, xs, ws = make_problem(m, n, k, seed=0)
+    out = run_gpu(xq, wq, xs, ws)
+    rows = torch.randperm(m, generator=torch.Generator().manual_seed(2))[:64]
+    ref = tr.gemm_a8w8_blockscale_ref(xq[rows], wq, xs[rows], ws)
+    assert tr.check_allclose_ratio(out.cpu()[rows], ref, RTOL, ATOL) == 0.0
