@@ -65,15 +65,17 @@ FP8BS_HD bool amax_allows_fast_path(uint32_t amax_bits)
 }
 
 // Correctly rounded x / s from the correctly rounded reciprocal r = RN(1 / s):
-//     q0 = RN(x * r);  e = RN(x - q0 * s) (exact, one FMA);  q = RN(q0 + e * r)
+//     q0 = RN(x * r);  t = q0 * s - x (exact, one FMA);  q = RN(q0 - t * r)
 // With r = RN(1/s) this sequence returns RN(x / s) for binary32 operands whenever no
 // intermediate under/overflows (Markstein's theorem); the CPU tests additionally compare it
 // with IEEE division for every 16-bit-float x against every reachable scale.
+// The residual is formed as q0*s - x and subtracted (rather than x - q0*s and added) so that
+// x = -0 yields -0, as IEEE division does: t = (-0)*s + (+0) = +0, q = (-0)*r + (-0) = -0.
 FP8BS_HD float div_by_scale(float x, float s, float r)
 {
     float q0 = x * r;
-    float e  = fma32(-q0, s, x);
-    return fma32(e, r, q0);
+    float t  = fma32(q0, s, -x);
+    return fma32(-t, r, q0);
 }
 
 // Software e4m3fn conversion (round to nearest even on the real value), used on the rare slow

@@ -33,7 +33,8 @@ __device__ __forceinline__ void unpack8(const u32x4& c, float* v)
         }
         else
         {
-            f16x2 h      = __builtin_bit_cast(f16x2, c[i]);
+            const uint32_t w = c[i]; // copy first: bit_cast straight from a vector element misreads
+            f16x2 h      = __builtin_bit_cast(f16x2, w);
             v[2 * i]     = (float)h.x;
             v[2 * i + 1] = (float)h.y;
         }

@@ -54,4 +54,12 @@ def assert_quant_bit_exact(y, s, x_cpu, group=128, in_dtype="bf16", what=""):
     sg = bits32(s).reshape(so.shape)
     bad_c = int((yg != yo).sum())
     bad_s = int((sg != so.view(np.uint32)).sum())
-    assert bad_c == 0 and bad_s == 0, f"{what}: {bad_c} code mismatches, {bad_s} scale mismatches"
+    detail = ""
+    if bad_c:
+        xc = codes16(x_cpu).reshape(yo.shape)
+        idx = np.argwhere(yg != yo)[:8]
+        detail = "; first mismatches (x code, got, want, scale bits): " + ", ".join(
+            f"{xc[tuple(i)]:#06x}:{yg[tuple(i)]:#04x}!={yo[tuple(i)]:#04x}@{so.view(np.uint32).reshape(-1)[np.ravel_multi_index(tuple(i), yo.shape) // group]:#010x}"
+            for i in idx
+        )
+    assert bad_c == 0 and bad_s == 0, f"{what}: {bad_c} code mismatches, {bad_s} scale mismatches{detail}"
