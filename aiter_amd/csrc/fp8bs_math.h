@@ -55,8 +55,12 @@ FP8BS_HD float fma32(float a, float b, float c)
 // float) lies in [kFastAmaxMin, kFastAmaxMax]: then scale = amax/448, its reciprocal, every
 // quotient (|q| <= 448.0001) and every residual below stay far from the subnormal and
 // overflow ranges, which is what the exactness argument needs.
-//   2^-100 <= amax <= 2^100
-constexpr uint32_t kFastAmaxMinBits = (127u - 100u) << 23;
+//   2^-80 <= amax <= 2^100
+// The lower bound also keeps the residual exact for every x whose quotient can reach the fp8
+// grid: |q| >= 2^-11 needs |x| >= amax * 2^-20 >= 2^-100, and the residual q0*s - x has its last
+// bit at 2^-47 |x| >= 2^-149.  Smaller x give |q| < 2^-11, which encodes as (signed) zero even if
+// the low bits of q are off.
+constexpr uint32_t kFastAmaxMinBits = (127u - 80u) << 23;
 constexpr uint32_t kFastAmaxMaxBits = (127u + 100u) << 23;
 
 FP8BS_HD bool amax_allows_fast_path(uint32_t amax_bits)
@@ -75,6 +79,11 @@ FP8BS_HD float div_by_scale(float x, float s, float r)
 {
     float q0 = x * r;
     float t  = fma32(q0, s, -x);
+#if !defined(__HIP_DEVICE_COMPILE__) && defined(__x86_64__)
+    // host builds only: keep the compiler from folding the negation of t into a fused
+    // negate-multiply-subtract, whose zero result has the other sign
+    __asm__ volatile("" : "+x"(t));
+#endif
     return fma32(-t, r, q0);
 }
 

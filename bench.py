@@ -1,0 +1,388 @@
+#!/usr/bin/env python3
+"""Benchmark of the FP8 block-scale path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload quant|prefill|decode|fused]
+                    [--no-also] [--no-cpu]
+
+A step is one pass of the hot path over one batch of synthetic input that is already resident
+in HBM.  The primary workload (default ``quant``) fills ``value``; the other workloads of the
+path are timed briefly as well and reported under ``also`` in the same JSON line.
+
+Workloads (BASELINE.json configs):
+  quant    config 2  x bf16 [16384,7168] (1 % channels x50) -> fp8 + fp32 scales, HBM-bound
+  prefill  config 4  blockscale GEMM M=8192 N=36864 K=7168, MFMA-bound
+  decode   config 3  blockscale GEMM M in {1,16,64} x {(7168,2048),(24576,1536),(2112,7168)}
+  fused    config 5  RMSNorm + 1x128 quant on [2048,7168], then GEMM N=4096
+
+Timing uses HIP events recorded on the stream the kernels are launched on (torch's current
+stream) around exactly K launches-worth of steps, bracketed by device synchronisation.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "blockscale GEMM TFLOP/s (% FP8 MFMA peak); group-quant GB/s (% HBM peak)"
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+FP8_PEAK_TFLOPS = 5000.0       # MI355X dense FP8 MFMA
+# The reference's own tuner measurement for the prefill shape on gfx950 / 256 CUs
+# (aiter/configs/model_configs/a8w8_blockscale_tuned_gemm_ds_v3.csv:6382), quoted in BASELINE.md.
+REF_PREFILL_TFLOPS = 2108.5
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="quant", choices=["quant", "prefill", "decode", "fused"])
+    ap.add_argument("--no-also", action="store_true", help="time only the primary workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    return ap.parse_args()
+
+
+def time_steps(torch, fn, steps, warmup):
+    """Average seconds per call of fn over exactly `steps` calls, HIP events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1e-3 / steps
+
+
+def gemm_bytes(m, n, k):
+    # algorithmic bytes: fp8 operands read once, 16-bit output written once, fp32 scales read once
+    return m * k + n * k + 2 * m * n + 4 * m * (k // 128) + 4 * ((n + 127) // 128) * (k // 128)
+
+
+# ---------------------------------------------------------------- workloads
+
+
+class QuantWorkload:
+    name = "quant"
+    M, K = 16384, 7168
+
+    def setup(self, torch, dev):
+        import aiter_amd
+        from aiter_amd import dtypes
+        from oracle import torch_ref as tr
+
+        self.aiter = aiter_amd
+        self.x_cpu = tr.make_activation(self.M, self.K, seed=0, outlier_frac=0.01)
+        # rotate over several inputs so that no pass finds its input in the 256 MB last-level cache
+        base = self.x_cpu.to(dev)
+        self.xs = [base, base.clone(), base.clone()]
+        self.y = torch.empty(self.M, self.K, dtype=dtypes.fp8, device=dev)
+        self.s = torch.empty(self.M, self.K // 128, dtype=torch.float32, device=dev)
+        self.i = 0
+
+    def step(self):
+        self.i = (self.i + 1) % len(self.xs)
+        self.aiter.dynamic_per_token_scaled_quant(self.y, self.xs[self.i].view(-1, 128), self.s)
+
+    def algorithmic_bytes(self):
+        return self.M * self.K * 2 + self.M * self.K + self.M * (self.K // 128) * 4
+
+    def describe(self):
+        return {
+            "workload": "config 2: standalone 1x128 dynamic FP8 group quant, x bf16 [16384,7168] "
+            "N(0,1) with 1% of channels x50 -> fp8 e4m3fn [16384,7168] + fp32 scales [16384,56]",
+            "M": self.M,
+            "K": self.K,
+            "group": 128,
+            "kernel": "group_quant_kernel",
+        }
+
+    def result(self, sec):
+        gbs = self.algorithmic_bytes() / sec / 1e9
+        roof = {
+            "bound": "hbm",
+            "achieved": gbs,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": gbs / HBM_PEAK_GBS,
+            "traffic": load_traffic("group_quant_kernel"),
+        }
+        return gbs, "GB/s", roof
+
+    def cpu_baseline(self, torch):
+        from oracle import torch_ref as tr
+
+        rows = 4096  # bounded sample: a quarter of the rows, same distribution
+        x = self.x_cpu[:rows]
+        tr.per_1x128_quant(x)
+        ts = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            tr.per_1x128_quant(x)
+            ts.append(time.perf_counter() - t0)
+        sec = sorted(ts)[len(ts) // 2]
+        by = rows * self.K * 3 + rows * (self.K // 128) * 4
+        return {
+            "value": by / sec / 1e9,
+            "unit": "GB/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"torch-CPU restatement of pertoken_quant on rows 0..{rows - 1} of the same "
+            f"input ([{rows},{self.K}] bf16), median of 5 runs, {sec * 1e3:.1f} ms each",
+        }
+
+
+class GemmWorkload:
+    def __init__(self, name, m, n, k, label):
+        self.name, self.M, self.N, self.K, self.label = name, m, n, k, label
+
+    def setup(self, torch, dev):
+        import aiter_amd
+        from aiter_amd import dtypes
+
+        self.aiter = aiter_amd
+        g = torch.Generator(device=dev).manual_seed(0)
+        m, n, k = self.M, self.N, self.K
+
+        # fp8 codes with the distribution the quantisers produce are irrelevant to speed; use
+        # random finite codes and positive scales (the parity tests cover real quantised data)
+        def codes(r, c):
+            t = torch.randint(0, 256, (r, c), generator=g, device=dev, dtype=torch.int32).to(torch.uint8)
+            t[(t & 0x7F) == 0x7F] = 0x38
+            return t.view(dtypes.fp8)
+
+        nbuf = 1 if (n * k) > (1 << 28) else 3  # rotate weights unless they already exceed the LLC
+        self.xq = codes(m, k)
+        self.wqs = [codes(n, k) for _ in range(nbuf)]
+        self.xs = torch.rand(m, k // 128, generator=g, device=dev) * 0.02 + 0.001
+        self.ws = torch.rand((n + 127) // 128, k // 128, generator=g, device=dev) * 0.002 + 0.0001
+        self.out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+        self.i = 0
+
+    def step(self):
+        self.i = (self.i + 1) % len(self.wqs)
+        self.aiter.gemm_a8w8_blockscale_ck(self.xq, self.wqs[self.i], self.xs, self.ws, self.out, splitK=-1)
+
+    def flops(self):
+        return 2.0 * self.M * self.N * self.K
+
+    def describe(self):
+        return {"workload": self.label, "M": self.M, "N": self.N, "K": self.K, "kernel": "gemm_a8w8_blockscale"}
+
+    def result(self, sec):
+        tf = self.flops() / sec / 1e12
+        gbs = gemm_bytes(self.M, self.N, self.K) / sec / 1e9
+        if self.M >= 1024:
+            roof = {"bound": "mfma", "achieved": tf, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": tf / FP8_PEAK_TFLOPS, "traffic": load_traffic("gemm_prefill")}
+            return tf, "TFLOP/s", roof
+        roof = {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": gbs / HBM_PEAK_GBS, "traffic": None}
+        return gbs, "GB/s", roof
+
+    def cpu_baseline(self, torch):
+        from oracle import torch_ref as tr
+
+        rows = min(self.M, 16)
+        ncols = min(self.N, 4096)
+        xq = self.xq[:rows].cpu()
+        wq = self.wqs[0][:ncols].cpu()
+        xs = self.xs[:rows].cpu()
+        ws = self.ws[: (ncols + 127) // 128].cpu()
+        tr.gemm_a8w8_blockscale_ref(xq, wq, xs, ws)
+        t0 = time.perf_counter()
+        tr.gemm_a8w8_blockscale_ref(xq, wq, xs, ws)
+        sec = time.perf_counter() - t0
+        return {
+            "value": 2.0 * rows * ncols * self.K / sec / 1e12,
+            "unit": "TFLOP/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"torch-CPU restatement (dequantise to fp32 + F.linear) on a [{rows},{self.K}] x "
+            f"[{ncols},{self.K}]^T slice, one timed run of {sec * 1e3:.0f} ms, dequantisation included",
+        }
+
+
+class FusedWorkload:
+    name = "fused"
+    M, K, N = 2048, 7168, 4096
+
+    def setup(self, torch, dev):
+        import aiter_amd
+        from aiter_amd import dtypes
+        from oracle import torch_ref as tr
+
+        self.aiter = aiter_amd
+        self.x_cpu = tr.make_activation(self.M, self.K, seed=0)
+        g = torch.Generator().manual_seed(1)
+        self.w_cpu = (torch.rand(self.K, generator=g) + 0.5).bfloat16()
+        self.x = self.x_cpu.to(dev)
+        self.nw = self.w_cpu.to(dev)
+        self.y = torch.empty(self.M, self.K, dtype=dtypes.fp8, device=dev)
+        self.s = torch.empty(self.M, self.K // 128, dtype=torch.float32, device=dev)
+        gd = torch.Generator(device=dev).manual_seed(2)
+        wq = torch.randint(0, 256, (self.N, self.K), generator=gd, device=dev, dtype=torch.int32).to(torch.uint8)
+        wq[(wq & 0x7F) == 0x7F] = 0x38
+        self.wq = wq.view(dtypes.fp8)
+        self.ws = torch.rand(self.N // 128, self.K // 128, generator=gd, device=dev) * 0.002 + 0.0001
+        self.out = torch.empty(self.M, self.N, dtype=torch.bfloat16, device=dev)
+
+    def step(self):
+        self.aiter.rmsnorm2d_fwd_with_dynamicquant(self.y, self.x, self.s, self.nw, 1e-6, 0, group_size=128)
+        self.aiter.gemm_a8w8_blockscale_ck(self.y, self.wq, self.s, self.ws, self.out, splitK=-1)
+
+    def step_norm_only(self):
+        self.aiter.rmsnorm2d_fwd_with_dynamicquant(self.y, self.x, self.s, self.nw, 1e-6, 0, group_size=128)
+
+    def describe(self):
+        return {
+            "workload": "config 5: fused RMSNorm + 1x128 FP8 quant on x bf16 [2048,7168], then blockscale "
+            "GEMM with N=4096, K=7168",
+            "M": self.M, "N": self.N, "K": self.K, "kernel": "rmsnorm_kernel + gemm_a8w8_blockscale",
+        }
+
+    def norm_bytes(self):
+        return self.M * self.K * 3 + self.K * 2 + self.M * (self.K // 128) * 4
+
+    def result(self, sec):
+        tf = 2.0 * self.M * self.N * self.K / sec / 1e12
+        roof = {"bound": "mfma", "achieved": tf, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": tf / FP8_PEAK_TFLOPS, "traffic": None}
+        return tf, "TFLOP/s", roof
+
+    def cpu_baseline(self, torch):
+        from oracle import torch_ref as tr
+
+        rows = 512
+        x = self.x_cpu[:rows]
+        tr.rmsnorm_quant_ref(x, self.w_cpu, 1e-6)
+        t0 = time.perf_counter()
+        tr.rmsnorm_quant_ref(x, self.w_cpu, 1e-6)
+        sec = time.perf_counter() - t0
+        by = rows * self.K * 3 + self.K * 2 + rows * (self.K // 128) * 4
+        return {"value": by / sec / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+                "sample": f"torch-CPU F.rms_norm + pertoken_quant on rows 0..{rows - 1} ({sec * 1e3:.1f} ms); "
+                "the GEMM half is covered by the prefill workload's baseline"}
+
+
+def load_traffic(kernel):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE + WRITE_SIZE, calibrated on
+    a plain copy kernel); the numbers live in profiles/traffic.json beside the rocprof summaries."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(kernel, {}).get("hbm_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
+
+
+DECODE_SHAPES = [(m, n, k) for (n, k) in [(7168, 2048), (24576, 1536), (2112, 7168)] for m in (1, 16, 64)]
+
+
+def make_workload(name):
+    if name == "quant":
+        return QuantWorkload()
+    if name == "prefill":
+        return GemmWorkload("prefill", 8192, 36864, 7168,
+                            "config 4: prefill blockscale GEMM M=8192 N=36864 K=7168 (fused gate+up FFN), "
+                            "fp8 e4m3fn operands, 1x128 / 128x128 fp32 scales, bf16 out")
+    if name == "decode":
+        return GemmWorkload("decode", 64, 24576, 1536,
+                            "config 3: decode blockscale GEMM M=64 N=24576 K=1536 (largest of the nine decode shapes)")
+    if name == "fused":
+        return FusedWorkload()
+    raise ValueError(name)
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU's throughput; --gpus {args.gpus} is not supported in this build "
+              "(nothing on this path uses a second GPU).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (no CPU fallback exists for the product path)", file=sys.stderr)
+        sys.exit(1)
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+
+    wl = make_workload(args.workload)
+    wl.setup(torch, dev)
+    sec = time_steps(torch, wl.step, args.steps, args.warmup)
+    value, unit, roof = wl.result(sec)
+
+    line = {
+        "metric": METRIC,
+        "value": value,
+        "unit": unit,
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": sec * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3fn (fp32 scales and accumulation)",
+        "data": "synthetic",
+        "config": wl.describe(),
+        "roofline": roof,
+    }
+    if args.workload == "prefill":
+        line["vs_reference_tuned_csv"] = value / REF_PREFILL_TFLOPS
+
+    if not args.no_cpu:
+        torch.set_num_threads(os.cpu_count() or 1)
+        line["cpu_baseline"] = wl.cpu_baseline(torch)
+
+    if not args.no_also:
+        also = {}
+        del wl
+        torch.cuda.empty_cache()
+        for name in ("quant", "prefill", "fused"):
+            if name == args.workload:
+                continue
+            w2 = make_workload(name)
+            w2.setup(torch, dev)
+            steps2 = 10 if name == "prefill" else 30
+            s2 = time_steps(torch, w2.step, steps2, 3)
+            v2, u2, r2 = w2.result(s2)
+            entry = {"value": v2, "unit": u2, "us_per_step": s2 * 1e6, "steps": steps2, "roofline": r2,
+                     "config": w2.describe()}
+            if name == "prefill":
+                entry["vs_reference_tuned_csv"] = v2 / REF_PREFILL_TFLOPS
+            if name == "fused":
+                sn = time_steps(torch, w2.step_norm_only, 30, 3)
+                gb = w2.norm_bytes() / sn / 1e9
+                entry["norm_quant"] = {"us": sn * 1e6, "GB/s": gb, "frac_of_hbm_peak": gb / HBM_PEAK_GBS}
+            also[name] = entry
+            del w2
+            torch.cuda.empty_cache()
+        dec = []
+        for (m, n, k) in DECODE_SHAPES:
+            w3 = GemmWorkload("decode", m, n, k, "decode")
+            w3.setup(torch, dev)
+            s3 = time_steps(torch, w3.step, 50, 5)
+            gbs = gemm_bytes(m, n, k) / s3 / 1e9
+            dec.append({"M": m, "N": n, "K": k, "us": s3 * 1e6, "GB/s": gbs, "frac_of_hbm_peak": gbs / HBM_PEAK_GBS})
+            del w3
+        also["decode"] = dec
+        line["also"] = also
+
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

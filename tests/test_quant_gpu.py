@@ -109,8 +109,9 @@ def test_special_groups_follow_torch():
         [1.0, nan, 2.0, -3.0] + [0.5] * 124,          # NaN group
         [2.0**-133, 2.0**-133, 2.0**-134, 0.0] + [0.0] * 124,  # scale becomes subnormal
         [2.0**-132, -(2.0**-133), 2.0**-133 * 3, 0.0] + [2.0**-133] * 124,  # bf16 subnormals
-        [2.0**-101, -(2.0**-101), 2.0**-104, 0.0] + [2.0**-110] * 124,      # just below the fast range
-        [2.0**-100, -(2.0**-100), 2.0**-104, 0.0] + [2.0**-110] * 124,      # first fast-path amax
+        [2.0**-81, -(2.0**-81), 2.0**-84, 0.0] + [2.0**-90] * 124,          # just below the fast range
+        [2.0**-80, -(2.0**-80), 2.0**-84, 0.0] + [2.0**-99] * 124,          # first fast-path amax
+        [2.0**-80, -(2.0**-133), 2.0**-120, 2.0**-100] + [2.0**-98] * 124,  # tiny x beside it
         [2.0**100, -(2.0**100), 2.0**94, 0.0] + [2.0**90] * 124,            # last fast-path amax
         [2.0**101, -(2.0**101), 2.0**94, 0.0] + [2.0**92] * 124,            # just above
         [3.0e38, -3.0e38, 1.0e30, 1.0] + [0.0] * 124, # huge amax
