@@ -117,8 +117,10 @@ __device__ __forceinline__ uint32_t group_max_u32(uint32_t v)
 // the software conversion.  NaN/inf follow what the host division does in the torch reference:
 // a NaN element keeps its own sign, other elements of a NaN group get the (positive) NaN of
 // the scale; inf/inf is the default NaN, which has the sign bit set on x86.
+// Inlined on purpose: an out-of-line call would give the kernel a private (scratch) segment,
+// and waves that need scratch are dispatched far more slowly than the HBM stream can be fed.
 template <int LPG>
-__device__ __noinline__ void quant16_slow(const float (&v)[16], u32x4& codes, float& scale)
+__device__ __forceinline__ void quant16_slow(const float (&v)[16], u32x4& codes, float& scale)
 {
     uint32_t mm = 0;
 #pragma unroll
@@ -270,7 +272,7 @@ __global__ __launch_bounds__(kQuantBlock) void group_quant_kernel(QuantKernelPar
 template <In16 DT, int GS>
 static hipError_t launch_group_quant_t(const QuantArgs& a, hipStream_t stream)
 {
-    constexpr int UNITS = 2;
+    constexpr int UNITS = 1;
     constexpr int LPG   = GS / 16;
     constexpr int GPB   = kQuantBlock / LPG * UNITS;
     QuantKernelParams p;
