@@ -17,7 +17,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_NAME = "libaiter_fp8bs.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 
-SOURCES = ["abi.hip", "norm_quant_kernels.hip", "gemm_blockscale_kernels.hip"]
+SOURCES = ["abi.hip", "norm_quant_kernels.hip", "gemm_blockscale_kernels.hip", "gemm_prefill.hip", "gemm_decode.hip"]
 
 # -ffp-contract=off: the quantiser's rounding sequence must stay one IEEE operation per step.
 # The packed-fp32 target feature is switched off for device code on purpose; the host pass

@@ -12,59 +12,11 @@
 // a lane then owns 4 consecutive n for one m, which makes (a) the scale of its 4 accumulators
 // one scalar per lane, xs[m,kb]*ws[nb,kb], and (b) its output 4 consecutive 16-bit values.
 #include "fp8bs_launch.h"
+#include "gemm_common.h"
 
 #include <string.h>
 
 namespace fp8bs {
-
-typedef int      i32x8 __attribute__((ext_vector_type(8)));
-typedef int      i32x4 __attribute__((ext_vector_type(4)));
-typedef float    f32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-
-__device__ __forceinline__ f32x4 mfma_16x16x128_fp8(const i32x8& a, const i32x8& b, const f32x4& c)
-{
-    // cbsz = blgp = 0 selects e4m3 for both operands; zero scale operands select the
-    // unscaled instruction
-    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
-}
-
-template <In16 DT>
-__device__ __forceinline__ uint32_t pack2(float lo, float hi)
-{
-    if constexpr(DT == In16::bf16)
-    {
-        __bf16 a = (__bf16)lo, b = (__bf16)hi;
-        return (uint32_t)__builtin_bit_cast(unsigned short, a) |
-               ((uint32_t)__builtin_bit_cast(unsigned short, b) << 16);
-    }
-    else
-    {
-        _Float16 a = (_Float16)lo, b = (_Float16)hi;
-        return (uint32_t)__builtin_bit_cast(unsigned short, a) |
-               ((uint32_t)__builtin_bit_cast(unsigned short, b) << 16);
-    }
-}
-
-struct GemmKernelParams
-{
-    const uint8_t* xq;
-    const uint8_t* wq;
-    const float*   xs;
-    const float*   ws;
-    uint16_t*      out;
-    int32_t        M, N, K;
-    int64_t        lda, ldb;
-    int32_t        kblocks; // K / 128
-};
-
-// LDS tile: rows of 128 bytes (one K block); the 16-byte chunk c of row r lives at chunk
-// c ^ (r & 7) so that the 16 rows a quarter-wave reads with one ds_read_b128 spread over banks.
-__device__ __forceinline__ uint32_t lds_off(uint32_t row, uint32_t chunk)
-{
-    return row * 128u + ((chunk ^ (row & 7u)) << 4);
-}
 
 // ---------------------------------------------------------------- generic tile kernel
 // BM x BN output tile per block (m = activation rows, n = weight rows), WAVES_M x WAVES_N
@@ -207,7 +159,7 @@ static hipError_t launch_tile(const GemmKernelParams& p, hipStream_t stream)
     return hipGetLastError();
 }
 
-static const char* const kKernelNames = "tile_16x256,tile_64x128,tile_128x128";
+static const char* const kKernelNames = "tile_16x256,tile_64x128,tile_128x128,prefill_256x256,decode_stream";
 
 const char* gemm_kernel_names() { return kKernelNames; }
 
@@ -218,12 +170,12 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
     const char* name = (a.kernel_name && a.kernel_name[0]) ? a.kernel_name : nullptr;
     if(name == nullptr)
     {
-        if(a.M <= 16)
-            name = "tile_16x256";
-        else if(a.M <= 64)
-            name = "tile_64x128";
-        else
+        if(gemm_decode_supports(p))
+            name = "decode_stream";
+        else if(a.M < 256 || !gemm_prefill_supports(p))
             name = "tile_128x128";
+        else
+            name = "prefill_256x256";
     }
     if(strcmp(name, "tile_16x256") == 0)
         return launch_tile<DT, 16, 256, 1, 4>(p, stream);
@@ -231,6 +183,29 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
         return launch_tile<DT, 64, 128, 2, 2>(p, stream);
     if(strcmp(name, "tile_128x128") == 0)
         return launch_tile<DT, 128, 128, 2, 2>(p, stream);
+    if(strcmp(name, "decode_stream") == 0)
+    {
+        if(!gemm_decode_supports(p))
+        {
+            *why = "decode_stream handles 1 <= M <= 64";
+            return hipErrorInvalidValue;
+        }
+        return launch_gemm_decode(p, DT, a.split_k_log2, a.device_id, stream);
+    }
+    if(a.split_k_log2 > 0)
+    {
+        *why = "splitK > 0 is only available with the decode_stream kernel (M <= 64)";
+        return hipErrorInvalidValue;
+    }
+    if(strcmp(name, "prefill_256x256") == 0)
+    {
+        if(!gemm_prefill_supports(p))
+        {
+            *why = "prefill_256x256 needs N % 4 == 0 and operand matrices below 4 GiB";
+            return hipErrorInvalidValue;
+        }
+        return launch_gemm_prefill(p, DT, stream);
+    }
     *why = "unknown kernelName (see aiter_fp8bs_gemm_kernel_names())";
     return hipErrorInvalidValue;
 }
@@ -252,11 +227,6 @@ hipError_t launch_gemm_blockscale(const GemmArgs& a, hipStream_t stream, const c
     p.lda     = a.lda;
     p.ldb     = a.ldb;
     p.kblocks = (int32_t)(a.K / 128);
-    if(a.split_k_log2 > 0)
-    {
-        *why = "splitK > 0 is not available for this kernel";
-        return hipErrorInvalidValue;
-    }
     return a.out_dtype == In16::bf16 ? dispatch<In16::bf16>(a, p, stream, why)
                                      : dispatch<In16::fp16>(a, p, stream, why);
 }

@@ -1,0 +1,304 @@
+// Prefill-shape block-scale FP8 GEMM (large M): MFMA-bound.
+//
+// 256 (m) x 256 (n) output tile per workgroup, one 128-wide K block per step, 8 waves laid out
+// 2 (n) x 4 (m) so that each wave owns 128 n x 64 m = 8 x 4 MFMA tiles (128 fp32 accumulators
+// per lane).  Both operand slabs are brought in with direct global->LDS loads
+// (global_load_lds_dwordx4: no VGPR staging, no ds_write) into a two-stage ring, so the loads of
+// K block kb+1 fly while block kb is multiplied.  Per K block every 16x16 tile costs one
+// v_mfma_f32_16x16x128_f8f6f4 (32 cycles) plus 4 fp32 FMAs that fold the unscaled product into
+// the accumulators with the scale xs[m,kb]*ws[n/128,kb].
+//
+// Workgroups are renumbered so that the 32 tiles resident on one XCD at a time form a compact
+// 8 (m) x 4 (n) patch: each XCD's L2 then serves every operand slab to several CUs.
+#include "gemm_common.h"
+
+namespace fp8bs {
+
+namespace {
+
+constexpr int kBM = 256, kBN = 256, kThreads = 512;
+constexpr int kStageBytes = (kBM + kBN) * 128; // 64 KiB: 256 weight rows then 256 activation rows
+constexpr int kStages = 2;
+constexpr int kGroupN = 4; // n tiles swept together by consecutive workgroups
+
+// 16-byte chunk c of stage row r is stored at chunk c ^ ((r >> 1) & 7): the 16 rows one
+// quarter-wave reads with a ds_read_b128 then fall on 16 different 16-byte bank groups.
+__device__ __forceinline__ uint32_t swz(uint32_t row, uint32_t chunk)
+{
+    return row * 128u + ((chunk ^ ((row >> 1) & 7u)) << 4);
+}
+
+__device__ __forceinline__ i32x8 read_frag(const uint8_t* base, uint32_t row, uint32_t kg)
+{
+    i32x4 lo = *(const i32x4*)(base + swz(row, 2 * kg));
+    i32x4 hi = *(const i32x4*)(base + swz(row, 2 * kg + 1));
+    return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+}
+
+template <In16 DT>
+__global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams p, int tiles_m,
+                                                                int tiles_n)
+{
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int l16 = lane & 15, kg = lane >> 4;
+    const int wn = wave & 1, wm = wave >> 1; // n half (128 rows), m quarter (64 rows)
+
+    // ---- tile choice: XCD-aware renumbering, then n-groups swept m-fastest
+    const int total = tiles_m * tiles_n;
+    int       v     = blockIdx.x;
+    if((total & 7) == 0)
+        v = (v & 7) * (total >> 3) + (v >> 3); // workgroups go round-robin over the 8 XCDs
+    const int group  = v / (kGroupN * tiles_m);
+    const int within = v - group * (kGroupN * tiles_m);
+    const int gn     = min(kGroupN, tiles_n - group * kGroupN);
+    const int tm     = within / gn;
+    const int tn     = group * kGroupN + (within - tm * gn);
+    const int m0 = tm * kBM, n0 = tn * kBN;
+
+    typedef const volatile i32x4 __attribute__((address_space(3)))* lds_vec_ptr;
+    typedef uint8_t __attribute__((address_space(3)))*              lds_byte_ptr;
+    const lds_byte_ptr smem3 = (lds_byte_ptr)smem;
+
+    // ---- global -> LDS plan: per stage 64 units of 8 rows (1 KiB); wave w moves units i*8+w.
+    // Lane p of a unit fills LDS chunk p, i.e. stage row 8u + p/8, stored chunk p%8, which must
+    // hold the row's logical chunk (p%8) ^ ((row>>1)&7).
+    uint32_t goff[8];
+#pragma unroll
+    for(int i = 0; i < 8; ++i)
+    {
+        const uint32_t r = 64u * i + 8u * wave + (lane >> 3);
+        const uint32_t c = (lane & 7u) ^ ((r >> 1) & 7u);
+        if(i < 4)
+        {
+            uint32_t n = n0 + r;
+            n          = n < (uint32_t)p.N ? n : (uint32_t)p.N - 1;
+            goff[i]    = n * (uint32_t)p.ldb + c * 16u;
+        }
+        else
+        {
+            uint32_t m = m0 + (r - 256u);
+            m          = m < (uint32_t)p.M ? m : (uint32_t)p.M - 1;
+            goff[i]    = m * (uint32_t)p.lda + c * 16u;
+        }
+    }
+    // One LDS-direct load (global_load_lds_dwordx4): lane p's 16 bytes land at M0 + 16 p.
+    // Written as asm on purpose: the compiler models the builtin as a flat access that may touch
+    // LDS and from then on waits for every outstanding LDS read in full.  The loads are not
+    // visible to the compiler's wait-count bookkeeping, so every consumer sits behind an
+    // explicit s_waitcnt vmcnt(0) and a workgroup barrier.
+    auto dma16 = [](uint32_t lds_dst, uint32_t voff, const uint8_t* sbase) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(lds_dst), "v"(voff), "s"(sbase)
+                     : "memory");
+    };
+
+    // ---- scales: one x_scale row per m tile of this lane, one w_scale block per wave
+    uint32_t xs_off[4];
+#pragma unroll
+    for(int j = 0; j < 4; ++j)
+    {
+        uint32_t m = m0 + wm * 64 + j * 16 + l16;
+        m          = m < (uint32_t)p.M ? m : (uint32_t)p.M - 1;
+        xs_off[j]  = m * (uint32_t)p.kblocks;
+    }
+    uint32_t nb = (uint32_t)(n0 + wn * 128) >> 7;
+    nb          = min(nb, (uint32_t)((p.N + 127) / 128 - 1));
+    const float* ws_row = p.ws + (size_t)nb * p.kblocks;
+
+    // ---- LDS read addresses.  A fragment is 32 bytes of one row: logical chunks 2kg and 2kg+1.
+    // Tile rows start at multiples of 16, so the swizzle term depends on l16 only and every
+    // tile is reached with an immediate offset from these four per-lane bases.
+    const uint32_t sw     = (uint32_t)(l16 >> 1) & 7u;
+    const uint32_t lo_off = (uint32_t)l16 * 128u + (((2u * kg) ^ sw) << 4);
+    const uint32_t hi_off = (uint32_t)l16 * 128u + (((2u * kg + 1u) ^ sw) << 4);
+    const uint32_t w_base = (uint32_t)wn * (128u * 128u);
+    const uint32_t x_base = (uint32_t)kBN * 128u + (uint32_t)wm * (64u * 128u);
+
+    float acc[8][4][4];
+#pragma unroll
+    for(int i = 0; i < 8; ++i)
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+#pragma unroll
+            for(int r = 0; r < 4; ++r)
+                acc[i][j][r] = 0.f;
+
+    // The K loop is written as an explicit instruction stream.  Every 16x16 tile costs one MFMA
+    // (32 cycles in the matrix pipe) and 4 FMAs that fold its unscaled product into the
+    // accumulators.  To keep the matrix pipe fed from a single wave, the FMAs of tile t-2 are
+    // issued behind the MFMA of tile t: by then the older product has been written back, so no
+    // wait states are needed, and the in-order issue never parks on a result that is still in
+    // flight.  Products rotate through four register quads; the last two tiles of a K block are
+    // folded in after the first two MFMAs of the next one.  `asm volatile` keeps this order; the
+    // LDS reads are volatile loads so they stay where they are written (ahead of their use) while
+    // the compiler still derives their wait counts.
+#define FP8BS_MFMA(P, A, B) \
+    asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=&v"(P) : "v"(A), "v"(B))
+#define FP8BS_FMA4(ACC, P, S)                                                              \
+    do                                                                                     \
+    {                                                                                      \
+        asm volatile("v_fmac_f32 %0, %1, %2" : "+v"((ACC)[0]) : "v"((P)[0]), "v"(S));      \
+        asm volatile("v_fmac_f32 %0, %1, %2" : "+v"((ACC)[1]) : "v"((P)[1]), "v"(S));      \
+        asm volatile("v_fmac_f32 %0, %1, %2" : "+v"((ACC)[2]) : "v"((P)[2]), "v"(S));      \
+        asm volatile("v_fmac_f32 %0, %1, %2" : "+v"((ACC)[3]) : "v"((P)[3]), "v"(S));      \
+    } while(0)
+
+    auto read_frag_v = [&](uint32_t stage_off, uint32_t tile_off) -> i32x8 {
+        const i32x4 lo = *(lds_vec_ptr)(smem3 + stage_off + lo_off + tile_off);
+        const i32x4 hi = *(lds_vec_ptr)(smem3 + stage_off + hi_off + tile_off);
+        return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+
+    // w_scale of this wave's n block for 64 consecutive K blocks lives in one VGPR (lane = K
+    // block) and is picked with v_readlane: a scalar load inside the loop would share the LGKM
+    // counter with the LDS reads and force them to be waited for in full.
+    auto load_ws_window = [&](int kb0) -> float {
+        const int k = kb0 + lane;
+        return ws_row[k < p.kblocks ? k : p.kblocks - 1];
+    };
+    float ws_vec = load_ws_window(0);
+    auto  ws_at  = [&](int kb) -> float {
+        return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(ws_vec), kb & 63));
+    };
+
+    float sx[4], wsc;
+    {
+        const uint32_t dst0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(smem3 + wave * 1024));
+#pragma unroll
+        for(int i = 0; i < 8; ++i)
+            dma16(dst0 + i * 8192, goff[i], i < 4 ? p.wq : p.xq);
+    }
+#pragma unroll
+    for(int j = 0; j < 4; ++j)
+        sx[j] = p.xs[xs_off[j]];
+    wsc = ws_at(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's LDS-direct loads have landed
+    __syncthreads();
+
+    f32x4 P[4];
+#pragma unroll
+    for(int q = 0; q < 4; ++q)
+        P[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float psc2 = 0.f, psc3 = 0.f; // scales of the two tiles still waiting to be folded in
+
+    for(int kb = 0; kb < p.kblocks; ++kb)
+    {
+        const int      cur      = kb & 1;
+        const uint32_t stage    = (uint32_t)cur * kStageBytes;
+        const int      kn       = kb + 1 < p.kblocks ? kb + 1 : kb; // last pass re-fetches, unused
+        const uint32_t dma_dst  = __builtin_amdgcn_readfirstlane(
+            (uint32_t)(uintptr_t)(smem3 + (cur ^ 1) * kStageBytes + wave * 1024));
+        const size_t   dma_koff = (size_t)kn * 128;
+
+        float nsx[4], nws;
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+            nsx[j] = p.xs[xs_off[j] + kn];
+        if((kn & 63) == 0 && kn != kb)
+            ws_vec = load_ws_window(kn);
+        nws = ws_at(kn);
+
+        float sc[4];
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+            sc[j] = sx[j] * wsc;
+
+        i32x8 bx[4], aw[2];
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+            bx[j] = read_frag_v(stage, x_base + j * 2048);
+        aw[0] = read_frag_v(stage, w_base);
+
+#pragma unroll
+        for(int t = 0; t < 32; ++t)
+        {
+            const int i = t >> 2, j = t & 3;
+            if(j == 0 && i < 7)
+                aw[(i + 1) & 1] = read_frag_v(stage, w_base + (i + 1) * 2048);
+            FP8BS_MFMA(P[t & 3], aw[i & 1], bx[j]);
+            if(j == 1)
+            {
+                dma16(dma_dst + i * 8192, goff[i], (i < 4 ? p.wq : p.xq) + dma_koff);
+            }
+            if(t == 0)
+                FP8BS_FMA4(acc[7][2], P[2], psc2);
+            else if(t == 1)
+                FP8BS_FMA4(acc[7][3], P[3], psc3);
+            else
+                FP8BS_FMA4(acc[(t - 2) >> 2][(t - 2) & 3], P[(t - 2) & 3], sc[(t - 2) & 3]);
+        }
+        psc2 = sc[2];
+        psc3 = sc[3];
+
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+            sx[j] = nsx[j];
+        wsc = nws;
+    }
+    // drain: the last two products (the barrier above is far more than the 11 wait states an
+    // 8-pass MFMA result needs, the explicit nops make that independent of it)
+    asm volatile("s_nop 15\n s_nop 15\n s_nop 15" ::: "memory");
+    FP8BS_FMA4(acc[7][2], P[2], psc2);
+    FP8BS_FMA4(acc[7][3], P[3], psc3);
+#undef FP8BS_MFMA
+#undef FP8BS_FMA4
+
+    // ---- epilogue: lane owns out[m][n .. n+3] for each of its 8 x 4 tiles
+#pragma unroll
+    for(int j = 0; j < 4; ++j)
+    {
+        const int m = m0 + wm * 64 + j * 16 + l16;
+        if(m >= p.M)
+            continue;
+#pragma unroll
+        for(int i = 0; i < 8; ++i)
+        {
+            const int n   = n0 + wn * 128 + i * 16 + kg * 4;
+            uint16_t* dst = p.out + (size_t)m * p.N + n;
+            if(n + 3 < p.N)
+            {
+                *(u32x2*)dst = u32x2{pack2<DT>(acc[i][j][0], acc[i][j][1]),
+                                     pack2<DT>(acc[i][j][2], acc[i][j][3])};
+            }
+            else
+            {
+#pragma unroll
+                for(int r = 0; r < 4; ++r)
+                    if(n + r < p.N)
+                        dst[r] = (uint16_t)(pack2<DT>(acc[i][j][r], 0.f) & 0xffffu);
+            }
+        }
+    }
+}
+
+} // namespace
+
+bool gemm_prefill_supports(const GemmKernelParams& p)
+{
+    // 32-bit byte offsets inside the operand matrices, 8-byte aligned output rows
+    return p.kblocks >= 1 && (uint64_t)p.N * (uint64_t)p.ldb < (1ull << 32) &&
+           (uint64_t)p.M * (uint64_t)p.lda < (1ull << 32) &&
+           (uint64_t)p.M * (uint64_t)p.kblocks < (1ull << 32) && (p.N % 4) == 0;
+}
+
+hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, hipStream_t stream)
+{
+    const int    tiles_m = (p.M + kBM - 1) / kBM, tiles_n = (p.N + kBN - 1) / kBN;
+    const size_t smem    = (size_t)kStages * kStageBytes;
+    auto         kernel  = out_dtype == In16::bf16 ? gemm_prefill_kernel<In16::bf16>
+                                                   : gemm_prefill_kernel<In16::fp16>;
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)smem);
+    if(e != hipSuccess)
+        return e;
+    hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(kThreads), smem, stream, p, tiles_m,
+                       tiles_n);
+    return hipGetLastError();
+}
+
+} // namespace fp8bs

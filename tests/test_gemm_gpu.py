@@ -62,15 +62,32 @@ def test_config1_plumbing():
     assert np.all(np.abs(out.cpu().float().numpy() - o64) <= 2.0**-8 * np.abs(o64) + 1e-4)
 
 
-@pytest.mark.parametrize("kernel", [None, "tile_16x256", "tile_64x128", "tile_128x128"])
+@pytest.mark.parametrize("kernel", [None, "tile_16x256", "tile_64x128", "tile_128x128", "prefill_256x256", "decode_stream"])
 @pytest.mark.parametrize(
     "m,n,k",
     [(1, 128, 128), (1, 2112, 512), (16, 256, 1024), (17, 384, 256), (64, 2112, 1024), (130, 520, 384), (257, 1000, 256)],
 )
 def test_shapes_and_tiles(kernel, m, n, k):
+    if kernel == "decode_stream" and m > 64:
+        with pytest.raises(RuntimeError, match="decode_stream handles"):
+            run_gpu(*make_problem(m, n, k), kernel=kernel)
+        return
     xq, wq, xs, ws = make_problem(m, n, k, seed=m + n + k)
     out = run_gpu(xq, wq, xs, ws, kernel=kernel)
     assert_close_to_f64(out, xq, wq, xs, ws, f"{kernel} {m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (512, 768, 1024), (300, 1000, 384), (1024, 2112, 512), (257, 260, 256)])
+def test_prefill_kernel_shapes(m, n, k):
+    xq, wq, xs, ws = make_problem(m, n, k, seed=m + n + k, outliers=0.01)
+    out = run_gpu(xq, wq, xs, ws, kernel="prefill_256x256")
+    assert_close_to_f64(out, xq, wq, xs, ws, f"prefill {m}x{n}x{k}")
+    # the library's own choice for these sizes gives the same bits as the named kernel or the
+    # generic tile kernel (same per-block products, same accumulation order over K blocks)
+    auto = run_gpu(xq, wq, xs, ws)
+    tile = run_gpu(xq, wq, xs, ws, kernel="tile_128x128")
+    assert torch.equal(out.view(torch.int16), tile.view(torch.int16))
+    assert torch.equal(auto.view(torch.int16), tile.view(torch.int16))
 
 
 def test_one_hot_isolates_single_scale_product():
@@ -143,6 +160,31 @@ def test_strided_operands_and_guard_bands():
     torch.cuda.synchronize()
     chk()
     assert_close_to_f64(out, xq, wq, xs, ws, "strided")
+
+
+@pytest.mark.parametrize("m,n,k,splitk", [(1, 64, 128, 0), (5, 200, 512, 0), (5, 200, 512, 2), (16, 2112, 1024, 3),
+                                            (17, 384, 4096, -1), (33, 130, 2304, 1), (48, 1000, 7168, -1),
+                                            (64, 256, 6144, 4), (64, 8192, 256, -1)])
+def test_decode_stream_kernel(m, n, k, splitk):
+    xq, wq, xs, ws = make_problem(m, n, k, seed=m + n + k + 1, outliers=0.01)
+    out = run_gpu(xq, wq, xs, ws, kernel="decode_stream", splitK=splitk)
+    assert_close_to_f64(out, xq, wq, xs, ws, f"decode_stream {m}x{n}x{k} splitK={splitk}")
+    # K splitting only regroups the fp32 additions: still within a few fp32 ulps of one chunk,
+    # and bit-identical from run to run (partials are added in a fixed order)
+    again = run_gpu(xq, wq, xs, ws, kernel="decode_stream", splitK=splitk)
+    assert torch.equal(out.view(torch.int16), again.view(torch.int16))
+    one = run_gpu(xq, wq, xs, ws, kernel="tile_16x256")
+    assert (out.view(torch.int16) != one.view(torch.int16)).float().mean().item() < 0.02
+
+
+def test_decode_split_k_repeated_calls_leave_tickets_clean():
+    # the split-K tickets must return to zero after every call, also when shapes change
+    for (m, n, k) in [(16, 2112, 7168), (1, 2112, 7168), (64, 2112, 7168), (16, 7168, 2048), (16, 2112, 7168)]:
+        xq, wq, xs, ws = make_problem(m, n, k, seed=n + k)
+        a = run_gpu(xq, wq, xs, ws)
+        b = run_gpu(xq, wq, xs, ws)
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+        assert_close_to_f64(a, xq, wq, xs, ws, f"repeat {m}x{n}x{k}")
 
 
 @pytest.mark.parametrize("m", [1, 16, 64])
