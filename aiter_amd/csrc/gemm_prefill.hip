@@ -17,7 +17,8 @@ namespace fp8bs {
 namespace {
 
 constexpr int kBM = 256, kBN = 256, kThreads = 512;
-constexpr int kStageBytes = (kBM + kBN) * 128; // 64 KiB: 256 weight rows then 256 activation rows
+constexpr int kSlabBytes  = (kBM + kBN) * 128; // 64 KiB: 256 weight rows then 256 activation rows
+constexpr int kStageBytes = kSlabBytes + kBM * 4; // + this K block's x_scale for the 256 rows
 constexpr int kStages = 2;
 constexpr int kGroupN = 4; // n tiles swept together by consecutive workgroups
 
@@ -95,15 +96,22 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
                      : "memory");
     };
 
-    // ---- scales: one x_scale row per m tile of this lane, one w_scale block per wave
-    uint32_t xs_off[4];
-#pragma unroll
-    for(int j = 0; j < 4; ++j)
+    // x_scale of K block kb for the tile's 256 rows: one 4-byte LDS-direct load per 64 rows
+    // (waves 0..3), lane l -> row 64 w + l, landing behind the operand slabs of the stage.
+    auto dma4 = [](uint32_t lds_dst, uint32_t voff, const void* sbase) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                     :
+                     : "s"(lds_dst), "v"(voff), "s"(sbase)
+                     : "memory");
+    };
+    uint32_t xs_goff; // byte offset of this lane's x_scale row (waves 0..3 only)
     {
-        uint32_t m = m0 + wm * 64 + j * 16 + l16;
+        uint32_t m = m0 + 64u * (wave & 3) + lane;
         m          = m < (uint32_t)p.M ? m : (uint32_t)p.M - 1;
-        xs_off[j]  = m * (uint32_t)p.kblocks;
+        xs_goff    = m * (uint32_t)p.kblocks * 4u;
     }
+
+    // ---- scales: x_scale comes through LDS with each stage, w_scale: one block per wave
     uint32_t nb = (uint32_t)(n0 + wn * 128) >> 7;
     nb          = min(nb, (uint32_t)((p.N + 127) / 128 - 1));
     const float* ws_row = p.ws + (size_t)nb * p.kblocks;
@@ -164,19 +172,21 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(ws_vec), kb & 63));
     };
 
-    float sx[4], wsc;
+    float wsc;
     {
         const uint32_t dst0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(smem3 + wave * 1024));
 #pragma unroll
         for(int i = 0; i < 8; ++i)
             dma16(dst0 + i * 8192, goff[i], i < 4 ? p.wq : p.xq);
+        if(wave < 4)
+            dma4(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(smem3 + kSlabBytes + wave * 256)),
+                 xs_goff, p.xs);
     }
-#pragma unroll
-    for(int j = 0; j < 4; ++j)
-        sx[j] = p.xs[xs_off[j]];
     wsc = ws_at(0);
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's LDS-direct loads have landed
     __syncthreads();
+    // LDS address of this lane's x_scale for m tile 0 (tile j sits 64 bytes further)
+    const uint32_t xs_lds = (uint32_t)kSlabBytes + ((uint32_t)wm * 64u + (uint32_t)l16) * 4u;
 
     f32x4 P[4];
 #pragma unroll
@@ -193,24 +203,25 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
             (uint32_t)(uintptr_t)(smem3 + (cur ^ 1) * kStageBytes + wave * 1024));
         const size_t   dma_koff = (size_t)kn * 128;
 
-        float nsx[4], nws;
-#pragma unroll
-        for(int j = 0; j < 4; ++j)
-            nsx[j] = p.xs[xs_off[j] + kn];
         if((kn & 63) == 0 && kn != kb)
             ws_vec = load_ws_window(kn);
-        nws = ws_at(kn);
+        const float nws = ws_at(kn);
 
-        float sc[4];
-#pragma unroll
-        for(int j = 0; j < 4; ++j)
-            sc[j] = sx[j] * wsc;
-
+        // fragment reads in the order the first MFMAs need them: all 8 waves read at once
+        // right after the barrier, so the fewer bytes stand between a wave and its first MFMA
+        // the sooner the matrix pipe restarts
         i32x8 bx[4], aw[2];
+        aw[0] = read_frag_v(stage, w_base);
 #pragma unroll
         for(int j = 0; j < 4; ++j)
             bx[j] = read_frag_v(stage, x_base + j * 2048);
-        aw[0] = read_frag_v(stage, w_base);
+        float sc[4];
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+        {
+            typedef const volatile float __attribute__((address_space(3)))* lds_f32_ptr;
+            sc[j] = *(lds_f32_ptr)(smem3 + stage + xs_lds + j * 64) * wsc;
+        }
 
 #pragma unroll
         for(int t = 0; t < 32; ++t)
@@ -219,10 +230,14 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
             if(j == 0 && i < 7)
                 aw[(i + 1) & 1] = read_frag_v(stage, w_base + (i + 1) * 2048);
             FP8BS_MFMA(P[t & 3], aw[i & 1], bx[j]);
-            if(j == 1)
+            if((t & 1) == 1 && t < 16) // the 8 LDS-direct loads ride behind the first 16 MFMAs
             {
+                const int i = t >> 1;
                 dma16(dma_dst + i * 8192, goff[i], (i < 4 ? p.wq : p.xq) + dma_koff);
             }
+            if(t == 16 && wave < 4)
+                dma4(__builtin_amdgcn_readfirstlane(dma_dst - wave * 1024 + kSlabBytes + wave * 256),
+                     xs_goff + (uint32_t)kn * 4u, p.xs);
             if(t == 0)
                 FP8BS_FMA4(acc[7][2], P[2], psc2);
             else if(t == 1)
@@ -233,11 +248,9 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         psc2 = sc[2];
         psc3 = sc[3];
 
+        // vmcnt(0): this wave's share of the next stage is in LDS
         __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
-#pragma unroll
-        for(int j = 0; j < 4; ++j)
-            sx[j] = nsx[j];
         wsc = nws;
     }
     // drain: the last two products (the barrier above is far more than the 11 wait states an
