@@ -172,7 +172,6 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(ws_vec), kb & 63));
     };
 
-    float wsc;
     {
         const uint32_t dst0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(smem3 + wave * 1024));
 #pragma unroll
@@ -182,17 +181,38 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
             dma4(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(smem3 + kSlabBytes + wave * 256)),
                  xs_goff, p.xs);
     }
-    wsc = ws_at(0);
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's LDS-direct loads have landed
     __syncthreads();
     // LDS address of this lane's x_scale for m tile 0 (tile j sits 64 bytes further)
     const uint32_t xs_lds = (uint32_t)kSlabBytes + ((uint32_t)wm * 64u + (uint32_t)l16) * 4u;
 
+    // ---- the K loop, skewed by a quarter of a K block.
+    // Issue order of one iteration (32 MFMA slots):
+    //   slots 0..7   the last 8 tiles (weight fragments 6 and 7) of the PREVIOUS K block, whose
+    //                operands are already in registers.  They keep the matrix pipe busy while
+    //                the first fragments of this K block travel from LDS, which would otherwise
+    //                be dead time right after the barrier (every wave reads at once).
+    //   slots 8..31  tiles of weight fragments 0..5 of this K block.
+    // The FMAs that fold a product into the accumulators trail their MFMA by two slots (the
+    // product is written back by then: no wait states), also across the iteration boundary.
+    // Registers: weight fragments rotate through 4 buffers (fragment i lives in buffer i & 3,
+    // so 6 and 7 of one K block and 0 and 1 of the next never collide); an activation fragment
+    // is replaced by the next K block's as soon as its two deferred tiles have been issued.
     f32x4 P[4];
 #pragma unroll
     for(int q = 0; q < 4; ++q)
         P[q] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float psc2 = 0.f, psc3 = 0.f; // scales of the two tiles still waiting to be folded in
+    i32x8 bx[4], aw[4];
+#pragma unroll
+    for(int q = 0; q < 4; ++q)
+    {
+        // first iteration: the "previous K block" is all zero codes with zero scales
+        bx[q] = i32x8{0, 0, 0, 0, 0, 0, 0, 0};
+        aw[q] = i32x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+    float scp[4] = {0.f, 0.f, 0.f, 0.f}; // x_scale * w_scale of the previous K block, per m tile
+
+    typedef const volatile float __attribute__((address_space(3)))* lds_f32_ptr;
 
     for(int kb = 0; kb < p.kblocks; ++kb)
     {
@@ -203,61 +223,87 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
             (uint32_t)(uintptr_t)(smem3 + (cur ^ 1) * kStageBytes + wave * 1024));
         const size_t   dma_koff = (size_t)kn * 128;
 
-        if((kn & 63) == 0 && kn != kb)
-            ws_vec = load_ws_window(kn);
-        const float nws = ws_at(kn);
+        if((kb & 63) == 0 && kb != 0)
+            ws_vec = load_ws_window(kb);
+        const float wsc = ws_at(kb);
 
-        // fragment reads in the order the first MFMAs need them: all 8 waves read at once
-        // right after the barrier, so the fewer bytes stand between a wave and its first MFMA
-        // the sooner the matrix pipe restarts
-        i32x8 bx[4], aw[2];
-        aw[0] = read_frag_v(stage, w_base);
-#pragma unroll
-        for(int j = 0; j < 4; ++j)
-            bx[j] = read_frag_v(stage, x_base + j * 2048);
+        aw[0] = read_frag_v(stage, w_base); // weight fragment 0 of this K block
         float sc[4];
 #pragma unroll
         for(int j = 0; j < 4; ++j)
-        {
-            typedef const volatile float __attribute__((address_space(3)))* lds_f32_ptr;
             sc[j] = *(lds_f32_ptr)(smem3 + stage + xs_lds + j * 64) * wsc;
-        }
 
 #pragma unroll
-        for(int t = 0; t < 32; ++t)
+        for(int q = 0; q < 32; ++q)
         {
-            const int i = t >> 2, j = t & 3;
-            if(j == 0 && i < 7)
-                aw[(i + 1) & 1] = read_frag_v(stage, w_base + (i + 1) * 2048);
-            FP8BS_MFMA(P[t & 3], aw[i & 1], bx[j]);
-            if((t & 1) == 1 && t < 16) // the 8 LDS-direct loads ride behind the first 16 MFMAs
+            if(q == 2)
+                aw[1] = read_frag_v(stage, w_base + 1 * 2048);
+
+            if(q < 8) // deferred tile (6 + (q & 1), q >> 1) of the previous K block
+                FP8BS_MFMA(P[q & 3], aw[2 + (q & 1)], bx[q >> 1]);
+            else      // tile ((q - 8) >> 2, (q - 8) & 3) of this K block
+                FP8BS_MFMA(P[q & 3], aw[((q - 8) >> 2) & 3], bx[(q - 8) & 3]);
+
+            // LDS reads that the slot just issued has made room for
+            if(q < 8 && (q & 1))
+                bx[q >> 1] = read_frag_v(stage, x_base + (q >> 1) * 2048);
+            if(q == 6)
+                aw[2] = read_frag_v(stage, w_base + 2 * 2048);
+            if(q == 7)
+                aw[3] = read_frag_v(stage, w_base + 3 * 2048);
+            if(q == 11)
+                aw[0] = read_frag_v(stage, w_base + 4 * 2048);
+            if(q == 15)
+                aw[1] = read_frag_v(stage, w_base + 5 * 2048);
+            if(q == 19)
+                aw[2] = read_frag_v(stage, w_base + 6 * 2048);
+            if(q == 23)
+                aw[3] = read_frag_v(stage, w_base + 7 * 2048);
+
+            // next stage: 8 slab loads and the x_scale column, behind the first 17 slots
+            if((q & 1) == 1 && q < 16)
             {
-                const int i = t >> 1;
-                dma16(dma_dst + i * 8192, goff[i], (i < 4 ? p.wq : p.xq) + dma_koff);
+                const int u = q >> 1;
+                dma16(dma_dst + u * 8192, goff[u], (u < 4 ? p.wq : p.xq) + dma_koff);
             }
-            if(t == 16 && wave < 4)
+            if(q == 16 && wave < 4)
                 dma4(__builtin_amdgcn_readfirstlane(dma_dst - wave * 1024 + kSlabBytes + wave * 256),
                      xs_goff + (uint32_t)kn * 4u, p.xs);
-            if(t == 0)
-                FP8BS_FMA4(acc[7][2], P[2], psc2);
-            else if(t == 1)
-                FP8BS_FMA4(acc[7][3], P[3], psc3);
-            else
-                FP8BS_FMA4(acc[(t - 2) >> 2][(t - 2) & 3], P[(t - 2) & 3], sc[(t - 2) & 3]);
-        }
-        psc2 = sc[2];
-        psc3 = sc[3];
 
-        // vmcnt(0): this wave's share of the next stage is in LDS
+            // fold in the product issued two slots ago
+            if(q == 0)
+                FP8BS_FMA4(acc[5][2], P[2], scp[2]);
+            else if(q == 1)
+                FP8BS_FMA4(acc[5][3], P[3], scp[3]);
+            else if(q < 10)
+                FP8BS_FMA4(acc[6 + ((q - 2) & 1)][(q - 2) >> 1], P[(q - 2) & 3], scp[(q - 2) >> 1]);
+            else
+                FP8BS_FMA4(acc[(q - 10) >> 2][(q - 10) & 3], P[(q - 2) & 3], sc[(q - 10) & 3]);
+        }
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+            scp[j] = sc[j];
+
+        // vmcnt(0): this wave's share of the next stage is in LDS; the barrier (which also
+        // waits for this wave's outstanding LDS reads) publishes it and retires the stage just read
         __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
-        wsc = nws;
     }
-    // drain: the last two products (the barrier above is far more than the 11 wait states an
-    // 8-pass MFMA result needs, the explicit nops make that independent of it)
-    asm volatile("s_nop 15\n s_nop 15\n s_nop 15" ::: "memory");
-    FP8BS_FMA4(acc[7][2], P[2], psc2);
-    FP8BS_FMA4(acc[7][3], P[3], psc3);
+    // tail: the 8 deferred tiles of the last K block, then drain the two products in flight
+#pragma unroll
+    for(int q = 0; q < 8; ++q)
+    {
+        FP8BS_MFMA(P[q & 3], aw[2 + (q & 1)], bx[q >> 1]);
+        if(q == 0)
+            FP8BS_FMA4(acc[5][2], P[2], scp[2]);
+        else if(q == 1)
+            FP8BS_FMA4(acc[5][3], P[3], scp[3]);
+        else
+            FP8BS_FMA4(acc[6 + ((q - 2) & 1)][(q - 2) >> 1], P[(q - 2) & 3], scp[(q - 2) >> 1]);
+    }
+    asm volatile("s_nop 15\n s_nop 15\n s_nop 15" ::: "memory"); // >= 11 wait states after the last MFMA
+    FP8BS_FMA4(acc[6][3], P[2], scp[3]);
+    FP8BS_FMA4(acc[7][3], P[3], scp[3]);
 #undef FP8BS_MFMA
 #undef FP8BS_FMA4
 
