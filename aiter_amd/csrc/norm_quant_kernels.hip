@@ -108,6 +108,38 @@ __device__ __forceinline__ uint32_t group_max_u32(uint32_t v)
     return v;
 }
 
+// sum of a double over the 64 lanes of a wave, same value in every lane.  DPP permutes inside
+// each row of 16 lanes (no LDS traffic, unlike ds_bpermute-based shuffles), then the four row
+// sums are read with v_readlane and added in a fixed order.
+__device__ __forceinline__ double dpp_add_f64(double v, int which)
+{
+    uint32_t lo = (uint32_t)__double2loint(v), hi = (uint32_t)__double2hiint(v);
+    uint32_t plo, phi;
+    switch(which)
+    {
+    case 0: plo = dpp_u32<kDppXor1>(lo); phi = dpp_u32<kDppXor1>(hi); break;
+    case 1: plo = dpp_u32<kDppXor2>(lo); phi = dpp_u32<kDppXor2>(hi); break;
+    case 2: plo = dpp_u32<kDppHalfMirror>(lo); phi = dpp_u32<kDppHalfMirror>(hi); break;
+    default: plo = dpp_u32<kDppRowMirror>(lo); phi = dpp_u32<kDppRowMirror>(hi); break;
+    }
+    return v + __hiloint2double((int)phi, (int)plo);
+}
+
+__device__ __forceinline__ double wave_sum_f64(double v)
+{
+    v = dpp_add_f64(v, 0);
+    v = dpp_add_f64(v, 1);
+    v = dpp_add_f64(v, 2);
+    v = dpp_add_f64(v, 3); // every lane now holds the sum of its row of 16
+    const uint32_t lo = (uint32_t)__double2loint(v), hi = (uint32_t)__double2hiint(v);
+    double         r[4];
+#pragma unroll
+    for(int k = 0; k < 4; ++k)
+        r[k] = __hiloint2double((int)__builtin_amdgcn_readlane(hi, 16 * k),
+                                (int)__builtin_amdgcn_readlane(lo, 16 * k));
+    return (r[0] + r[1]) + (r[2] + r[3]);
+}
+
 // ---------------------------------------------------------------- the quant stage
 // v[16]: this lane's 16 consecutive elements of its group (already widened to fp32).
 // codes: their 16 e4m3fn codes in memory order.  scale: the group's scale (same in all lanes).
@@ -311,7 +343,7 @@ hipError_t launch_group_quant(const QuantArgs& a, hipStream_t stream)
 }
 
 // ---------------------------------------------------------------- RMSNorm (+add) (+quant)
-// One block per row, one lane per 16 consecutive elements (hidden <= 8192 -> <= 512 lanes).
+// One block per row, one or two 16-element units per lane (hidden <= 8192).
 // The sum of squares is accumulated in fp64 (each 16-bit float square is exact there), so the
 // mean is the correctly rounded one regardless of reduction order up to ~2^-45 relative.
 
@@ -332,128 +364,175 @@ struct NormKernelParams
     int32_t         gemma_norm;
 };
 
-template <In16 DT, bool ADD, int GS /* 0 = no quant */>
+template <In16 DT, bool ADD, int GS /* 0 = no quant */, int U /* 16-element units per lane */>
 __global__ __launch_bounds__(512) void rmsnorm_kernel(NormKernelParams p)
 {
-    const uint32_t row   = blockIdx.x;
-    const int      t     = threadIdx.x;
-    const int      e0    = t * 16;
-    const bool     act0  = e0 < p.hidden;     // first 8 elements present
-    const bool     act1  = e0 + 8 < p.hidden; // second 8 elements present
-
-    float v[16];
+    const uint32_t row = blockIdx.x;
+    const int      t   = threadIdx.x;
+    // unit j of this lane covers elements [e0[j], e0[j] + 16); consecutive lanes hold
+    // consecutive units, so loads coalesce and the lanes of one quant group stay adjacent
+    int  e0[U];
+    bool act0[U], act1[U];
 #pragma unroll
-    for(int i = 0; i < 16; ++i)
-        v[i] = 0.0f;
-
-    if(act0)
+    for(int j = 0; j < U; ++j)
     {
-        const u32x4* src = (const u32x4*)(p.x + (size_t)row * p.x_stride + e0);
-        unpack8<DT>(src[0], v);
-        if(act1)
-            unpack8<DT>(src[1], v + 8);
+        e0[j]   = (t + j * (int)blockDim.x) * 16;
+        act0[j] = e0[j] < p.hidden;     // first 8 elements present
+        act1[j] = e0[j] + 8 < p.hidden; // second 8 elements present
+    }
+
+    // every request of the lane (row, residual, weight) is issued before anything is consumed;
+    // the weight would otherwise pay its latency a second time behind the reduction
+    u32x4 xraw[U][2], rraw[U][2], wraw[U][2];
+#pragma unroll
+    for(int j = 0; j < U; ++j)
+    {
+        const u32x4 z = {0, 0, 0, 0};
+        xraw[j][0] = xraw[j][1] = rraw[j][0] = rraw[j][1] = wraw[j][0] = wraw[j][1] = z;
+        if(act0[j])
+        {
+            const u32x4* src = (const u32x4*)(p.x + (size_t)row * p.x_stride + e0[j]);
+            xraw[j][0]       = src[0];
+            if(act1[j])
+                xraw[j][1] = src[1];
+            if constexpr(ADD)
+            {
+                const u32x4* rs =
+                    (const u32x4*)(p.res_in + (size_t)row * p.res_in_stride + e0[j]);
+                rraw[j][0] = rs[0];
+                if(act1[j])
+                    rraw[j][1] = rs[1];
+            }
+            const u32x4* wsrc = (const u32x4*)(p.weight + e0[j]);
+            wraw[j][0]        = wsrc[0];
+            if(act1[j])
+                wraw[j][1] = wsrc[1];
+        }
+    }
+
+    float  v[U][16];
+    double ss = 0.0;
+#pragma unroll
+    for(int j = 0; j < U; ++j)
+    {
+        unpack8<DT>(xraw[j][0], v[j]);
+        unpack8<DT>(xraw[j][1], v[j] + 8);
         if constexpr(ADD)
         {
-            float        r[16];
-            const u32x4* rs = (const u32x4*)(p.res_in + (size_t)row * p.res_in_stride + e0);
-            unpack8<DT>(rs[0], r);
-            if(act1)
-                unpack8<DT>(rs[1], r + 8);
+            float r[16];
+            unpack8<DT>(rraw[j][0], r);
+            unpack8<DT>(rraw[j][1], r + 8);
             uint32_t h[16];
 #pragma unroll
             for(int i = 0; i < 16; ++i)
             {
-                h[i] = round16<DT>(v[i] + r[i]);
-                v[i] = widen16<DT>(h[i]);
+                h[i]    = round16<DT>(v[j][i] + r[i]);
+                v[j][i] = widen16<DT>(h[i]);
             }
-            u32x4* ro = (u32x4*)(p.res_out + (size_t)row * p.res_out_stride + e0);
-            ro[0]     = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16),
-                          h[6] | (h[7] << 16)};
-            if(act1)
-                ro[1] = u32x4{h[8] | (h[9] << 16), h[10] | (h[11] << 16), h[12] | (h[13] << 16),
-                              h[14] | (h[15] << 16)};
+            if(act0[j])
+            {
+                u32x4* ro = (u32x4*)(p.res_out + (size_t)row * p.res_out_stride + e0[j]);
+                ro[0]     = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16),
+                              h[6] | (h[7] << 16)};
+                if(act1[j])
+                    ro[1] = u32x4{h[8] | (h[9] << 16), h[10] | (h[11] << 16),
+                                  h[12] | (h[13] << 16), h[14] | (h[15] << 16)};
+            }
         }
+#pragma unroll
+        for(int i = 0; i < 16; ++i)
+            ss = __builtin_fma((double)v[j][i], (double)v[j][i], ss);
     }
+    ss = wave_sum_f64(ss);
 
-    double ss = 0.0;
-#pragma unroll
-    for(int i = 0; i < 16; ++i)
-        ss = __builtin_fma((double)v[i], (double)v[i], ss);
-#pragma unroll
-    for(int off = 32; off >= 1; off >>= 1)
-        ss += __shfl_xor(ss, off, 64);
-
-    __shared__ double part[8];
-    const int         wave = t >> 6, n_waves = blockDim.x >> 6;
+    // eight slots whatever the block size: the waves that do not exist contribute zeros, so the
+    // read-back is four wide LDS loads and a fixed tree of seven additions
+    __shared__ __attribute__((aligned(16))) double part[8];
+    const int wave = t >> 6, n_waves = blockDim.x >> 6;
     if((t & 63) == 0)
         part[wave] = ss;
+    if(t >= n_waves && t < 8)
+        part[t] = 0.0;
     __syncthreads();
-    double tot = 0.0;
-    for(int w = 0; w < n_waves; ++w)
-        tot += part[w];
+    double pr[8];
+#pragma unroll
+    for(int w = 0; w < 8; ++w)
+        pr[w] = part[w];
+    const double tot = ((pr[0] + pr[1]) + (pr[2] + pr[3])) + ((pr[4] + pr[5]) + (pr[6] + pr[7]));
 
     const float mean = (float)(tot / (double)p.hidden);
     const float rstd = 1.0f / sqrtf(mean + p.eps); // correctly rounded sqrt and division
 
-    if(!act0)
-        return;
-
+#pragma unroll
+    for(int j = 0; j < U; ++j)
     {
-        float        w[16];
-        const u32x4* ws = (const u32x4*)(p.weight + e0);
-        unpack8<DT>(ws[0], w);
-        if(act1)
-            unpack8<DT>(ws[1], w + 8);
-        else
+        if(!act0[j])
+            continue;
+        float w[16];
+        unpack8<DT>(wraw[j][0], w);
+        unpack8<DT>(wraw[j][1], w + 8);
+        if(p.gemma_norm) // uniform branch: the common case pays nothing for it
         {
 #pragma unroll
-            for(int i = 8; i < 16; ++i)
-                w[i] = 0.0f;
+            for(int i = 0; i < 16; ++i)
+                w[i] = 1.0f + w[i];
         }
         uint32_t h[16];
 #pragma unroll
         for(int i = 0; i < 16; ++i)
         {
-            float wf = p.gemma_norm ? 1.0f + w[i] : w[i];
-            float tt = v[i] * rstd;
-            float u  = tt * wf;
+            float tt = v[j][i] * rstd;
+            float u  = tt * w[i];
             h[i]     = round16<DT>(u);
-            v[i]     = widen16<DT>(h[i]);
+            v[j][i]  = widen16<DT>(h[i]);
         }
         if constexpr(GS == 0)
         {
-            u32x4* o = (u32x4*)(p.out16 + (size_t)row * p.out_stride + e0);
+            u32x4* o = (u32x4*)(p.out16 + (size_t)row * p.out_stride + e0[j]);
             o[0]     = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16),
                          h[6] | (h[7] << 16)};
-            if(act1)
+            if(act1[j])
                 o[1] = u32x4{h[8] | (h[9] << 16), h[10] | (h[11] << 16), h[12] | (h[13] << 16),
                              h[14] | (h[15] << 16)};
         }
-    }
-
-    if constexpr(GS != 0)
-    {
-        constexpr int LPG = GS / 16;
-        u32x4         codes;
-        float         s;
-        quant16<LPG>(v, codes, s);
-        *(u32x4*)(p.out8 + (size_t)row * p.out_stride + e0) = codes;
-        if(t % LPG == 0)
+        else
         {
-            const uint32_t gpr = (uint32_t)p.hidden / GS;
-            const uint32_t col = (uint32_t)t / LPG;
-            size_t idx = p.transpose_scale ? (size_t)col * p.rows + row : (size_t)row * gpr + col;
-            p.scale[idx] = s;
+            constexpr int LPG = GS / 16;
+            u32x4         codes;
+            float         s;
+            quant16<LPG>(v[j], codes, s);
+            *(u32x4*)(p.out8 + (size_t)row * p.out_stride + e0[j]) = codes;
+            const int unit = e0[j] >> 4;
+            if(unit % LPG == 0)
+            {
+                const uint32_t gpr = (uint32_t)p.hidden / GS;
+                const uint32_t col = (uint32_t)unit / LPG;
+                size_t         idx =
+                    p.transpose_scale ? (size_t)col * p.rows + row : (size_t)row * gpr + col;
+                p.scale[idx] = s;
+            }
         }
     }
 }
 
+// Rows of more than 2048 elements give each lane two units: the whole problem then fits the
+// chip in one round of blocks at the usual row counts, instead of two dependent rounds.
 template <In16 DT, bool ADD, int GS>
 static hipError_t launch_rmsnorm_t(const NormKernelParams& p, hipStream_t stream)
 {
-    int lanes   = (p.hidden + 15) / 16;
-    int threads = (lanes + 63) / 64 * 64;
-    hipLaunchKernelGGL((rmsnorm_kernel<DT, ADD, GS>), dim3(p.rows), dim3(threads), 0, stream, p);
+    const int units = (p.hidden + 15) / 16;
+    if(units > 128)
+    {
+        const int threads = ((units + 1) / 2 + 63) / 64 * 64;
+        hipLaunchKernelGGL((rmsnorm_kernel<DT, ADD, GS, 2>), dim3(p.rows), dim3(threads), 0,
+                           stream, p);
+    }
+    else
+    {
+        const int threads = (units + 63) / 64 * 64;
+        hipLaunchKernelGGL((rmsnorm_kernel<DT, ADD, GS, 1>), dim3(p.rows), dim3(threads), 0,
+                           stream, p);
+    }
     return hipGetLastError();
 }
 
