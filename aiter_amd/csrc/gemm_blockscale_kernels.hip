@@ -183,14 +183,16 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
         return launch_tile<DT, 64, 128, 2, 2>(p, stream);
     if(strcmp(name, "tile_128x128") == 0)
         return launch_tile<DT, 128, 128, 2, 2>(p, stream);
-    if(strcmp(name, "decode_stream") == 0)
+    // "decode_stream" alone, or "decode_stream:r=2,s=4,w=4,g=256" to pin its work split
+    if(strncmp(name, "decode_stream", 13) == 0 && (name[13] == 0 || name[13] == ':'))
     {
+        const char* tuning = name[13] == ':' ? name + 14 : nullptr;
         if(!gemm_decode_supports(p))
         {
             *why = "decode_stream handles 1 <= M <= 64";
             return hipErrorInvalidValue;
         }
-        return launch_gemm_decode(p, DT, a.split_k_log2, a.device_id, stream);
+        return launch_gemm_decode(p, DT, a.split_k_log2, a.device_id, stream, tuning);
     }
     if(a.split_k_log2 > 0)
     {

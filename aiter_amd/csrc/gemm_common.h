@@ -59,7 +59,7 @@ __device__ __forceinline__ uint32_t lds_off(uint32_t row, uint32_t chunk)
 hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, hipStream_t stream);
 bool       gemm_prefill_supports(const GemmKernelParams& p);
 hipError_t launch_gemm_decode(const GemmKernelParams& p, In16 out_dtype, int split_k_log2, int device_id,
-                              hipStream_t stream);
+                              hipStream_t stream, const char* tuning = nullptr);
 bool       gemm_decode_supports(const GemmKernelParams& p);
 
 } // namespace fp8bs

@@ -1,256 +1,418 @@
-// Decode-shape block-scale FP8 GEMM (M <= 64): weight streaming, HBM-bound.
+// Decode-shape block-scale FP8 GEMM (M <= 64): weight streaming, bound by how fast a compute
+// unit can pull bytes in.
 //
-// The weight matrix is read exactly once, straight from global memory into registers in the
-// MFMA "A" operand layout (lane = weight row l%16, 32 bytes of one 128-wide K block), with every
-// load of a wave's share issued before anything is consumed, so a wave keeps up to 32 KiB in
-// flight and the whole matrix is requested from HBM at once.  The (small) activation matrix and
-// its scales are staged once per workgroup in LDS and shared by its 4 waves.
+// A compute unit keeps only a few tens of KiB of memory requests in flight, so the kernel is
+// built to (a) spread the weight matrix over every compute unit of the chip, (b) bring each
+// byte in exactly once, straight into registers in MFMA operand layout, and (c) keep the
+// activations from multiplying that traffic.
 //
-// Work split: a workgroup owns 64 weight rows (16 per wave) and one K chunk.  When N alone gives
-// too few workgroups to keep the memory system busy, K is split across workgroups as well; the
-// fp32 partial tiles go to a workspace and the last workgroup to finish a row block (an atomic
-// ticket) adds them in a fixed order, so results do not depend on arrival order.
+// Work split.  A workgroup owns a group of R 16-row weight tiles and one K range; its waves
+// split that K range between them, 4 K blocks (512 bytes of every row) per wave and step.
+// A wave therefore needs only its own K slice of the activations, which it keeps in registers
+// as MFMA "B" fragments for the life of the workgroup; no LDS staging, no re-reads.  The
+// per-wave fp32 partial tiles are added through LDS in wave order.  A workgroup that owns
+// several row groups walks them with the next group's weights already requested.
+//
+// When N alone gives too few workgroups to cover the chip, the K range is also split across
+// workgroups; their fp32 partial tiles go to a workspace and the last workgroup to finish a
+// row group (an atomic ticket) adds them in split order, so results never depend on timing.
 #include "gemm_common.h"
+
+#include <stdlib.h>
+#include <string.h>
 
 namespace fp8bs {
 
 namespace {
 
-constexpr int kRowsPerWave = 16, kWaves = 4, kRowsPerBlock = kRowsPerWave * kWaves;
-constexpr int kThreads   = 64 * kWaves;
-constexpr int kMaxChunkKb = 16; // K blocks per chunk: 16 x 2 loads x 16 B = 512 B in flight per lane
+constexpr int kStepKb = 4; // K blocks per wave and step
+constexpr int kMaxDynamicLds = 128 * 1024;
 
 struct DecodeParams
 {
     GemmKernelParams g;
-    int32_t  m_tiles;      // ceil(M / 16), 1..4
-    int32_t  chunk_kb;     // K blocks per workgroup chunk
-    int32_t  chunk_kb_pad; // chunk_kb rounded up to a multiple of 8 (LDS row pitch)
-    int32_t  splits;       // number of K chunks
-    float*   partial;      // [splits][n_blocks * 64][m_tiles * 16] fp32 when splits > 1
-    uint32_t* tickets;     // [n_blocks] zero between launches
+    int32_t   n_tiles;      // ceil(N / 16)
+    int32_t   n_groups;     // ceil(n_tiles / R)
+    int32_t   kb_per_split; // K blocks per workgroup-level K range
+    int32_t   splits;       // number of such ranges (grid.y)
+    int32_t   bf16_out;
+    int32_t   park_slots;   // row groups whose partial tiles fit in LDS between two flushes
+    int32_t   xs_vec4;      // x_scale rows can be read four K blocks at a time (16-byte aligned)
+    float*    partial;      // [splits][n_groups][R * MT * 64] x 4 fp32 when splits > 1
+    uint32_t  partial_bytes;
+    uint32_t* tickets;      // [n_groups], zero between launches
 };
 
-__device__ __forceinline__ uint32_t x_lds_off(uint32_t row, uint32_t kb, uint32_t chunk, uint32_t row_bytes)
+__device__ __forceinline__ u32x2 pack4(const f32x4& v, bool bf)
 {
-    return row * row_bytes + kb * 128u + ((chunk ^ (row & 7u)) << 4);
+    return bf ? u32x2{pack2<In16::bf16>(v[0], v[1]), pack2<In16::bf16>(v[2], v[3])}
+              : u32x2{pack2<In16::fp16>(v[0], v[1]), pack2<In16::fp16>(v[2], v[3])};
 }
 
-template <In16 DT, int MT, int KBMAX>
-__global__ __launch_bounds__(kThreads) void gemm_decode_kernel(DecodeParams p)
+template <int MT>
+constexpr int decode_max_waves()
+{
+    return 4; // one wave per SIMD: each may use the whole 512-register file
+}
+
+// FULL: every step of every wave holds exactly 4 K blocks (K is a multiple of 512), which
+// makes the multiply straight-line code; otherwise the block count of a step is a run-time value.
+template <int MT, int R, bool SINGLE, bool FULL>
+__global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kernel(DecodeParams p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const GemmKernelParams& g = p.g;
 
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int nw   = (int)blockDim.x >> 6;
     const int l16 = lane & 15, kg = lane >> 4;
-    const int nblk  = blockIdx.x;            // 64-row block of the weight
     const int split = blockIdx.y;
-    const int kb0   = split * p.chunk_kb;
-    const int nkb   = min(p.chunk_kb, g.kblocks - kb0);
-    const int n_row = nblk * kRowsPerBlock + wave * kRowsPerWave + l16;
-    const int n_ld  = n_row < g.N ? n_row : g.N - 1; // ragged N: load a valid row, never store it
+    const int kb_lo = split * p.kb_per_split;
+    const int kb_hi = min(kb_lo + p.kb_per_split, g.kblocks);
+    constexpr int E = R * MT * 64; // f32x4 elements of a workgroup's output tile set
 
-    // ---- 1. activations for this K chunk -> LDS with LDS-direct loads (no registers, all in
-    // flight at once).  One instruction moves one activation row x 8 K blocks (1 KiB): lane p
-    // fills LDS chunk p of that KiB = K block p/8, stored chunk p%8, which must hold the row's
-    // logical chunk (p%8) ^ (row&7).  Rows and K blocks past the end are clamped (re-fetched,
-    // never used).  Issued before the weight loads so that they are the oldest in the queue.
-    const uint32_t x_row_bytes = (uint32_t)p.chunk_kb_pad * 128u;
-    uint8_t*       sX          = smem;
-    float*         sS          = (float*)(smem + (size_t)MT * 16 * x_row_bytes);
-    {
-        typedef uint8_t __attribute__((address_space(3)))* lds_byte_ptr;
-        const uint32_t lds0   = (uint32_t)(uintptr_t)(lds_byte_ptr)smem;
-        const int      groups = p.chunk_kb_pad >> 3;          // 8-K-block groups per row
-        const int      units  = MT * 16 * groups;             // 1 KiB units in the chunk
-        for(int u = wave; u < units; u += kWaves)
-        {
-            const int row = u / groups, grp = u - row * groups;
-            const int m   = row < g.M ? row : g.M - 1;
-            int       kb  = grp * 8 + (lane >> 3);
-            kb            = kb < nkb ? kb : nkb - 1;
-            const uint32_t c    = (uint32_t)(lane & 7) ^ (uint32_t)(row & 7);
-            const uint32_t voff = (uint32_t)m * (uint32_t)g.lda + (uint32_t)(kb0 + kb) * 128u + c * 16u;
-            const uint32_t dst  = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)row * x_row_bytes + (uint32_t)grp * 1024u);
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                         :
-                         : "s"(dst), "v"(voff), "s"(g.xq)
-                         : "memory");
-        }
-    }
-    // x_scale of the chunk: at most 4 values per thread, all requested before any is used
-    float sval[4];
-    {
-        const int total = MT * 16 * nkb;
-#pragma unroll
-        for(int i = 0; i < 4; ++i)
-        {
-            const int q   = t + i * kThreads;
-            const int qq  = q < total ? q : total - 1;
-            const int row = qq / nkb, k = qq - row * nkb;
-            const int m   = row < g.M ? row : g.M - 1;
-            sval[i]       = g.xs[(size_t)m * g.kblocks + kb0 + k];
-        }
-    }
+    // Global loads are issued row-segment-wise: 8 consecutive lanes fetch one 128-byte K block of
+    // one row, so a load instruction touches 8 cache lines in full.  (Fetching straight into the
+    // MFMA layout, 16 rows x 16 bytes per quarter wave, costs a tag lookup per 16 bytes and
+    // caps a compute unit far below what the memory system delivers.)  The wave then turns each
+    // 16-row x 128-byte unit into MFMA fragments through a private 2 KiB LDS slot: written as
+    // loaded, read back fragment-wise; the bank swizzle of that slot is applied on the global
+    // side, by which 16-byte chunk of its row a lane fetches.
+    const int crow = lane >> 3, cchunk = (lane & 7) ^ crow;
+    uint8_t*  slot = smem + (size_t)wave * 2048;
+    auto      settle = [&](const u32x4(&raw)[2]) -> i32x8 {
+        *(u32x4*)(slot + lane * 16)        = raw[0];
+        *(u32x4*)(slot + 1024 + lane * 16) = raw[1];
+        const i32x4 lo = *(const i32x4*)(slot + lds_off(l16, 2 * kg));
+        const i32x4 hi = *(const i32x4*)(slot + lds_off(l16, 2 * kg + 1));
+        return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
 
-    // w_scale of this wave's rows: one 128-row block (16 | 128, so a wave never straddles two).
-    // The block index is wave-uniform; saying so turns these into scalar loads that are all
-    // issued here instead of one dependent vector load per K block inside the multiply loop.
-    const int nb = __builtin_amdgcn_readfirstlane(
-        min((nblk * kRowsPerBlock + wave * kRowsPerWave) >> 7, (g.N + 127) / 128 - 1));
-    const float* ws_row = g.ws + (size_t)nb * g.kblocks + kb0;
-    float        wsv[KBMAX];
-#pragma unroll
-    for(int k = 0; k < KBMAX; ++k)
-        wsv[k] = ws_row[k < nkb ? k : nkb - 1];
-
-    // ---- 2. every weight load of this wave, up front and unconditional: the kernel is
-    // instantiated for chunk capacities of 4, 8, 12 and 16 K blocks, and the (at most 3) slots
-    // past the end of a shorter chunk re-read its last K block (a cache hit, never used).
-    // Straight-line loads let the compiler count them, so each K block below waits only for its
-    // own two loads and the multiply overlaps the arrival of the rest.
-    u32x4 wlo[KBMAX], whi[KBMAX];
-    {
-        const uint8_t* wp = g.wq + (size_t)n_ld * g.ldb + (size_t)kb0 * 128 + kg * 32;
-#pragma unroll
-        for(int k = 0; k < KBMAX; ++k)
-        {
-            const int kk = k < nkb ? k : nkb - 1;
-            wlo[k]       = __builtin_nontemporal_load((const u32x4*)(wp + kk * 128));
-            whi[k]       = __builtin_nontemporal_load((const u32x4*)(wp + kk * 128 + 16));
-        }
-    }
-    {
-        // Using the scale values makes the compiler wait for their loads; loads return in
-        // order, so the older LDS-direct loads of this wave have landed by then as well.
-        const int total = MT * 16 * nkb;
-#pragma unroll
-        for(int i = 0; i < 4; ++i)
-        {
-            const int q = t + i * kThreads;
-            if(q < total)
-            {
-                const int row = q / nkb, k = q - row * nkb;
-                sS[row * p.chunk_kb + k] = sval[i];
-            }
-        }
-    }
-    __syncthreads();
-
-    // ---- 3. multiply: one MFMA per (K block, m tile), scaled into fp32 accumulators
-    f32x4 acc[MT];
+    // activation rows this lane fetches (two per m tile: rows crow and 8 + crow of the tile) and
+    // the row whose scales it needs (rows past M re-read the last one, never stored)
+    const uint8_t* xrow[MT][2];
+    const float*   xsrow[MT];
 #pragma unroll
     for(int j = 0; j < MT; ++j)
-        acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-#pragma unroll
-    for(int k = 0; k < KBMAX; ++k)
     {
-        if(k < nkb)
-        {
-            // activation fragments and scales of this K block first (LDS), then the weights
-            i32x8 bx[MT];
-            float sc[MT];
 #pragma unroll
-            for(int j = 0; j < MT; ++j)
-            {
-                const uint32_t row = j * 16 + l16;
-                const i32x4    lo  = *(const i32x4*)(sX + x_lds_off(row, k, 2 * kg, x_row_bytes));
-                const i32x4    hi  = *(const i32x4*)(sX + x_lds_off(row, k, 2 * kg + 1, x_row_bytes));
-                bx[j]              = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                sc[j]              = sS[row * p.chunk_kb + k] * wsv[k];
-            }
-            const i32x8 aw = i32x8{(int)wlo[k][0], (int)wlo[k][1], (int)wlo[k][2], (int)wlo[k][3],
-                                   (int)whi[k][0], (int)whi[k][1], (int)whi[k][2], (int)whi[k][3]};
-            f32x4 part[MT];
-#pragma unroll
-            for(int j = 0; j < MT; ++j)
-                part[j] = mfma_16x16x128_fp8(aw, bx[j], f32x4{0.f, 0.f, 0.f, 0.f});
-#pragma unroll
-            for(int j = 0; j < MT; ++j)
-#pragma unroll
-                for(int r = 0; r < 4; ++r)
-                    acc[j][r] = __builtin_fmaf(part[j][r], sc[j], acc[j][r]);
-        }
+        for(int h = 0; h < 2; ++h)
+            xrow[j][h] = g.xq + (size_t)min(j * 16 + h * 8 + crow, g.M - 1) * g.lda + cchunk * 16;
+        xsrow[j] = g.xs + (size_t)min(j * 16 + l16, g.M - 1) * g.kblocks;
     }
 
-    // lane owns out[m = j*16 + l16][n .. n+3], n = block row base + wave*16 + kg*4
-    const int n_out = nblk * kRowsPerBlock + wave * kRowsPerWave + kg * 4;
+    i32x8 bx[MT][kStepKb];
+    float xsv[MT][kStepKb];
+    f32x4 acc[R][MT];
 
-    auto store_out = [&](const f32x4 (&v)[MT]) {
+    // K block i of a step that starts at kb0 and holds nk (1..4) blocks; slots past the end
+    // re-read the last block (a cache hit) and are never multiplied
+    auto kslot = [&](int kb0, int nk, int i) { return FULL ? kb0 + i : kb0 + (i < nk ? i : nk - 1); };
+
+    // Requests go out row by row with a row's K blocks back to back (512 contiguous bytes per
+    // row close together in time suits the DRAM pages), weights first: they come from furthest
+    // away.  Loads return in order, so the activation tiles, requested last, can be multiplied
+    // one m tile at a time while the later ones are still on their way.
+    auto issue_w = [&](int grp, int kb0, int nk, u32x4(&raw)[R][kStepKb][2], float(&s)[R][kStepKb]) {
+#pragma unroll
+        for(int r = 0; r < R; ++r)
+        {
+            const int    tile = min(grp * R + r, p.n_tiles - 1);
+            const float* wsp  = g.ws + (size_t)((tile * 16) >> 7) * g.kblocks; // wave-uniform
+#pragma unroll
+            for(int h = 0; h < 2; ++h)
+            {
+                const int      n  = min(tile * 16 + h * 8 + crow, g.N - 1);
+                const uint8_t* wp = g.wq + (size_t)n * g.ldb + cchunk * 16;
+#pragma unroll
+                for(int i = 0; i < kStepKb; ++i)
+                    raw[r][i][h] =
+                        __builtin_nontemporal_load((const u32x4*)(wp + (size_t)kslot(kb0, nk, i) * 128));
+            }
+#pragma unroll
+            for(int i = 0; i < kStepKb; ++i)
+                s[r][i] = wsp[kslot(kb0, nk, i)];
+        }
+    };
+    auto issue_x = [&](int kb0, int nk, u32x4(&raw)[MT][kStepKb][2]) {
 #pragma unroll
         for(int j = 0; j < MT; ++j)
         {
-            const int m = j * 16 + l16;
-            if(m >= g.M)
-                continue;
-            uint16_t* dst = g.out + (size_t)m * g.N + n_out;
-            if(n_out + 3 < g.N && (g.N & 3) == 0)
-                *(u32x2*)dst = u32x2{pack2<DT>(v[j][0], v[j][1]), pack2<DT>(v[j][2], v[j][3])};
+#pragma unroll
+            for(int h = 0; h < 2; ++h)
+#pragma unroll
+                for(int i = 0; i < kStepKb; ++i)
+                    raw[j][i][h] = *(const u32x4*)(xrow[j][h] + (size_t)kslot(kb0, nk, i) * 128);
+            if((FULL || nk == kStepKb) && p.xs_vec4) // the four scales of the step in one load
+            {
+                const f32x4 v = *(const f32x4*)(xsrow[j] + kb0);
+#pragma unroll
+                for(int i = 0; i < kStepKb; ++i)
+                    xsv[j][i] = v[i];
+            }
             else
             {
 #pragma unroll
-                for(int r = 0; r < 4; ++r)
-                    if(n_out + r < g.N)
-                        dst[r] = (uint16_t)(pack2<DT>(v[j][r], 0.f) & 0xffffu);
+                for(int i = 0; i < kStepKb; ++i)
+                    xsv[j][i] = xsrow[j][kslot(kb0, nk, i)];
             }
         }
     };
 
-    if(p.splits == 1)
-    {
-        store_out(acc);
-        return;
-    }
-
-    // ---- 4. split K: park the partial tile, take a ticket, last one in adds them up.
-    // The workgroups of one row block run on different XCDs, whose L2 caches are not coherent
-    // with each other.  Instead of device-wide fences (which write back and invalidate a whole
-    // L2, once per workgroup), every access to the exchanged data is itself device-coherent:
-    // partials are written with agent-scope stores (write-through) and waited for (vmcnt 0)
-    // before this workgroup's ticket is taken with an agent-scope atomic; the last workgroup
-    // reads them back with agent-scope loads, which cannot be served from a stale L2 line.
-    const size_t n_pad   = (size_t)gridDim.x * kRowsPerBlock;
-    const size_t m_pad   = (size_t)MT * 16;
-    const size_t plane   = n_pad * m_pad; // one split's partials, laid out [m][n_pad]
-    float*       my_part = p.partial + (size_t)split * plane;
-#pragma unroll
-    for(int j = 0; j < MT; ++j)
-    {
-        float* dst = my_part + (size_t)(j * 16 + l16) * n_pad + n_out;
-#pragma unroll
-        for(int r = 0; r < 4; ++r)
-            __hip_atomic_store(dst + r, acc[j][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): the stores above have reached memory
-    __shared__ uint32_t s_ticket;
-    __syncthreads();
-    if(t == 0)
-        s_ticket = __hip_atomic_fetch_add(p.tickets + nblk, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if(s_ticket != (uint32_t)p.splits - 1)
-        return;
-    if(t == 0) // leave the ticket ready for the next launch
-        __hip_atomic_store(p.tickets + nblk, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-
-    f32x4 sum[MT];
-#pragma unroll
-    for(int j = 0; j < MT; ++j)
-        sum[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for(int s = 0; s < p.splits; ++s) // fixed order: independent of which workgroup came last
-    {
-        const float* part = p.partial + (size_t)s * plane;
+    auto settle_x = [&](const u32x4(&raw)[MT][kStepKb][2]) {
 #pragma unroll
         for(int j = 0; j < MT; ++j)
-        {
-            const float* src = part + (size_t)(j * 16 + l16) * n_pad + n_out;
 #pragma unroll
-            for(int r = 0; r < 4; ++r)
-                sum[j][r] += __hip_atomic_load(src + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for(int i = 0; i < kStepKb; ++i)
+                bx[j][i] = settle(raw[j][i]);
+    };
+    // one weight unit at a time: fragments out of the raw registers, then its MT tile products,
+    // scaled and accumulated
+    auto multiply = [&](int nk, const u32x4(&wraw)[R][kStepKb][2], const float(&s)[R][kStepKb]) {
+#pragma unroll
+        for(int r = 0; r < R; ++r)
+#pragma unroll
+            for(int i = 0; i < kStepKb; ++i)
+            {
+                if(FULL || i < nk) // wave-uniform
+                {
+                    const i32x8 w = settle(wraw[r][i]);
+#pragma unroll
+                    for(int j = 0; j < MT; ++j)
+                    {
+                        const f32x4 part = mfma_16x16x128_fp8(w, bx[j][i], f32x4{0.f, 0.f, 0.f, 0.f});
+                        const float sc   = xsv[j][i] * s[r][i];
+#pragma unroll
+                        for(int c = 0; c < 4; ++c)
+                            acc[r][j][c] = __builtin_fmaf(part[c], sc, acc[r][j][c]);
+                    }
+                }
+            }
+    };
+    auto clear_acc = [&]() {
+#pragma unroll
+        for(int r = 0; r < R; ++r)
+#pragma unroll
+            for(int j = 0; j < MT; ++j)
+                acc[r][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    };
+
+    // element e of a group's tile set -> (row tile r, m tile j, lane ln): that lane's 4 outputs
+    auto store_out = [&](int grp, int e, const f32x4& v) {
+        const int r = e / (MT * 64), j = (e >> 6) % MT, ln = e & 63;
+        const int tile = grp * R + r;
+        const int m = j * 16 + (ln & 15), n = tile * 16 + (ln >> 4) * 4;
+        if(tile >= p.n_tiles || m >= g.M)
+            return;
+        uint16_t* dst = g.out + (size_t)m * g.N + n;
+        const u32x2 o = pack4(v, p.bf16_out != 0);
+        if(n + 3 < g.N && (g.N & 3) == 0)
+            *(u32x2*)dst = o;
+        else
+        {
+#pragma unroll
+            for(int c = 0; c < 4; ++c)
+                if(n + c < g.N)
+                    dst[c] = (uint16_t)((o[c >> 1] >> (16 * (c & 1))) & 0xffffu);
+        }
+    };
+
+    __shared__ uint32_t s_ticket;
+    const __amdgpu_buffer_rsrc_t part_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(p.partial, 0, p.splits > 1 ? (int)p.partial_bytes : 0, 0x00020000);
+    constexpr int kCoherent = 16; // cache-policy bit sc1: served by memory, not by a per-XCD L2
+
+    // Per-wave partial tiles are parked in LDS without any synchronisation while the workgroup
+    // streams through its row groups; every p.park_slots groups (and at the end) they are added
+    // up in wave order and stored.
+    f32x4* const parked = (f32x4*)(smem + (size_t)nw * 2048);
+    auto park = [&](int q) {
+        f32x4* mine = parked + ((size_t)q * nw + wave) * E;
+#pragma unroll
+        for(int r = 0; r < R; ++r)
+#pragma unroll
+            for(int j = 0; j < MT; ++j)
+                mine[(r * MT + j) * 64 + lane] = acc[r][j];
+    };
+    // sum over the waves of element e of a parked tile set, in wave order; all reads are issued
+    // before the first addition (reads past the last wave repeat it and are not added)
+    constexpr int kMaxWaves = decode_max_waves<MT>();
+    auto          wave_sum  = [&](const f32x4* red, int e) -> f32x4 {
+        f32x4 v[kMaxWaves];
+#pragma unroll
+        for(int w = 0; w < kMaxWaves; ++w)
+            v[w] = red[(size_t)min(w, nw - 1) * E + e];
+        f32x4 sum = v[0];
+#pragma unroll
+        for(int w = 1; w < kMaxWaves; ++w)
+            sum = w < nw ? sum + v[w] : sum;
+        return sum;
+    };
+    auto flush_group_split = [&](int grp, const f32x4* red) {
+        // The workgroups that share a row group run on different XCDs, whose L2 caches are not
+        // coherent with each other; every access to the exchanged tiles therefore bypasses them
+        // (sc1), and the stores are waited for before the ticket is taken.
+        for(int e = t; e < E; e += (int)blockDim.x)
+        {
+            const f32x4    s   = wave_sum(red, e);
+            const uint32_t off = (uint32_t)(((size_t)split * p.n_groups + grp) * E + e) * 16u;
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, s), part_rsrc, off, 0, kCoherent);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): the stores above have reached memory
+        __syncthreads();
+        if(t == 0)
+            s_ticket = __hip_atomic_fetch_add(p.tickets + grp, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if(s_ticket != (uint32_t)p.splits - 1)
+            return;
+        if(t == 0) // leave the ticket ready for the next launch
+            __hip_atomic_store(p.tickets + grp, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for(int e = t; e < E; e += (int)blockDim.x)
+        {
+            f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
+            for(int sp = 0; sp < p.splits; ++sp) // split order, whoever arrived last
+            {
+                const uint32_t off = (uint32_t)(((size_t)sp * p.n_groups + grp) * E + e) * 16u;
+                s += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, off, 0, kCoherent));
+            }
+            store_out(grp, e, s);
+        }
+    };
+    // groups first_grp, first_grp + gridDim.x, ... (count of them) are parked in slots 0..count-1
+    auto flush = [&](int first_grp, int count, bool last) {
+        __syncthreads();
+        if(p.splits == 1)
+        {
+            // four elements per thread and pass, all LDS reads of a pass issued together
+            const int total = count * E, T = (int)blockDim.x;
+            for(int base = t; base < total; base += 4 * T)
+            {
+                f32x4 sum[4];
+#pragma unroll
+                for(int u = 0; u < 4; ++u)
+                {
+                    const int idx = min(base + u * T, total - 1);
+                    const int q = idx / E, e = idx - q * E;
+                    sum[u] = wave_sum(parked + (size_t)q * nw * E, e);
+                }
+#pragma unroll
+                for(int u = 0; u < 4; ++u)
+                {
+                    const int idx = base + u * T;
+                    if(idx < total)
+                    {
+                        const int q = idx / E, e = idx - q * E;
+                        store_out(first_grp + q * (int)gridDim.x, e, sum[u]);
+                    }
+                }
+            }
+        }
+        else
+        {
+            for(int q = 0; q < count; ++q)
+                flush_group_split(first_grp + q * (int)gridDim.x, parked + (size_t)q * nw * E);
+        }
+        if(!last)
+            __syncthreads(); // the slots are free again
+    };
+
+    const int stride = gridDim.x;
+    int       grp = blockIdx.x, q = 0, q_first = grp;
+    auto      parked_one = [&](bool last) {
+        park(q);
+        if(++q == p.park_slots || last)
+        {
+            flush(q_first, q, last);
+            q       = 0;
+            q_first = grp + stride;
+        }
+    };
+
+    if constexpr(SINGLE)
+    {
+        // one step per wave covers the K range: activations stay in registers for the life of
+        // the workgroup, and while a row group is multiplied the next one's weights are already
+        // requested into the other of two register sets (no copies: reading a register that a
+        // load is still to fill would wait for that load)
+        const int kb0 = kb_lo + wave * kStepKb;
+        const int nk  = max(0, min(kStepKb, kb_hi - kb0));
+        u32x4     raw_a[R][kStepKb][2], raw_b[R][kStepKb][2];
+        float     ws_a[R][kStepKb], ws_b[R][kStepKb];
+        {
+            u32x4      xraw[MT][kStepKb][2];
+            const bool more = grp + stride < p.n_groups;
+            clear_acc();
+            if(nk > 0)
+            {
+                issue_w(grp, kb0, nk, raw_a, ws_a);
+                issue_x(kb0, nk, xraw);
+                settle_x(xraw); // the raw activation registers are free before the prefetch
+                if(more)
+                {
+                    issue_w(grp + stride, kb0, nk, raw_b, ws_b);
+                    multiply(nk, raw_a, ws_a);
+                }
+                else
+                    multiply(nk, raw_a, ws_a);
+            }
+            parked_one(!more);
+            grp += stride;
+        }
+        while(grp < p.n_groups) // raw_b holds this group
+        {
+            bool more = grp + stride < p.n_groups;
+            clear_acc();
+            if(nk > 0)
+            {
+                if(more)
+                {
+                    issue_w(grp + stride, kb0, nk, raw_a, ws_a);
+                    multiply(nk, raw_b, ws_b);
+                }
+                else
+                    multiply(nk, raw_b, ws_b);
+            }
+            parked_one(!more);
+            grp += stride;
+            if(grp >= p.n_groups)
+                break;
+            more = grp + stride < p.n_groups; // raw_a holds this group
+            clear_acc();
+            if(nk > 0)
+            {
+                if(more)
+                {
+                    issue_w(grp + stride, kb0, nk, raw_b, ws_b);
+                    multiply(nk, raw_a, ws_a);
+                }
+                else
+                    multiply(nk, raw_a, ws_a);
+            }
+            parked_one(!more);
+            grp += stride;
         }
     }
-    store_out(sum);
+    else
+    {
+        // long K: every wave takes several steps; activations are re-read per row group
+        for(; grp < p.n_groups; grp += stride)
+        {
+            clear_acc();
+            for(int kb0 = kb_lo + wave * kStepKb; kb0 < kb_hi; kb0 += nw * kStepKb)
+            {
+                const int nk = min(kStepKb, kb_hi - kb0);
+                u32x4     wraw[R][kStepKb][2];
+                u32x4     xraw[MT][kStepKb][2];
+                float     wsv[R][kStepKb];
+                issue_w(grp, kb0, nk, wraw, wsv);
+                issue_x(kb0, nk, xraw);
+                settle_x(xraw);
+                multiply(nk, wraw, wsv);
+            }
+            parked_one(grp + stride >= p.n_groups);
+        }
+    }
 }
 
 // workspace for split-K partials and tickets, one per device, grown on demand and kept for the
@@ -265,30 +427,30 @@ struct Workspace
 constexpr int kMaxDevices = 64;
 Workspace     g_ws[kMaxDevices];
 
-hipError_t ensure_workspace(int dev, size_t partial_floats, size_t n_tickets, hipStream_t stream,
+hipError_t ensure_workspace(int dev, size_t partial_bytes, size_t n_tickets, hipStream_t stream,
                             Workspace** out)
 {
     if(dev < 0 || dev >= kMaxDevices)
         return hipErrorInvalidDevice;
     Workspace& w = g_ws[dev];
-    if(w.partial_size < partial_floats)
+    if(w.partial_size < partial_bytes)
     {
         if(w.partial)
             (void)hipFree(w.partial);
         w.partial      = nullptr;
         w.partial_size = 0;
-        hipError_t e   = hipMalloc((void**)&w.partial, partial_floats * sizeof(float));
+        hipError_t e   = hipMalloc((void**)&w.partial, partial_bytes);
         if(e != hipSuccess)
             return e;
-        w.partial_size = partial_floats;
+        w.partial_size = partial_bytes;
     }
     if(w.n_tickets < n_tickets)
     {
         if(w.tickets)
             (void)hipFree(w.tickets);
-        w.tickets   = nullptr;
-        w.n_tickets = 0;
-        size_t n    = n_tickets < 4096 ? 4096 : n_tickets;
+        w.tickets    = nullptr;
+        w.n_tickets  = 0;
+        size_t     n = n_tickets < 4096 ? 4096 : n_tickets;
         hipError_t e = hipMalloc((void**)&w.tickets, n * sizeof(uint32_t));
         if(e != hipSuccess)
             return e;
@@ -301,86 +463,166 @@ hipError_t ensure_workspace(int dev, size_t partial_floats, size_t n_tickets, hi
     return hipSuccess;
 }
 
+// reads "key=value" integers out of a comma-separated tuning string; 0 when absent
+int tuning_value(const char* tuning, const char* key)
+{
+    if(tuning == nullptr)
+        return 0;
+    const size_t klen = strlen(key);
+    for(const char* s = tuning; *s;)
+    {
+        if(strncmp(s, key, klen) == 0 && s[klen] == '=')
+            return atoi(s + klen + 1);
+        const char* c = strchr(s, ',');
+        if(c == nullptr)
+            break;
+        s = c + 1;
+    }
+    return 0;
+}
+
+template <int MT, int R, bool SINGLE, bool FULL>
+hipError_t launch_one(const DecodeParams& p, dim3 grid, int waves, size_t smem, hipStream_t stream)
+{
+    auto        kernel = gemm_decode_kernel<MT, R, SINGLE, FULL>;
+    static bool raised[kMaxDevices]; // dynamic LDS above the default limit needs opting in, once
+    int         dev = 0;
+    (void)hipGetDevice(&dev);
+    if(dev >= 0 && dev < kMaxDevices && !raised[dev])
+    {
+        hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           kMaxDynamicLds);
+        if(e != hipSuccess)
+            return e;
+        raised[dev] = true;
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(64 * waves), smem, stream, p);
+    return hipGetLastError();
+}
+
+template <int MT, int R>
+hipError_t launch_mt_r(const DecodeParams& p, bool single, bool full, dim3 grid, int waves, size_t smem,
+                       hipStream_t stream)
+{
+    if(single)
+        return full ? launch_one<MT, R, true, true>(p, grid, waves, smem, stream)
+                    : launch_one<MT, R, true, false>(p, grid, waves, smem, stream);
+    return full ? launch_one<MT, R, false, true>(p, grid, waves, smem, stream)
+                : launch_one<MT, R, false, false>(p, grid, waves, smem, stream);
+}
+
+template <int MT>
+hipError_t launch_mt(const DecodeParams& p, int rows, bool single, bool full, dim3 grid, int waves,
+                     size_t smem, hipStream_t stream)
+{
+    return rows == 2 ? launch_mt_r<MT, 2>(p, single, full, grid, waves, smem, stream)
+                     : launch_mt_r<MT, 1>(p, single, full, grid, waves, smem, stream);
+}
+
 } // namespace
 
 bool gemm_decode_supports(const GemmKernelParams& p) { return p.M >= 1 && p.M <= 64 && p.kblocks >= 1; }
 
-// split_k_log2 < 0: choose.  Otherwise 2^split_k_log2 chunks (rounded so chunks hold <= 16 K blocks).
+// split_k_log2 < 0: choose.  Otherwise 2^split_k_log2 K ranges (rounded to whole steps).
+// `tuning` may override the choices: "r=<row tiles per group>,s=<K ranges>,w=<waves>,g=<grid.x>".
 hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int split_k_log2, int device_id,
-                              hipStream_t stream)
+                              hipStream_t stream, const char* tuning)
 {
     DecodeParams p{};
-    p.g       = g;
-    p.m_tiles = (g.M + 15) / 16;
-    const int n_blocks = (g.N + kRowsPerBlock - 1) / kRowsPerBlock;
+    p.g           = g;
+    p.bf16_out    = out_dtype == In16::bf16 ? 1 : 0;
+    p.n_tiles     = (g.N + 15) / 16;
+    p.xs_vec4     = ((g.kblocks & 3) == 0 && ((uintptr_t)g.xs & 15) == 0) ? 1 : 0;
+    const int mt        = (g.M + 15) / 16;
+    const int max_waves = 4;
+    const int steps     = (g.kblocks + kStepKb - 1) / kStepKb;
+    const int kChipCus  = 256;
 
-    int splits;
-    if(split_k_log2 >= 0)
-        splits = 1 << split_k_log2;
-    else
-    {
-        // Splitting K costs an fp32 round trip of the output tile through device-coherent
-        // stores and loads, which measured slower than it gains unless N alone leaves most of the
-        // chip idle: split only while fewer than ~100 workgroups exist.
-        splits = 1;
-        while(n_blocks * splits < 100 && splits * 2 <= g.kblocks)
-            splits *= 2;
-    }
-    if(splits > g.kblocks)
-        splits = g.kblocks;
-    int chunk_kb = (g.kblocks + splits - 1) / splits;
-    if(chunk_kb > kMaxChunkKb)
-    {
-        chunk_kb = kMaxChunkKb;
-    }
-    splits     = (g.kblocks + chunk_kb - 1) / chunk_kb;
-    p.chunk_kb = chunk_kb;
-    p.chunk_kb_pad = (chunk_kb + 7) / 8 * 8;
-    p.splits   = splits;
+    // Two row tiles per group halve the activation traffic and double what a wave keeps in
+    // flight: taken when the activations are wide (their re-reads then cost more than idle
+    // compute units) or when that still leaves a workgroup for nearly every compute unit.
+    int rows = tuning_value(tuning, "r");
+    if(rows != 1 && rows != 2)
+        rows = (mt >= 3 || p.n_tiles >= 2 * (kChipCus - kChipCus / 8)) ? 2 : 1;
+    p.n_groups = (p.n_tiles + rows - 1) / rows;
 
+    int splits = tuning_value(tuning, "s");
+    if(splits <= 0)
+    {
+        if(split_k_log2 >= 0)
+            splits = 1 << split_k_log2;
+        else
+        {
+            // Split K across workgroups only while every workgroup still gets a compute unit of
+            // its own (one workgroup fills a compute unit's registers) and at least two steps.
+            splits = kChipCus / p.n_groups;
+            if(splits > steps / 2)
+                splits = steps / 2;
+            if(splits < 1)
+                splits = 1;
+        }
+    }
+    if(splits > steps)
+        splits = steps;
+    int steps_per_split = (steps + splits - 1) / splits;
+    splits              = (steps + steps_per_split - 1) / steps_per_split;
+    p.kb_per_split      = steps_per_split * kStepKb;
+    p.splits            = splits;
+
+    int waves = tuning_value(tuning, "w");
+    if(waves <= 0 || waves > max_waves)
+        waves = steps_per_split < max_waves ? steps_per_split : max_waves;
+    const bool single = steps_per_split <= waves;
+    const bool full   = (g.kblocks % kStepKb) == 0;
+
+    int gx = tuning_value(tuning, "g");
+    if(gx <= 0)
+    {
+        gx = p.n_groups;
+        if(single && p.n_groups * splits > 2 * kChipCus)
+        {
+            const int per_split = (kChipCus + splits - 1) / splits;
+            const int iters     = (p.n_groups + per_split - 1) / per_split;
+            gx                  = (p.n_groups + iters - 1) / iters;
+        }
+    }
+    if(gx > p.n_groups)
+        gx = p.n_groups;
+
+    const size_t tile_set = (size_t)rows * mt * 64 * 16; // bytes of one group's fp32 tile set
     if(splits > 1)
     {
+        const size_t bytes = (size_t)splits * p.n_groups * tile_set;
+        if(bytes >= ((size_t)1 << 31))
+            return hipErrorInvalidValue;
         Workspace* w = nullptr;
-        size_t     partial_floats = (size_t)splits * n_blocks * kRowsPerBlock * p.m_tiles * 16;
-        hipError_t e = ensure_workspace(device_id, partial_floats, (size_t)n_blocks, stream, &w);
+        hipError_t e = ensure_workspace(device_id, bytes, (size_t)p.n_groups, stream, &w);
         if(e != hipSuccess)
             return e;
-        p.partial = w->partial;
-        p.tickets = w->tickets;
+        p.partial       = w->partial;
+        p.partial_bytes = (uint32_t)bytes;
+        p.tickets       = w->tickets;
     }
 
-    const size_t smem = (size_t)p.m_tiles * 16 * p.chunk_kb_pad * 128 + (size_t)p.m_tiles * 16 * chunk_kb * 4;
-    dim3         grid(n_blocks, splits);
-    const bool   bf = out_dtype == In16::bf16;
-#define FP8BS_LAUNCH_DECODE(MT, KB)                                                               \
-    {                                                                                             \
-        auto       kernel = bf ? gemm_decode_kernel<In16::bf16, MT, KB>                           \
-                               : gemm_decode_kernel<In16::fp16, MT, KB>;                          \
-        hipError_t e      = hipFuncSetAttribute((const void*)kernel,                              \
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
-        if(e != hipSuccess)                                                                       \
-            return e;                                                                             \
-        hipLaunchKernelGGL(kernel, grid, dim3(kThreads), smem, stream, p);                        \
-    }
-#define FP8BS_LAUNCH_DECODE_KB(MT)                     \
-    if(chunk_kb <= 4)                                  \
-        FP8BS_LAUNCH_DECODE(MT, 4)                     \
-    else if(chunk_kb <= 8)                             \
-        FP8BS_LAUNCH_DECODE(MT, 8)                     \
-    else if(chunk_kb <= 12)                            \
-        FP8BS_LAUNCH_DECODE(MT, 12)                    \
-    else                                               \
-        FP8BS_LAUNCH_DECODE(MT, 16)
-    switch(p.m_tiles)
+    // LDS: a 2 KiB transposition slot per wave, then as many parked tile sets as the workgroup
+    // has row groups to walk (bounded by the LDS budget; it flushes when they are full)
+    const int    iters = (p.n_groups + gx - 1) / gx;
+    const size_t slots = (size_t)waves * 2048;
+    int          park  = (int)((kMaxDynamicLds - slots) / ((size_t)waves * tile_set));
+    if(park > iters)
+        park = iters;
+    if(tuning_value(tuning, "p") > 0 && tuning_value(tuning, "p") < park)
+        park = tuning_value(tuning, "p");
+    p.park_slots      = park;
+    const size_t smem = slots + (size_t)park * waves * tile_set;
+    const dim3   grid(gx, splits);
+    switch(mt)
     {
-    case 1: FP8BS_LAUNCH_DECODE_KB(1) break;
-    case 2: FP8BS_LAUNCH_DECODE_KB(2) break;
-    case 3: FP8BS_LAUNCH_DECODE_KB(3) break;
-    default: FP8BS_LAUNCH_DECODE_KB(4) break;
+    case 1: return launch_mt<1>(p, rows, single, full, grid, waves, smem, stream);
+    case 2: return launch_mt<2>(p, rows, single, full, grid, waves, smem, stream);
+    case 3: return launch_mt<3>(p, rows, single, full, grid, waves, smem, stream);
+    default: return launch_mt<4>(p, rows, single, full, grid, waves, smem, stream);
     }
-#undef FP8BS_LAUNCH_DECODE_KB
-#undef FP8BS_LAUNCH_DECODE
-    return hipGetLastError();
 }
 
 } // namespace fp8bs
