@@ -135,10 +135,12 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                 s[r][i] = wsp[kslot(kb0, nk, i)];
         }
     };
-    auto issue_x = [&](int kb0, int nk, u32x4(&raw)[MT][kStepKb][2]) {
+    auto issue_x = [&](int kb0, int nk, u32x4(&raw)[MT][kStepKb][2], int j_lo, int j_hi) {
 #pragma unroll
         for(int j = 0; j < MT; ++j)
         {
+            if(j < j_lo || j >= j_hi) // compile-time bounds at every call site
+                continue;
 #pragma unroll
             for(int h = 0; h < 2; ++h)
 #pragma unroll
@@ -166,6 +168,36 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
 #pragma unroll
             for(int i = 0; i < kStepKb; ++i)
                 bx[j][i] = settle(raw[j][i]);
+    };
+    // first row group of a workgroup: weight fragments are ready, activation fragments are formed
+    // (and kept) one m tile at a time, each multiplied at once
+    auto multiply_first = [&](int nk, const i32x8(&aw)[R][kStepKb], const float(&s)[R][kStepKb],
+                              const u32x4(&xraw)[MT][kStepKb][2], int j_lo, int j_hi) {
+#pragma unroll
+        for(int j = 0; j < MT; ++j)
+        {
+            if(j < j_lo || j >= j_hi) // compile-time bounds at every call site
+                continue;
+#pragma unroll
+            for(int i = 0; i < kStepKb; ++i)
+                bx[j][i] = settle(xraw[j][i]);
+#pragma unroll
+            for(int i = 0; i < kStepKb; ++i)
+            {
+                if(FULL || i < nk) // wave-uniform
+                {
+#pragma unroll
+                    for(int r = 0; r < R; ++r)
+                    {
+                        const f32x4 part = mfma_16x16x128_fp8(aw[r][i], bx[j][i], f32x4{0.f, 0.f, 0.f, 0.f});
+                        const float sc   = xsv[j][i] * s[r][i];
+#pragma unroll
+                        for(int c = 0; c < 4; ++c)
+                            acc[r][j][c] = __builtin_fmaf(part[c], sc, acc[r][j][c]);
+                    }
+                }
+            }
+        }
     };
     // one weight unit at a time: fragments out of the raw registers, then its MT tile products,
     // scaled and accumulated
@@ -345,16 +377,28 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
             clear_acc();
             if(nk > 0)
             {
+                // Requests are throttled by the memory system, so the instruction stream does
+                // useful work between them: the weight fragments are formed while the second
+                // half of the activations is still being requested, and each m tile is
+                // multiplied as soon as its own fragments are in.
+                constexpr int kHalf = (MT + 1) / 2;
                 issue_w(grp, kb0, nk, raw_a, ws_a);
-                issue_x(kb0, nk, xraw);
-                settle_x(xraw); // the raw activation registers are free before the prefetch
-                if(more)
+                issue_x(kb0, nk, xraw, 0, kHalf);
+                i32x8 aw[R][kStepKb];
+#pragma unroll
+                for(int r = 0; r < R; ++r)
+#pragma unroll
+                    for(int i = 0; i < kStepKb; ++i)
+                        aw[r][i] = settle(raw_a[r][i]);
+                issue_x(kb0, nk, xraw, kHalf, MT);
+                multiply_first(nk, aw, ws_a, xraw, 0, kHalf);
+                if(more) // the next group's weights, now that half of the raw registers are free
                 {
                     issue_w(grp + stride, kb0, nk, raw_b, ws_b);
-                    multiply(nk, raw_a, ws_a);
+                    multiply_first(nk, aw, ws_a, xraw, kHalf, MT);
                 }
                 else
-                    multiply(nk, raw_a, ws_a);
+                    multiply_first(nk, aw, ws_a, xraw, kHalf, MT);
             }
             parked_one(!more);
             grp += stride;
@@ -406,7 +450,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                 u32x4     xraw[MT][kStepKb][2];
                 float     wsv[R][kStepKb];
                 issue_w(grp, kb0, nk, wraw, wsv);
-                issue_x(kb0, nk, xraw);
+                issue_x(kb0, nk, xraw, 0, MT);
                 settle_x(xraw);
                 multiply(nk, wraw, wsv);
             }
