@@ -177,6 +177,28 @@ def test_decode_stream_kernel(m, n, k, splitk):
     assert (out.view(torch.int16) != one.view(torch.int16)).float().mean().item() < 0.02
 
 
+@pytest.mark.parametrize("m,n,k,tuning", [
+    (3, 4096, 1024, "r=2,g=7,p=2"),        # 128 row groups over 7 workgroups, partial tiles flushed every 2
+    (20, 3000, 640, "r=1,g=5,p=3"),        # K not a multiple of 512, ragged N, two m tiles
+    (64, 2112, 7168, "r=2,s=2,g=4"),       # K split across workgroups, several steps per wave, 17 groups each
+    (40, 1536, 2048, "r=2,s=2,w=2,g=3"),   # two waves per workgroup
+    (1, 24576, 1536, "g=16"),              # 48 row groups per workgroup, weights prefetched group by group
+    (64, 512, 512, "w=1"),                 # one wave: nothing to add across waves
+    (33, 1000, 896, "r=2,s=7"),            # one step per K range, last range short
+])
+def test_decode_work_split_overrides(m, n, k, tuning):
+    # the work split is a launch-time choice; every split must give the same answer up to fp32
+    # regrouping, and the same bits from run to run
+    xq, wq, xs, ws = make_problem(m, n, k, seed=m * 7 + n + k, outliers=0.01)
+    name = "decode_stream:" + tuning
+    out = run_gpu(xq, wq, xs, ws, kernel=name, splitK=-1)
+    assert_close_to_f64(out, xq, wq, xs, ws, f"{name} {m}x{n}x{k}")
+    again = run_gpu(xq, wq, xs, ws, kernel=name, splitK=-1)
+    assert torch.equal(out.view(torch.int16), again.view(torch.int16))
+    auto = run_gpu(xq, wq, xs, ws, kernel="decode_stream", splitK=-1)
+    assert (out.view(torch.int16) != auto.view(torch.int16)).float().mean().item() < 0.02
+
+
 def test_decode_split_k_repeated_calls_leave_tickets_clean():
     # the split-K tickets must return to zero after every call, also when shapes change
     for (m, n, k) in [(16, 2112, 7168), (1, 2112, 7168), (64, 2112, 7168), (16, 7168, 2048), (16, 2112, 7168)]:
