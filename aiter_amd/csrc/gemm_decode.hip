@@ -36,7 +36,7 @@ struct DecodeParams
     int32_t   kb_per_split; // K blocks per workgroup-level K range
     int32_t   splits;       // number of such ranges (grid.y)
     int32_t   bf16_out;
-    int32_t   park_slots;   // row groups whose partial tiles fit in LDS between two flushes
+    int32_t   grid_x, waves; // launch dimensions, passed explicitly: the implicit ones cost a dependent load
     int32_t   xs_vec4;      // x_scale rows can be read four K blocks at a time (16-byte aligned)
     float*    partial;      // [splits][n_groups][R * MT * 64] x 4 fp32 when splits > 1
     uint32_t  partial_bytes;
@@ -63,9 +63,20 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const GemmKernelParams& g = p.g;
 
+    // Kernel arguments arrive through scalar loads, which the compiler places per basic block:
+    // three dependent round trips before the first weight request.  Naming every argument
+    // here puts all of them into the entry block, behind a single wait.
+#define FP8BS_TOUCH(x) asm volatile("" ::"s"(x))
+    FP8BS_TOUCH(g.xq); FP8BS_TOUCH(g.wq); FP8BS_TOUCH(g.xs); FP8BS_TOUCH(g.ws); FP8BS_TOUCH(g.out);
+    FP8BS_TOUCH(g.M); FP8BS_TOUCH(g.N); FP8BS_TOUCH(g.lda); FP8BS_TOUCH(g.ldb); FP8BS_TOUCH(g.kblocks);
+    FP8BS_TOUCH(p.n_tiles); FP8BS_TOUCH(p.n_groups); FP8BS_TOUCH(p.kb_per_split); FP8BS_TOUCH(p.splits);
+    FP8BS_TOUCH(p.bf16_out); FP8BS_TOUCH(p.xs_vec4); FP8BS_TOUCH(p.partial); FP8BS_TOUCH(p.partial_bytes);
+    FP8BS_TOUCH(p.tickets); FP8BS_TOUCH(p.grid_x); FP8BS_TOUCH(p.waves);
+#undef FP8BS_TOUCH
+
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int nw   = (int)blockDim.x >> 6;
+    const int nw   = p.waves;
     const int l16 = lane & 15, kg = lane >> 4;
     const int split = blockIdx.y;
     const int kb_lo = split * p.kb_per_split;
@@ -255,11 +266,11 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
         __builtin_amdgcn_make_buffer_rsrc(p.partial, 0, p.splits > 1 ? (int)p.partial_bytes : 0, 0x00020000);
     constexpr int kCoherent = 16; // cache-policy bit sc1: served by memory, not by a per-XCD L2
 
-    // Per-wave partial tiles are parked in LDS without any synchronisation while the workgroup
-    // streams through its row groups; every p.park_slots groups (and at the end) they are added
-    // up in wave order and stored.
+    // Per-wave partial tiles of a row group are parked in one of two LDS slots; they are added up
+    // in wave order and stored while the workgroup waits for the next group's weights, so only
+    // the last group's sum is left for the end.
     f32x4* const parked = (f32x4*)(smem + (size_t)nw * 2048);
-    auto park = [&](int q) {
+    auto         park   = [&](int q) {
         f32x4* mine = parked + ((size_t)q * nw + wave) * E;
 #pragma unroll
         for(int r = 0; r < R; ++r)
@@ -285,7 +296,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
         // The workgroups that share a row group run on different XCDs, whose L2 caches are not
         // coherent with each other; every access to the exchanged tiles therefore bypasses them
         // (sc1), and the stores are waited for before the ticket is taken.
-        for(int e = t; e < E; e += (int)blockDim.x)
+        for(int e = t; e < E; e += (nw * 64))
         {
             const f32x4    s   = wave_sum(red, e);
             const uint32_t off = (uint32_t)(((size_t)split * p.n_groups + grp) * E + e) * 16u;
@@ -300,7 +311,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
             return;
         if(t == 0) // leave the ticket ready for the next launch
             __hip_atomic_store(p.tickets + grp, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        for(int e = t; e < E; e += (int)blockDim.x)
+        for(int e = t; e < E; e += (nw * 64))
         {
             f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
             for(int sp = 0; sp < p.splits; ++sp) // split order, whoever arrived last
@@ -311,54 +322,44 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
             store_out(grp, e, s);
         }
     };
-    // groups first_grp, first_grp + gridDim.x, ... (count of them) are parked in slots 0..count-1
-    auto flush = [&](int first_grp, int count, bool last) {
+    // adds up and stores the group parked in `slot`; the barrier makes every wave's tiles visible
+    // (and, one group later, guarantees that the other slot has been read before it is reused)
+    auto flush_one = [&](int fgrp, int which) {
         __syncthreads();
+        const f32x4* red = parked + (size_t)which * nw * E;
         if(p.splits == 1)
         {
             // four elements per thread and pass, all LDS reads of a pass issued together
-            const int total = count * E, T = (int)blockDim.x;
-            for(int base = t; base < total; base += 4 * T)
+            const int T = (nw * 64);
+            for(int base = t; base < E; base += 4 * T)
             {
                 f32x4 sum[4];
 #pragma unroll
                 for(int u = 0; u < 4; ++u)
-                {
-                    const int idx = min(base + u * T, total - 1);
-                    const int q = idx / E, e = idx - q * E;
-                    sum[u] = wave_sum(parked + (size_t)q * nw * E, e);
-                }
+                    sum[u] = wave_sum(red, min(base + u * T, E - 1));
 #pragma unroll
                 for(int u = 0; u < 4; ++u)
-                {
-                    const int idx = base + u * T;
-                    if(idx < total)
-                    {
-                        const int q = idx / E, e = idx - q * E;
-                        store_out(first_grp + q * (int)gridDim.x, e, sum[u]);
-                    }
-                }
+                    if(base + u * T < E)
+                        store_out(fgrp, base + u * T, sum[u]);
             }
         }
         else
-        {
-            for(int q = 0; q < count; ++q)
-                flush_group_split(first_grp + q * (int)gridDim.x, parked + (size_t)q * nw * E);
-        }
-        if(!last)
-            __syncthreads(); // the slots are free again
+            flush_group_split(fgrp, red);
     };
 
-    const int stride = gridDim.x;
-    int       grp = blockIdx.x, q = 0, q_first = grp;
-    auto      parked_one = [&](bool last) {
-        park(q);
-        if(++q == p.park_slots || last)
+    const int stride = p.grid_x;
+    int       grp = blockIdx.x, prev = -1, pslot = 0;
+    // to be called between requesting the next group's weights and multiplying the current one
+    auto flush_prev = [&]() {
+        if(prev >= 0)
         {
-            flush(q_first, q, last);
-            q       = 0;
-            q_first = grp + stride;
+            flush_one(prev, pslot);
+            pslot ^= 1;
         }
+    };
+    auto park_current = [&]() {
+        park(pslot);
+        prev = grp;
     };
 
     if constexpr(SINGLE)
@@ -383,57 +384,81 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                 // multiplied as soon as its own fragments are in.
                 constexpr int kHalf = (MT + 1) / 2;
                 issue_w(grp, kb0, nk, raw_a, ws_a);
-                issue_x(kb0, nk, xraw, 0, kHalf);
-                i32x8 aw[R][kStepKb];
-#pragma unroll
-                for(int r = 0; r < R; ++r)
-#pragma unroll
-                    for(int i = 0; i < kStepKb; ++i)
-                        aw[r][i] = settle(raw_a[r][i]);
-                issue_x(kb0, nk, xraw, kHalf, MT);
-                multiply_first(nk, aw, ws_a, xraw, 0, kHalf);
-                if(more) // the next group's weights, now that half of the raw registers are free
+                if constexpr(MT <= 2)
                 {
-                    issue_w(grp + stride, kb0, nk, raw_b, ws_b);
-                    multiply_first(nk, aw, ws_a, xraw, kHalf, MT);
+                    // narrow activations leave registers to spare: the second group's weights
+                    // are requested at once, behind the first group's and the activations
+                    issue_x(kb0, nk, xraw, 0, MT);
+                    if(more)
+                    {
+                        issue_w(grp + stride, kb0, nk, raw_b, ws_b);
+                        settle_x(xraw);
+                        multiply(nk, raw_a, ws_a);
+                    }
+                    else
+                    {
+                        settle_x(xraw);
+                        multiply(nk, raw_a, ws_a);
+                    }
                 }
                 else
-                    multiply_first(nk, aw, ws_a, xraw, kHalf, MT);
+                {
+                    issue_x(kb0, nk, xraw, 0, kHalf);
+                    i32x8 aw[R][kStepKb];
+#pragma unroll
+                    for(int r = 0; r < R; ++r)
+#pragma unroll
+                        for(int i = 0; i < kStepKb; ++i)
+                            aw[r][i] = settle(raw_a[r][i]);
+                    issue_x(kb0, nk, xraw, kHalf, MT);
+                    multiply_first(nk, aw, ws_a, xraw, 0, kHalf);
+                    if(more) // the next group's weights, now that half of the raw registers are free
+                    {
+                        issue_w(grp + stride, kb0, nk, raw_b, ws_b);
+                        multiply_first(nk, aw, ws_a, xraw, kHalf, MT);
+                    }
+                    else
+                        multiply_first(nk, aw, ws_a, xraw, kHalf, MT);
+                }
             }
-            parked_one(!more);
+            park_current();
             grp += stride;
         }
         while(grp < p.n_groups) // raw_b holds this group
         {
             bool more = grp + stride < p.n_groups;
             clear_acc();
-            if(nk > 0)
+            if(nk > 0 && more)
             {
-                if(more)
-                {
-                    issue_w(grp + stride, kb0, nk, raw_a, ws_a);
-                    multiply(nk, raw_b, ws_b);
-                }
-                else
+                issue_w(grp + stride, kb0, nk, raw_a, ws_a);
+                flush_prev();
+                multiply(nk, raw_b, ws_b);
+            }
+            else
+            {
+                flush_prev();
+                if(nk > 0)
                     multiply(nk, raw_b, ws_b);
             }
-            parked_one(!more);
+            park_current();
             grp += stride;
             if(grp >= p.n_groups)
                 break;
             more = grp + stride < p.n_groups; // raw_a holds this group
             clear_acc();
-            if(nk > 0)
+            if(nk > 0 && more)
             {
-                if(more)
-                {
-                    issue_w(grp + stride, kb0, nk, raw_b, ws_b);
-                    multiply(nk, raw_a, ws_a);
-                }
-                else
+                issue_w(grp + stride, kb0, nk, raw_b, ws_b);
+                flush_prev();
+                multiply(nk, raw_a, ws_a);
+            }
+            else
+            {
+                flush_prev();
+                if(nk > 0)
                     multiply(nk, raw_a, ws_a);
             }
-            parked_one(!more);
+            park_current();
             grp += stride;
         }
     }
@@ -443,6 +468,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
         for(; grp < p.n_groups; grp += stride)
         {
             clear_acc();
+            bool flushed = false;
             for(int kb0 = kb_lo + wave * kStepKb; kb0 < kb_hi; kb0 += nw * kStepKb)
             {
                 const int nk = min(kStepKb, kb_hi - kb0);
@@ -451,12 +477,20 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                 float     wsv[R][kStepKb];
                 issue_w(grp, kb0, nk, wraw, wsv);
                 issue_x(kb0, nk, xraw, 0, MT);
+                if(!flushed) // the previous group's sum, behind this group's first requests
+                {
+                    flush_prev();
+                    flushed = true;
+                }
                 settle_x(xraw);
                 multiply(nk, wraw, wsv);
             }
-            parked_one(grp + stride >= p.n_groups);
+            if(!flushed)
+                flush_prev();
+            park_current();
         }
     }
+    flush_prev();
 }
 
 // workspace for split-K partials and tickets, one per device, grown on demand and kept for the
@@ -648,17 +682,10 @@ hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int spl
         p.tickets       = w->tickets;
     }
 
-    // LDS: a 2 KiB transposition slot per wave, then as many parked tile sets as the workgroup
-    // has row groups to walk (bounded by the LDS budget; it flushes when they are full)
-    const int    iters = (p.n_groups + gx - 1) / gx;
-    const size_t slots = (size_t)waves * 2048;
-    int          park  = (int)((kMaxDynamicLds - slots) / ((size_t)waves * tile_set));
-    if(park > iters)
-        park = iters;
-    if(tuning_value(tuning, "p") > 0 && tuning_value(tuning, "p") < park)
-        park = tuning_value(tuning, "p");
-    p.park_slots      = park;
-    const size_t smem = slots + (size_t)park * waves * tile_set;
+    // LDS: a 2 KiB transposition slot per wave, then two slots of parked tile sets
+    const size_t smem = (size_t)waves * (2048 + 2 * tile_set);
+    p.grid_x          = gx;
+    p.waves           = waves;
     const dim3   grid(gx, splits);
     switch(mt)
     {

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the FP8 block-scale path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload quant|prefill|decode|fused]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload quant|prefill|decode|decode9|fused]
                     [--no-also] [--no-cpu]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
@@ -11,7 +11,9 @@ path are timed briefly as well and reported under ``also`` in the same JSON line
 Workloads (BASELINE.json configs):
   quant    config 2  x bf16 [16384,7168] (1 % channels x50) -> fp8 + fp32 scales, HBM-bound
   prefill  config 4  blockscale GEMM M=8192 N=36864 K=7168, MFMA-bound
-  decode   config 3  blockscale GEMM M in {1,16,64} x {(7168,2048),(24576,1536),(2112,7168)}
+  decode   config 3  blockscale GEMM M=64 N=24576 K=1536 (the largest decode shape)
+  decode9  config 3  all nine: M in {1,16,64} x (N,K) in {(7168,2048),(24576,1536),(2112,7168)};
+                     weights rotate through 640 MB so that every call reads them from HBM
   fused    config 5  RMSNorm + 1x128 quant on [2048,7168], then GEMM N=4096
 
 Timing uses HIP events recorded on the stream the kernels are launched on (torch's current
@@ -43,7 +45,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="quant", choices=["quant", "prefill", "decode", "fused", "copy"],
+    ap.add_argument("--workload", default="quant", choices=["quant", "prefill", "decode", "decode9", "fused", "copy"],
                     help="'copy' is a plain 1 GiB device copy used to calibrate the rocprofv3 FETCH_SIZE / "
                     "WRITE_SIZE counters; it is not part of the path")
     ap.add_argument("--no-also", action="store_true", help="time only the primary workload")
@@ -352,6 +354,46 @@ class CopyCalibration:
         return None
 
 
+class DecodeAllWorkload:
+    """All nine decode shapes of config 3, one launch each per step (shape after shape, so a kernel
+    trace of the run lists them in DECODE_SHAPES order)."""
+
+    name = "decode9"
+
+    def setup(self, torch, dev):
+        self.parts = [GemmWorkload("decode", m, n, k, "decode") for (m, n, k) in DECODE_SHAPES]
+        for w in self.parts:
+            w.setup(torch, dev)
+
+    def step(self):
+        for w in self.parts:
+            w.step()
+
+    def bytes(self):
+        return sum(gemm_bytes(w.M, w.N, w.K) for w in self.parts)
+
+    def describe(self):
+        return {"workload": "config 3: the nine decode blockscale GEMM shapes, one launch each per step",
+                "shapes": [list(sh) for sh in DECODE_SHAPES], "kernel": "gemm_a8w8_blockscale (decode_stream)"}
+
+    def result(self, sec):
+        gbs = self.bytes() / sec / 1e9
+        return gbs, "GB/s", {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": gbs / HBM_PEAK_GBS, "traffic": None}
+
+    def per_shape(self, torch, steps, warmup):
+        out = []
+        for w in self.parts:
+            s3 = time_launches(torch, w.step, steps, warmup)
+            gbs = gemm_bytes(w.M, w.N, w.K) / s3 / 1e9
+            out.append({"M": w.M, "N": w.N, "K": w.K, "kernel_us": s3 * 1e6, "GB/s": gbs,
+                        "frac_of_hbm_peak": gbs / HBM_PEAK_GBS})
+        return out
+
+    def cpu_baseline(self, torch):
+        return self.parts[-1].cpu_baseline(torch)
+
+
 def make_workload(name):
     if name == "copy":
         return CopyCalibration()
@@ -366,6 +408,8 @@ def make_workload(name):
                             "config 3: decode blockscale GEMM M=64 N=24576 K=1536 (largest of the nine decode shapes)")
     if name == "fused":
         return FusedWorkload()
+    if name == "decode9":
+        return DecodeAllWorkload()
     raise ValueError(name)
 
 
@@ -410,6 +454,10 @@ def main():
     }
     if args.workload == "prefill":
         line["vs_reference_tuned_csv"] = value / REF_PREFILL_TFLOPS
+    if args.workload == "decode9":
+        # shape after shape: steps + warmup launches each, in DECODE_SHAPES order
+        line["per_shape"] = wl.per_shape(torch, args.steps, args.warmup)
+        args.no_also = True
 
     if not args.no_cpu and args.workload != "copy":
         torch.set_num_threads(os.cpu_count() or 1)
