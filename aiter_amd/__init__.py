@@ -10,7 +10,14 @@ Everything computes in ``libaiter_fp8bs.so`` (hand-written HIP for gfx950, C ABI
 
 from . import dtypes
 from .enums import QuantType
-from .gemm_op_a8w8 import gemm_a8w8_blockscale, gemm_a8w8_blockscale_ck, gemm_kernel_names
+from .gemm_op_a8w8 import (
+    gemm_a8w8_blockscale,
+    gemm_a8w8_blockscale_bpreshuffle,
+    gemm_a8w8_blockscale_bpreshuffle_ck,
+    gemm_a8w8_blockscale_ck,
+    gemm_kernel_names,
+)
+from .shuffle import shuffle_weight
 from .quant import dynamic_per_token_scaled_quant, get_hip_quant, per_group_quant_hip
 from .rmsnorm import (
     add_rmsnorm,
@@ -25,6 +32,9 @@ __all__ = [
     "dtypes",
     "QuantType",
     "get_hip_quant",
+    "shuffle_weight",
+    "gemm_a8w8_blockscale_bpreshuffle",
+    "gemm_a8w8_blockscale_bpreshuffle_ck",
     "per_group_quant_hip",
     "dynamic_per_token_scaled_quant",
     "gemm_a8w8_blockscale",

@@ -34,6 +34,7 @@ _SIGNATURES = {
         _TP, _TP, _TP, _TP, _TP, _TP, ctypes.c_float, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
     ],
     "gemm_a8w8_blockscale": [_TP, _TP, _TP, _TP, _TP, ctypes.c_int64, ctypes.c_char_p],
+    "gemm_a8w8_blockscale_bpreshuffle": [_TP, _TP, _TP, _TP, _TP, ctypes.c_char_p],
 }
 EXPORTED_SYMBOLS = sorted(
     list(_SIGNATURES)

@@ -318,6 +318,105 @@ void rmsnorm_common(const char* fn, aiter_tensor_t* out, aiter_tensor_t* input,
 
 } // namespace
 
+static int gemm_blockscale_common(const char* fn, bool preshuffled, aiter_tensor_t* XQ, aiter_tensor_t* WQ,
+                                  aiter_tensor_t* x_scale, aiter_tensor_t* w_scale, aiter_tensor_t* Out,
+                                  int64_t splitK, const char* kernelName, aiter_stream_t stream)
+{
+    return guarded([&] {
+        check_tensor(fn, XQ, "XQ");
+        check_tensor(fn, WQ, "WQ");
+        check_tensor(fn, x_scale, "x_scale");
+        check_tensor(fn, w_scale, "w_scale");
+        check_tensor(fn, Out, "Out");
+        same_device(fn, {XQ, WQ, x_scale, w_scale, Out});
+        // csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale.cu:90-97
+        if(!is_fp8_like(XQ->dtype_) || !is_fp8_like(WQ->dtype_))
+            fail(fn, "XQ and WQ must be fp8, got ", dtype_name(XQ->dtype_), " and ",
+                 dtype_name(WQ->dtype_));
+        if(XQ->dtype_ != WQ->dtype_)
+            fail(fn, "Weights and activations should have the same dtype!");
+        if(x_scale->dtype_ != w_scale->dtype_)
+            fail(fn, "Scales should have the same dtype!");
+        if(x_scale->dtype_ != AITER_DTYPE_fp32)
+            fail(fn, "scales must be fp32, got ", dtype_name(x_scale->dtype_));
+        if(!is_f16_like(Out->dtype_))
+            fail(fn, "Out must be bf16 or fp16, got ", dtype_name(Out->dtype_));
+        if(XQ->ndim != 2 || WQ->ndim != 2 || Out->ndim != 2)
+            fail(fn, "XQ, WQ and Out must be 2-D");
+        const int64_t M = XQ->shape[0], K = XQ->shape[1], N = WQ->shape[0];
+        if(WQ->shape[1] != K)
+            fail(fn, "XQ is [", M, ",", K, "] but WQ is [", N, ",", WQ->shape[1], "]");
+        if(K % 128 != 0)
+            fail(fn, "K = ", K, " must be a multiple of the 128-wide scale block");
+        if(Out->shape[0] != M || Out->shape[1] != N || !contiguous(Out))
+            fail(fn, "Out must be a contiguous [", M, ",", N, "] tensor");
+        const int64_t kb = K / 128, nb = (N + 127) / 128;
+        if(!preshuffled)
+        {
+            if((int64_t)x_scale->numel_ != M * kb || !contiguous(x_scale))
+                fail(fn, "x_scale must be contiguous [", M, ",", kb, "], got ", x_scale->numel_,
+                     " elements");
+        }
+        else
+        {
+            // The pre-shuffled kernels read x_scale as [K/128][M] (column-major); callers pass
+            // either that buffer viewed as a contiguous [M, K/128] tensor or an [M, K/128] view
+            // with strides (1, M) (op_tests/test_gemm_a8w8_blockscale.py:112-125).  Both put
+            // element (m, kb) at kb * M + m.
+            const bool as_view = x_scale->ndim == 2 && x_scale->shape[0] == M && x_scale->shape[1] == kb &&
+                                 (M <= 1 || x_scale->strides[0] == 1) && (kb <= 1 || x_scale->strides[1] == M);
+            if((int64_t)x_scale->numel_ != M * kb || !(contiguous(x_scale) || as_view))
+                fail(fn, "x_scale must hold M*K/128 = ", M * kb,
+                     " column-major values (contiguous buffer, or [M,K/128] view with strides (1,M))");
+            if(N % 16 != 0)
+                fail(fn, "pre-shuffled weights need N % 16 == 0, got N = ", N);
+            if(N > 1 && WQ->strides[0] != K)
+                fail(fn, "pre-shuffled weights must be a contiguous [N, K] buffer");
+        }
+        if((int64_t)w_scale->numel_ != nb * kb || !contiguous(w_scale))
+            fail(fn, "w_scale must be contiguous [", nb, ",", kb, "], got ", w_scale->numel_,
+                 " elements");
+        if((K > 1 && XQ->strides[1] != 1) || (K > 1 && WQ->strides[1] != 1))
+            fail(fn, "XQ and WQ must be contiguous in K");
+        const int64_t lda = M > 1 ? XQ->strides[0] : K, ldb = N > 1 ? WQ->strides[0] : K;
+        if(lda < K || ldb < K || lda % 16 != 0 || ldb % 16 != 0)
+            fail(fn, "row strides of XQ/WQ must be >= K and multiples of 16 bytes");
+        check_aligned(fn, XQ, "XQ", 16);
+        check_aligned(fn, WQ, "WQ", 16);
+        check_aligned(fn, Out, "Out", 8);
+        check_aligned(fn, x_scale, "x_scale", 4);
+        check_aligned(fn, w_scale, "w_scale", 4);
+        if(M > 0x7fffffffLL / 2 || N > 0x7fffffffLL / 2 || K > 0x7fffffffLL / 2)
+            fail(fn, "problem too large");
+        if(splitK < -1 || splitK > 4)
+            fail(fn, "splitK = ", splitK, " outside -1..4");
+        if(M == 0 || N == 0)
+            return;
+
+        fp8bs::GemmArgs a{};
+        a.xq           = (const uint8_t*)XQ->ptr;
+        a.wq           = (const uint8_t*)WQ->ptr;
+        a.xs           = (const float*)x_scale->ptr;
+        a.ws           = (const float*)w_scale->ptr;
+        a.out          = Out->ptr;
+        a.M            = M;
+        a.N            = N;
+        a.K            = K;
+        a.lda          = lda;
+        a.ldb          = ldb;
+        a.out_dtype    = in16_of(Out->dtype_);
+        a.split_k_log2 = (int)splitK;
+        a.kernel_name  = kernelName;
+        a.device_id    = XQ->device_id;
+        a.w_shuffled   = preshuffled;
+        a.xs_col_major = preshuffled;
+        DeviceGuard guard(XQ->device_id);
+        const char* why = nullptr;
+        hipError_t  e   = fp8bs::launch_gemm_blockscale(a, (hipStream_t)stream, &why);
+        check_hip(fn, e, why);
+    });
+}
+
 extern "C" {
 
 int aiter_ctypes_abi_version(void) { return 2; }
@@ -448,79 +547,16 @@ int gemm_a8w8_blockscale(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t*
                          aiter_tensor_t* w_scale, aiter_tensor_t* Out, int64_t splitK,
                          const char* kernelName, aiter_stream_t stream)
 {
-    return guarded([&] {
-        const char* fn = "gemm_a8w8_blockscale";
-        check_tensor(fn, XQ, "XQ");
-        check_tensor(fn, WQ, "WQ");
-        check_tensor(fn, x_scale, "x_scale");
-        check_tensor(fn, w_scale, "w_scale");
-        check_tensor(fn, Out, "Out");
-        same_device(fn, {XQ, WQ, x_scale, w_scale, Out});
-        // csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale.cu:90-97
-        if(!is_fp8_like(XQ->dtype_) || !is_fp8_like(WQ->dtype_))
-            fail(fn, "XQ and WQ must be fp8, got ", dtype_name(XQ->dtype_), " and ",
-                 dtype_name(WQ->dtype_));
-        if(XQ->dtype_ != WQ->dtype_)
-            fail(fn, "Weights and activations should have the same dtype!");
-        if(x_scale->dtype_ != w_scale->dtype_)
-            fail(fn, "Scales should have the same dtype!");
-        if(x_scale->dtype_ != AITER_DTYPE_fp32)
-            fail(fn, "scales must be fp32, got ", dtype_name(x_scale->dtype_));
-        if(!is_f16_like(Out->dtype_))
-            fail(fn, "Out must be bf16 or fp16, got ", dtype_name(Out->dtype_));
-        if(XQ->ndim != 2 || WQ->ndim != 2 || Out->ndim != 2)
-            fail(fn, "XQ, WQ and Out must be 2-D");
-        const int64_t M = XQ->shape[0], K = XQ->shape[1], N = WQ->shape[0];
-        if(WQ->shape[1] != K)
-            fail(fn, "XQ is [", M, ",", K, "] but WQ is [", N, ",", WQ->shape[1], "]");
-        if(K % 128 != 0)
-            fail(fn, "K = ", K, " must be a multiple of the 128-wide scale block");
-        if(Out->shape[0] != M || Out->shape[1] != N || !contiguous(Out))
-            fail(fn, "Out must be a contiguous [", M, ",", N, "] tensor");
-        const int64_t kb = K / 128, nb = (N + 127) / 128;
-        if((int64_t)x_scale->numel_ != M * kb || !contiguous(x_scale))
-            fail(fn, "x_scale must be contiguous [", M, ",", kb, "], got ", x_scale->numel_,
-                 " elements");
-        if((int64_t)w_scale->numel_ != nb * kb || !contiguous(w_scale))
-            fail(fn, "w_scale must be contiguous [", nb, ",", kb, "], got ", w_scale->numel_,
-                 " elements");
-        if((K > 1 && XQ->strides[1] != 1) || (K > 1 && WQ->strides[1] != 1))
-            fail(fn, "XQ and WQ must be contiguous in K");
-        const int64_t lda = M > 1 ? XQ->strides[0] : K, ldb = N > 1 ? WQ->strides[0] : K;
-        if(lda < K || ldb < K || lda % 16 != 0 || ldb % 16 != 0)
-            fail(fn, "row strides of XQ/WQ must be >= K and multiples of 16 bytes");
-        check_aligned(fn, XQ, "XQ", 16);
-        check_aligned(fn, WQ, "WQ", 16);
-        check_aligned(fn, Out, "Out", 8);
-        check_aligned(fn, x_scale, "x_scale", 4);
-        check_aligned(fn, w_scale, "w_scale", 4);
-        if(M > 0x7fffffffLL / 2 || N > 0x7fffffffLL / 2 || K > 0x7fffffffLL / 2)
-            fail(fn, "problem too large");
-        if(splitK < -1 || splitK > 4)
-            fail(fn, "splitK = ", splitK, " outside -1..4");
-        if(M == 0 || N == 0)
-            return;
+    return gemm_blockscale_common("gemm_a8w8_blockscale", false, XQ, WQ, x_scale, w_scale, Out, splitK,
+                                  kernelName, stream);
+}
 
-        fp8bs::GemmArgs a{};
-        a.xq           = (const uint8_t*)XQ->ptr;
-        a.wq           = (const uint8_t*)WQ->ptr;
-        a.xs           = (const float*)x_scale->ptr;
-        a.ws           = (const float*)w_scale->ptr;
-        a.out          = Out->ptr;
-        a.M            = M;
-        a.N            = N;
-        a.K            = K;
-        a.lda          = lda;
-        a.ldb          = ldb;
-        a.out_dtype    = in16_of(Out->dtype_);
-        a.split_k_log2 = (int)splitK;
-        a.kernel_name  = kernelName;
-        a.device_id    = XQ->device_id;
-        DeviceGuard guard(XQ->device_id);
-        const char* why = nullptr;
-        hipError_t  e   = fp8bs::launch_gemm_blockscale(a, (hipStream_t)stream, &why);
-        check_hip(fn, e, why);
-    });
+int gemm_a8w8_blockscale_bpreshuffle(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t* x_scale,
+                                     aiter_tensor_t* w_scale, aiter_tensor_t* Out, const char* kernelName,
+                                     aiter_stream_t stream)
+{
+    return gemm_blockscale_common("gemm_a8w8_blockscale_bpreshuffle", true, XQ, WQ, x_scale, w_scale, Out,
+                                  -1, kernelName, stream);
 }
 
 } // extern "C"

@@ -71,7 +71,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_kernel(GemmK
             int row = q >> 3, c = q & 7;
             int n   = n0 + row;
             n       = n < p.N ? n : p.N - 1;
-            u32x4 d = *(const u32x4*)(p.wq + (size_t)n * p.ldb + (size_t)kb * 128 + c * 16);
+            u32x4 d = *(const u32x4*)w_chunk_ptr(p, n, kb, c);
             *(u32x4*)(sW + lds_off(row, c)) = d;
         }
         for(int q = t; q < BM * 8; q += T)
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_tile_kernel(GemmK
         float sc[MT];
 #pragma unroll
         for(int j = 0; j < MT; ++j)
-            sc[j] = p.xs[(size_t)mrow[j] * p.kblocks + kb];
+            sc[j] = p.xs[(size_t)mrow[j] * p.xs_m + (size_t)kb * p.xs_k];
 
 #pragma unroll
         for(int i = 0; i < NT; ++i)
@@ -189,7 +189,7 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
         const char* tuning = name[13] == ':' ? name + 14 : nullptr;
         if(!gemm_decode_supports(p))
         {
-            *why = "decode_stream handles 1 <= M <= 64";
+            *why = "decode_stream handles 1 <= M <= 64 (this layout of weights / x_scale included?)";
             return hipErrorInvalidValue;
         }
         return launch_gemm_decode(p, DT, a.split_k_log2, a.device_id, stream, tuning);
@@ -229,6 +229,9 @@ hipError_t launch_gemm_blockscale(const GemmArgs& a, hipStream_t stream, const c
     p.lda     = a.lda;
     p.ldb     = a.ldb;
     p.kblocks = (int32_t)(a.K / 128);
+    p.xs_m       = a.xs_col_major ? 1 : a.K / 128;
+    p.xs_k       = a.xs_col_major ? a.M : 1;
+    p.w_shuffled = a.w_shuffled ? 1 : 0;
     return a.out_dtype == In16::bf16 ? dispatch<In16::bf16>(a, p, stream, why)
                                      : dispatch<In16::fp16>(a, p, stream, why);
 }

@@ -45,7 +45,22 @@ struct GemmKernelParams
     int32_t        M, N, K;
     int64_t        lda, ldb;
     int32_t        kblocks; // K / 128
+    // x_scale element (m, kb) lives at xs[m * xs_m + kb * xs_k]: (K/128, 1) for the row-major
+    // layout of gemm_a8w8_blockscale, (1, M) for the column-major one of the pre-shuffled entry
+    int64_t        xs_m, xs_k;
+    // weights pre-shuffled with layout (16,16) (aiter/ops/shuffle.py:192-205): per 16-row tile
+    // and 32-byte K chunk, the 16 rows' first 16 bytes, then the 16 rows' second 16 bytes
+    int32_t        w_shuffled;
 };
+
+// address of the 16-byte chunk c (0..7) of K block kb of weight row n, in either layout
+__device__ __forceinline__ const uint8_t* w_chunk_ptr(const GemmKernelParams& p, int n, int kb, int c)
+{
+    if(p.w_shuffled)
+        return p.wq + (size_t)(n >> 4) * 16 * (size_t)p.K + (size_t)(kb * 4 + (c >> 1)) * 512 +
+               (size_t)(c & 1) * 256 + (size_t)(n & 15) * 16;
+    return p.wq + (size_t)n * p.ldb + (size_t)kb * 128 + (size_t)c * 16;
+}
 
 // LDS tile: rows of 128 bytes (one K block); the 16-byte chunk c of row r lives at chunk
 // c ^ (r & 7) so that the 16 rows a quarter-wave reads with one ds_read_b128 spread over banks.

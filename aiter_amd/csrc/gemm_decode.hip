@@ -57,7 +57,9 @@ constexpr int decode_max_waves()
 
 // FULL: every step of every wave holds exactly 4 K blocks (K is a multiple of 512), which
 // makes the multiply straight-line code; otherwise the block count of a step is a run-time value.
-template <int MT, int R, bool SINGLE, bool FULL>
+// SHUF: the weights are pre-shuffled (16,16): a lane's MFMA fragment is then two coalesced 16-byte
+// loads and needs no transposition.
+template <int MT, int R, bool SINGLE, bool FULL, bool SHUF>
 __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kernel(DecodeParams p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -69,6 +71,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
 #define FP8BS_TOUCH(x) asm volatile("" ::"s"(x))
     FP8BS_TOUCH(g.xq); FP8BS_TOUCH(g.wq); FP8BS_TOUCH(g.xs); FP8BS_TOUCH(g.ws); FP8BS_TOUCH(g.out);
     FP8BS_TOUCH(g.M); FP8BS_TOUCH(g.N); FP8BS_TOUCH(g.lda); FP8BS_TOUCH(g.ldb); FP8BS_TOUCH(g.kblocks);
+    FP8BS_TOUCH(g.K); FP8BS_TOUCH(g.xs_m); FP8BS_TOUCH(g.xs_k);
     FP8BS_TOUCH(p.n_tiles); FP8BS_TOUCH(p.n_groups); FP8BS_TOUCH(p.kb_per_split); FP8BS_TOUCH(p.splits);
     FP8BS_TOUCH(p.bf16_out); FP8BS_TOUCH(p.xs_vec4); FP8BS_TOUCH(p.partial); FP8BS_TOUCH(p.partial_bytes);
     FP8BS_TOUCH(p.tickets); FP8BS_TOUCH(p.grid_x); FP8BS_TOUCH(p.waves);
@@ -92,6 +95,10 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
     // side, by which 16-byte chunk of its row a lane fetches.
     const int crow = lane >> 3, cchunk = (lane & 7) ^ crow;
     uint8_t*  slot = smem + (size_t)wave * 2048;
+    auto      as_fragment = [&](const u32x4(&raw)[2]) -> i32x8 {
+        return i32x8{(int)raw[0][0], (int)raw[0][1], (int)raw[0][2], (int)raw[0][3],
+                     (int)raw[1][0], (int)raw[1][1], (int)raw[1][2], (int)raw[1][3]};
+    };
     auto      settle = [&](const u32x4(&raw)[2]) -> i32x8 {
         *(u32x4*)(slot + lane * 16)        = raw[0];
         *(u32x4*)(slot + 1024 + lane * 16) = raw[1];
@@ -110,7 +117,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
 #pragma unroll
         for(int h = 0; h < 2; ++h)
             xrow[j][h] = g.xq + (size_t)min(j * 16 + h * 8 + crow, g.M - 1) * g.lda + cchunk * 16;
-        xsrow[j] = g.xs + (size_t)min(j * 16 + l16, g.M - 1) * g.kblocks;
+        xsrow[j] = g.xs + (size_t)min(j * 16 + l16, g.M - 1) * g.xs_m;
     }
 
     i32x8 bx[MT][kStepKb];
@@ -131,15 +138,29 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
         {
             const int    tile = min(grp * R + r, p.n_tiles - 1);
             const float* wsp  = g.ws + (size_t)((tile * 16) >> 7) * g.kblocks; // wave-uniform
-#pragma unroll
-            for(int h = 0; h < 2; ++h)
+            if constexpr(SHUF)
             {
-                const int      n  = min(tile * 16 + h * 8 + crow, g.N - 1);
-                const uint8_t* wp = g.wq + (size_t)n * g.ldb + cchunk * 16;
+                // lane (l16, kg) of K block kk: 16 bytes at chunk (4 kk + kg), row l16, both halves
+                const uint8_t* wp = g.wq + (size_t)tile * 16 * (size_t)g.K + (size_t)kg * 512 + l16 * 16;
 #pragma unroll
                 for(int i = 0; i < kStepKb; ++i)
-                    raw[r][i][h] =
-                        __builtin_nontemporal_load((const u32x4*)(wp + (size_t)kslot(kb0, nk, i) * 128));
+#pragma unroll
+                    for(int h = 0; h < 2; ++h)
+                        raw[r][i][h] = __builtin_nontemporal_load(
+                            (const u32x4*)(wp + (size_t)kslot(kb0, nk, i) * 2048 + h * 256));
+            }
+            else
+            {
+#pragma unroll
+                for(int h = 0; h < 2; ++h)
+                {
+                    const int      n  = min(tile * 16 + h * 8 + crow, g.N - 1);
+                    const uint8_t* wp = g.wq + (size_t)n * g.ldb + cchunk * 16;
+#pragma unroll
+                    for(int i = 0; i < kStepKb; ++i)
+                        raw[r][i][h] = __builtin_nontemporal_load(
+                            (const u32x4*)(wp + (size_t)kslot(kb0, nk, i) * 128));
+                }
             }
 #pragma unroll
             for(int i = 0; i < kStepKb; ++i)
@@ -168,7 +189,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
             {
 #pragma unroll
                 for(int i = 0; i < kStepKb; ++i)
-                    xsv[j][i] = xsrow[j][kslot(kb0, nk, i)];
+                    xsv[j][i] = xsrow[j][(size_t)kslot(kb0, nk, i) * g.xs_k];
             }
         }
     };
@@ -220,7 +241,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
             {
                 if(FULL || i < nk) // wave-uniform
                 {
-                    const i32x8 w = settle(wraw[r][i]);
+                    const i32x8 w = SHUF ? as_fragment(wraw[r][i]) : settle(wraw[r][i]);
 #pragma unroll
                     for(int j = 0; j < MT; ++j)
                     {
@@ -409,7 +430,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                     for(int r = 0; r < R; ++r)
 #pragma unroll
                         for(int i = 0; i < kStepKb; ++i)
-                            aw[r][i] = settle(raw_a[r][i]);
+                            aw[r][i] = SHUF ? as_fragment(raw_a[r][i]) : settle(raw_a[r][i]);
                     issue_x(kb0, nk, xraw, kHalf, MT);
                     multiply_first(nk, aw, ws_a, xraw, 0, kHalf);
                     if(more) // the next group's weights, now that half of the raw registers are free
@@ -559,10 +580,10 @@ int tuning_value(const char* tuning, const char* key)
     return 0;
 }
 
-template <int MT, int R, bool SINGLE, bool FULL>
+template <int MT, int R, bool SINGLE, bool FULL, bool SHUF>
 hipError_t launch_one(const DecodeParams& p, dim3 grid, int waves, size_t smem, hipStream_t stream)
 {
-    auto        kernel = gemm_decode_kernel<MT, R, SINGLE, FULL>;
+    auto        kernel = gemm_decode_kernel<MT, R, SINGLE, FULL, SHUF>;
     static bool raised[kMaxDevices]; // dynamic LDS above the default limit needs opting in, once
     int         dev = 0;
     (void)hipGetDevice(&dev);
@@ -578,28 +599,34 @@ hipError_t launch_one(const DecodeParams& p, dim3 grid, int waves, size_t smem, 
     return hipGetLastError();
 }
 
-template <int MT, int R>
+template <int MT, int R, bool SHUF>
 hipError_t launch_mt_r(const DecodeParams& p, bool single, bool full, dim3 grid, int waves, size_t smem,
                        hipStream_t stream)
 {
     if(single)
-        return full ? launch_one<MT, R, true, true>(p, grid, waves, smem, stream)
-                    : launch_one<MT, R, true, false>(p, grid, waves, smem, stream);
-    return full ? launch_one<MT, R, false, true>(p, grid, waves, smem, stream)
-                : launch_one<MT, R, false, false>(p, grid, waves, smem, stream);
+        return full ? launch_one<MT, R, true, true, SHUF>(p, grid, waves, smem, stream)
+                    : launch_one<MT, R, true, false, SHUF>(p, grid, waves, smem, stream);
+    return full ? launch_one<MT, R, false, true, SHUF>(p, grid, waves, smem, stream)
+                : launch_one<MT, R, false, false, SHUF>(p, grid, waves, smem, stream);
 }
 
 template <int MT>
 hipError_t launch_mt(const DecodeParams& p, int rows, bool single, bool full, dim3 grid, int waves,
                      size_t smem, hipStream_t stream)
 {
-    return rows == 2 ? launch_mt_r<MT, 2>(p, single, full, grid, waves, smem, stream)
-                     : launch_mt_r<MT, 1>(p, single, full, grid, waves, smem, stream);
+    if(p.g.w_shuffled)
+        return rows == 2 ? launch_mt_r<MT, 2, true>(p, single, full, grid, waves, smem, stream)
+                         : launch_mt_r<MT, 1, true>(p, single, full, grid, waves, smem, stream);
+    return rows == 2 ? launch_mt_r<MT, 2, false>(p, single, full, grid, waves, smem, stream)
+                     : launch_mt_r<MT, 1, false>(p, single, full, grid, waves, smem, stream);
 }
 
 } // namespace
 
-bool gemm_decode_supports(const GemmKernelParams& p) { return p.M >= 1 && p.M <= 64 && p.kblocks >= 1; }
+bool gemm_decode_supports(const GemmKernelParams& p)
+{
+    return p.M >= 1 && p.M <= 64 && p.kblocks >= 1;
+}
 
 // split_k_log2 < 0: choose.  Otherwise 2^split_k_log2 K ranges (rounded to whole steps).
 // `tuning` may override the choices: "r=<row tiles per group>,s=<K ranges>,w=<waves>,g=<grid.x>".
@@ -610,7 +637,7 @@ hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int spl
     p.g           = g;
     p.bf16_out    = out_dtype == In16::bf16 ? 1 : 0;
     p.n_tiles     = (g.N + 15) / 16;
-    p.xs_vec4     = ((g.kblocks & 3) == 0 && ((uintptr_t)g.xs & 15) == 0) ? 1 : 0;
+    p.xs_vec4     = (g.xs_k == 1 && (g.xs_m & 3) == 0 && ((uintptr_t)g.xs & 15) == 0) ? 1 : 0;
     const int mt        = (g.M + 15) / 16;
     const int max_waves = 4;
     const int steps     = (g.kblocks + kStepKb - 1) / kStepKb;

@@ -36,7 +36,10 @@ __device__ __forceinline__ i32x8 read_frag(const uint8_t* base, uint32_t row, ui
     return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 }
 
-template <In16 DT>
+// SHUF: weights pre-shuffled (16,16).  A 16-row tile's K block is then 2 KiB of contiguous global
+// memory already in fragment order; the weight slab in LDS is a straight copy of it (tile after
+// tile), and a lane's fragment halves sit at kg*512 + l16*16 and 256 bytes further.
+template <In16 DT, bool SHUF>
 __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams p, int tiles_m,
                                                                 int tiles_n)
 {
@@ -71,7 +74,15 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     {
         const uint32_t r = 64u * i + 8u * wave + (lane >> 3);
         const uint32_t c = (lane & 7u) ^ ((r >> 1) & 7u);
-        if(i < 4)
+        if(i < 4 && SHUF)
+        {
+            // unit U = 8 i + wave is half of tile U/2's K block: 1 KiB, copied as it lies
+            const uint32_t U    = 8u * i + wave;
+            uint32_t       tile = ((uint32_t)n0 >> 4) + (U >> 1);
+            tile                = min(tile, ((uint32_t)p.N >> 4) - 1u);
+            goff[i]             = tile * 16u * (uint32_t)p.K + (U & 1u) * 1024u + (uint32_t)lane * 16u;
+        }
+        else if(i < 4)
         {
             uint32_t n = n0 + r;
             n          = n < (uint32_t)p.N ? n : (uint32_t)p.N - 1;
@@ -108,7 +119,7 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     {
         uint32_t m = m0 + 64u * (wave & 3) + lane;
         m          = m < (uint32_t)p.M ? m : (uint32_t)p.M - 1;
-        xs_goff    = m * (uint32_t)p.kblocks * 4u;
+        xs_goff    = m * (uint32_t)p.xs_m * 4u;
     }
 
     // ---- scales: x_scale comes through LDS with each stage, w_scale: one block per wave
@@ -122,6 +133,8 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     const uint32_t sw     = (uint32_t)(l16 >> 1) & 7u;
     const uint32_t lo_off = (uint32_t)l16 * 128u + (((2u * kg) ^ sw) << 4);
     const uint32_t hi_off = (uint32_t)l16 * 128u + (((2u * kg + 1u) ^ sw) << 4);
+    const uint32_t wlo_off = SHUF ? (uint32_t)kg * 512u + (uint32_t)l16 * 16u : lo_off;
+    const uint32_t whi_off = SHUF ? wlo_off + 256u : hi_off;
     const uint32_t w_base = (uint32_t)wn * (128u * 128u);
     const uint32_t x_base = (uint32_t)kBN * 128u + (uint32_t)wm * (64u * 128u);
 
@@ -154,6 +167,11 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         asm volatile("v_fmac_f32 %0, %1, %2" : "+v"((ACC)[3]) : "v"((P)[3]), "v"(S));      \
     } while(0)
 
+    auto read_frag_w = [&](uint32_t stage_off, uint32_t tile_off) -> i32x8 {
+        const i32x4 lo = *(lds_vec_ptr)(smem3 + stage_off + wlo_off + tile_off);
+        const i32x4 hi = *(lds_vec_ptr)(smem3 + stage_off + whi_off + tile_off);
+        return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
     auto read_frag_v = [&](uint32_t stage_off, uint32_t tile_off) -> i32x8 {
         const i32x4 lo = *(lds_vec_ptr)(smem3 + stage_off + lo_off + tile_off);
         const i32x4 hi = *(lds_vec_ptr)(smem3 + stage_off + hi_off + tile_off);
@@ -221,13 +239,14 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         const int      kn       = kb + 1 < p.kblocks ? kb + 1 : kb; // last pass re-fetches, unused
         const uint32_t dma_dst  = __builtin_amdgcn_readfirstlane(
             (uint32_t)(uintptr_t)(smem3 + (cur ^ 1) * kStageBytes + wave * 1024));
-        const size_t   dma_koff = (size_t)kn * 128;
+        const size_t   dma_koff   = (size_t)kn * 128;
+        const size_t   dma_koff_w = SHUF ? (size_t)kn * 2048 : dma_koff;
 
         if((kb & 63) == 0 && kb != 0)
             ws_vec = load_ws_window(kb);
         const float wsc = ws_at(kb);
 
-        aw[0] = read_frag_v(stage, w_base); // weight fragment 0 of this K block
+        aw[0] = read_frag_w(stage, w_base); // weight fragment 0 of this K block
         float sc[4];
 #pragma unroll
         for(int j = 0; j < 4; ++j)
@@ -237,7 +256,7 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         for(int q = 0; q < 32; ++q)
         {
             if(q == 2)
-                aw[1] = read_frag_v(stage, w_base + 1 * 2048);
+                aw[1] = read_frag_w(stage, w_base + 1 * 2048);
 
             if(q < 8) // deferred tile (6 + (q & 1), q >> 1) of the previous K block
                 FP8BS_MFMA(P[q & 3], aw[2 + (q & 1)], bx[q >> 1]);
@@ -248,27 +267,27 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
             if(q < 8 && (q & 1))
                 bx[q >> 1] = read_frag_v(stage, x_base + (q >> 1) * 2048);
             if(q == 6)
-                aw[2] = read_frag_v(stage, w_base + 2 * 2048);
+                aw[2] = read_frag_w(stage, w_base + 2 * 2048);
             if(q == 7)
-                aw[3] = read_frag_v(stage, w_base + 3 * 2048);
+                aw[3] = read_frag_w(stage, w_base + 3 * 2048);
             if(q == 11)
-                aw[0] = read_frag_v(stage, w_base + 4 * 2048);
+                aw[0] = read_frag_w(stage, w_base + 4 * 2048);
             if(q == 15)
-                aw[1] = read_frag_v(stage, w_base + 5 * 2048);
+                aw[1] = read_frag_w(stage, w_base + 5 * 2048);
             if(q == 19)
-                aw[2] = read_frag_v(stage, w_base + 6 * 2048);
+                aw[2] = read_frag_w(stage, w_base + 6 * 2048);
             if(q == 23)
-                aw[3] = read_frag_v(stage, w_base + 7 * 2048);
+                aw[3] = read_frag_w(stage, w_base + 7 * 2048);
 
             // next stage: 8 slab loads and the x_scale column, behind the first 17 slots
             if((q & 1) == 1 && q < 16)
             {
                 const int u = q >> 1;
-                dma16(dma_dst + u * 8192, goff[u], (u < 4 ? p.wq : p.xq) + dma_koff);
+                dma16(dma_dst + u * 8192, goff[u], u < 4 ? p.wq + dma_koff_w : p.xq + dma_koff);
             }
             if(q == 16 && wave < 4)
                 dma4(__builtin_amdgcn_readfirstlane(dma_dst - wave * 1024 + kSlabBytes + wave * 256),
-                     xs_goff + (uint32_t)kn * 4u, p.xs);
+                     xs_goff + (uint32_t)kn * (uint32_t)p.xs_k * 4u, p.xs);
 
             // fold in the product issued two slots ago
             if(q == 0)
@@ -342,15 +361,16 @@ bool gemm_prefill_supports(const GemmKernelParams& p)
     // 32-bit byte offsets inside the operand matrices, 8-byte aligned output rows
     return p.kblocks >= 1 && (uint64_t)p.N * (uint64_t)p.ldb < (1ull << 32) &&
            (uint64_t)p.M * (uint64_t)p.lda < (1ull << 32) &&
-           (uint64_t)p.M * (uint64_t)p.kblocks < (1ull << 32) && (p.N % 4) == 0;
+           (uint64_t)p.M * (uint64_t)p.kblocks < (1ull << 30) && (p.N % 4) == 0;
 }
 
 hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, hipStream_t stream)
 {
     const int    tiles_m = (p.M + kBM - 1) / kBM, tiles_n = (p.N + kBN - 1) / kBN;
     const size_t smem    = (size_t)kStages * kStageBytes;
-    auto         kernel  = out_dtype == In16::bf16 ? gemm_prefill_kernel<In16::bf16>
-                                                   : gemm_prefill_kernel<In16::fp16>;
+    const bool   bf      = out_dtype == In16::bf16;
+    auto         kernel  = p.w_shuffled ? (bf ? gemm_prefill_kernel<In16::bf16, true> : gemm_prefill_kernel<In16::fp16, true>)
+                                        : (bf ? gemm_prefill_kernel<In16::bf16, false> : gemm_prefill_kernel<In16::fp16, false>);
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)smem);
     if(e != hipSuccess)

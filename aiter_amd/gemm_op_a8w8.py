@@ -8,6 +8,8 @@ boundary disappears while the call signatures stay.
 
 from __future__ import annotations
 
+from typing import Optional
+
 import torch
 from torch import Tensor
 
@@ -50,6 +52,50 @@ def gemm_a8w8_blockscale(
     Y = torch.empty(m, n, dtype=dtype, device=XQ.device)
     # -1: the library chooses kernel and K split from the shape
     _ffi.call("gemm_a8w8_blockscale", XQ, WQ, x_scale, w_scale, Y, -1, "")
+    return Y
+
+
+def gemm_a8w8_blockscale_bpreshuffle_ck(
+    XQ: Tensor,
+    WQ: Tensor,
+    x_scale: Tensor,
+    w_scale: Tensor,
+    Out: Tensor,
+    kernelName: str = "",
+) -> Tensor:
+    """aiter/ops/gemm_op_a8w8.py:318-330: ``WQ`` holds ``shuffle_weight(w, layout=(16, 16))`` and
+    ``x_scale`` is column-major; writes ``Out`` and returns it."""
+    _ffi.call("gemm_a8w8_blockscale_bpreshuffle", XQ, WQ, x_scale, w_scale, Out, kernelName or "")
+    return Out
+
+
+def gemm_a8w8_blockscale_bpreshuffle(
+    XQ: Tensor,
+    WQ: Tensor,
+    x_scale: Tensor,
+    w_scale: Tensor,
+    dtype: torch.dtype = dtypes.bf16,
+    out: Optional[Tensor] = None,
+) -> Tensor:
+    """aiter/ops/gemm_op_a8w8.py:908-1087.
+
+    XQ [M,K] fp8; WQ [N,K] fp8 pre-shuffled with :func:`aiter_amd.shuffle_weight` (layout
+    (16,16)); x_scale the [M,K/128] scales stored column-major (what the quant kernels write
+    with ``transpose_scale=True``), either as a contiguous buffer or as a strided [M,K/128]
+    view; w_scale [ceil(N/128),K/128] fp32.  ``out``, when given, receives the result.
+    """
+    assert dtype in [dtypes.bf16, dtypes.fp16], f"Output {dtype=} is currently not supported in gemm_a8w8"
+    m = XQ.shape[0]
+    n = WQ.shape[0]
+    if out is not None:
+        assert out.shape == (m, n) and out.dtype == dtype and out.device == XQ.device, (
+            f"gemm_a8w8_blockscale_bpreshuffle: out buffer {tuple(out.shape)}/{out.dtype} != expected "
+            f"({m},{n})/{dtype}"
+        )
+        Y = out
+    else:
+        Y = torch.empty(m, n, dtype=dtype, device=XQ.device)
+    _ffi.call("gemm_a8w8_blockscale_bpreshuffle", XQ, WQ, x_scale, w_scale, Y, "")
     return Y
 
 

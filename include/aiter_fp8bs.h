@@ -140,6 +140,22 @@ int gemm_a8w8_blockscale(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t*
                          aiter_tensor_t* w_scale, aiter_tensor_t* Out, int64_t splitK,
                          const char* kernelName, aiter_stream_t stream);
 
+/*
+ * The same GEMM on pre-shuffled weights.  Replaces gemm_a8w8_blockscale_bpreshuffle,
+ * csrc/ck_gemm_a8w8_blockscale_bpreshuffle/gemm_a8w8_blockscale_bpreshuffle.cu:64-89 (declared
+ * include/gemm_a8w8_blockscale_bpreshuffle.h:7-13, binding aiter/ops/gemm_op_a8w8.py:318-330).
+ *   WQ      fp8 [N, K] contiguous, holding shuffle_weight(w, layout=(16,16))
+ *           (aiter/ops/shuffle.py:192-205): per 16-row tile and 32-byte K chunk, the 16 rows'
+ *           first 16 bytes, then their second 16 bytes.  N % 16 == 0.
+ *   x_scale fp32, M*K/128 values stored column-major: element (m, kb) at kb*M + m.  Accepted
+ *           as a contiguous buffer of any shape with that many elements or as an [M, K/128]
+ *           view with strides (1, M) (op_tests/test_gemm_a8w8_blockscale.py:112-125).
+ *   XQ, w_scale, Out, kernelName and the arithmetic are those of gemm_a8w8_blockscale.
+ */
+int gemm_a8w8_blockscale_bpreshuffle(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t* x_scale,
+                                     aiter_tensor_t* w_scale, aiter_tensor_t* Out,
+                                     const char* kernelName, aiter_stream_t stream);
+
 /* Comma-separated list of the tile kernels gemm_a8w8_blockscale can be asked for by name
  * (the counterpart of the reference's generated kernel zoo,
  * csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale_instance.py:73-117). */

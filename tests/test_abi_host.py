@@ -181,3 +181,22 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_ffi, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(RuntimeError, match="no fallback"):
         _ffi.load_library()
+
+
+def test_shuffle_weight_closed_form():
+    # independent statement of the (16,16) layout: byte b of half h of 32-wide chunk c of row r of
+    # tile t sits at t*16*K + c*512 + h*256 + r*16 + b
+    import aiter_amd
+
+    n, k = 48, 160
+    w = torch.arange(n * k, dtype=torch.int32).remainder(251).to(torch.uint8).view(n, k)
+    flat = aiter_amd.shuffle_weight(w).flatten()
+    for t, c, h, r, b in [(0, 0, 0, 0, 0), (2, 4, 1, 15, 15), (1, 3, 0, 7, 9), (2, 0, 1, 3, 0), (0, 4, 1, 0, 15)]:
+        assert flat[t * 16 * k + c * 512 + h * 256 + r * 16 + b] == w[t * 16 + r, c * 32 + h * 16 + b]
+    # it is a permutation, and leading dimensions are shuffled matrix by matrix
+    assert torch.equal(flat.sort().values, w.flatten().sort().values)
+    w3 = torch.stack([w, w.flip(0)])
+    s3 = aiter_amd.shuffle_weight(w3)
+    assert torch.equal(s3[0], aiter_amd.shuffle_weight(w)) and torch.equal(s3[1], aiter_amd.shuffle_weight(w.flip(0)))
+    with pytest.raises(ValueError):
+        aiter_amd.shuffle_weight(w[:40])
