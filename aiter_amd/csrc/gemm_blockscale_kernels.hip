@@ -170,12 +170,17 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
     const char* name = (a.kernel_name && a.kernel_name[0]) ? a.kernel_name : nullptr;
     if(name == nullptr)
     {
-        if(gemm_decode_supports(p))
+        // Up to 64 rows the weight-streaming kernel always wins.  Beyond that it re-reads the
+        // activations once per 32 weight rows, which pays only while the 256x256 tiling would
+        // leave most of the chip without a tile (measured crossover: about 48 tiles).
+        const int64_t prefill_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
+        const bool    stream        = gemm_decode_supports(p) && (p.M <= 64 || prefill_tiles < 48);
+        if(stream)
             name = "decode_stream";
-        else if(a.M < 256 || !gemm_prefill_supports(p))
-            name = "tile_128x128";
-        else
+        else if(gemm_prefill_supports(p))
             name = "prefill_256x256";
+        else
+            name = "tile_128x128";
     }
     if(strcmp(name, "tile_16x256") == 0)
         return launch_tile<DT, 16, 256, 1, 4>(p, stream);
@@ -189,7 +194,7 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
         const char* tuning = name[13] == ':' ? name + 14 : nullptr;
         if(!gemm_decode_supports(p))
         {
-            *why = "decode_stream handles 1 <= M <= 64 (this layout of weights / x_scale included?)";
+            *why = "decode_stream handles 1 <= M <= 512";
             return hipErrorInvalidValue;
         }
         return launch_gemm_decode(p, DT, a.split_k_log2, a.device_id, stream, tuning);

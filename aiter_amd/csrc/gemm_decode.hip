@@ -27,6 +27,7 @@ namespace {
 
 constexpr int kStepKb = 4; // K blocks per wave and step
 constexpr int kMaxDynamicLds = 128 * 1024;
+constexpr int kDecodeMaxM    = 512; // 8 chunks of 64 activation rows
 
 struct DecodeParams
 {
@@ -36,6 +37,7 @@ struct DecodeParams
     int32_t   kb_per_split; // K blocks per workgroup-level K range
     int32_t   splits;       // number of such ranges (grid.y)
     int32_t   bf16_out;
+    int32_t   m_chunks;     // chunks of MT x 16 activation rows a workgroup walks per row group
     int32_t   grid_x, waves; // launch dimensions, passed explicitly: the implicit ones cost a dependent load
     int32_t   xs_vec4;      // x_scale rows can be read four K blocks at a time (16-byte aligned)
     float*    partial;      // [splits][n_groups][R * MT * 64] x 4 fp32 when splits > 1
@@ -59,7 +61,8 @@ constexpr int decode_max_waves()
 // makes the multiply straight-line code; otherwise the block count of a step is a run-time value.
 // SHUF: the weights are pre-shuffled (16,16): a lane's MFMA fragment is then two coalesced 16-byte
 // loads and needs no transposition.
-template <int MT, int R, bool SINGLE, bool FULL, bool SHUF>
+// CHUNKED (SINGLE only): more than 64 activation rows, walked in chunks of MT x 16 per row group.
+template <int MT, int R, bool SINGLE, bool FULL, bool SHUF, bool CHUNKED>
 __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kernel(DecodeParams p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -74,7 +77,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
     FP8BS_TOUCH(g.K); FP8BS_TOUCH(g.xs_m); FP8BS_TOUCH(g.xs_k);
     FP8BS_TOUCH(p.n_tiles); FP8BS_TOUCH(p.n_groups); FP8BS_TOUCH(p.kb_per_split); FP8BS_TOUCH(p.splits);
     FP8BS_TOUCH(p.bf16_out); FP8BS_TOUCH(p.xs_vec4); FP8BS_TOUCH(p.partial); FP8BS_TOUCH(p.partial_bytes);
-    FP8BS_TOUCH(p.tickets); FP8BS_TOUCH(p.grid_x); FP8BS_TOUCH(p.waves);
+    FP8BS_TOUCH(p.tickets); FP8BS_TOUCH(p.grid_x); FP8BS_TOUCH(p.waves); FP8BS_TOUCH(p.m_chunks);
 #undef FP8BS_TOUCH
 
     const int t = threadIdx.x, lane = t & 63;
@@ -108,17 +111,22 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
     };
 
     // activation rows this lane fetches (two per m tile: rows crow and 8 + crow of the tile) and
-    // the row whose scales it needs (rows past M re-read the last one, never stored)
+    // the row whose scales it needs (rows past M re-read the last one, never stored), for the
+    // chunk of 64 rows that starts at m_base
     const uint8_t* xrow[MT][2];
     const float*   xsrow[MT];
+    auto           set_chunk = [&](int m_base) {
 #pragma unroll
-    for(int j = 0; j < MT; ++j)
-    {
+        for(int j = 0; j < MT; ++j)
+        {
 #pragma unroll
-        for(int h = 0; h < 2; ++h)
-            xrow[j][h] = g.xq + (size_t)min(j * 16 + h * 8 + crow, g.M - 1) * g.lda + cchunk * 16;
-        xsrow[j] = g.xs + (size_t)min(j * 16 + l16, g.M - 1) * g.xs_m;
-    }
+            for(int h = 0; h < 2; ++h)
+                xrow[j][h] =
+                    g.xq + (size_t)min(m_base + j * 16 + h * 8 + crow, g.M - 1) * g.lda + cchunk * 16;
+            xsrow[j] = g.xs + (size_t)min(m_base + j * 16 + l16, g.M - 1) * g.xs_m;
+        }
+    };
+    set_chunk(0);
 
     i32x8 bx[MT][kStepKb];
     float xsv[MT][kStepKb];
@@ -167,7 +175,8 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                 s[r][i] = wsp[kslot(kb0, nk, i)];
         }
     };
-    auto issue_x = [&](int kb0, int nk, u32x4(&raw)[MT][kStepKb][2], int j_lo, int j_hi) {
+    auto issue_x = [&](int kb0, int nk, u32x4(&raw)[MT][kStepKb][2], float(&xs_out)[MT][kStepKb], int j_lo,
+                       int j_hi) {
 #pragma unroll
         for(int j = 0; j < MT; ++j)
         {
@@ -183,13 +192,13 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                 const f32x4 v = *(const f32x4*)(xsrow[j] + kb0);
 #pragma unroll
                 for(int i = 0; i < kStepKb; ++i)
-                    xsv[j][i] = v[i];
+                    xs_out[j][i] = v[i];
             }
             else
             {
 #pragma unroll
                 for(int i = 0; i < kStepKb; ++i)
-                    xsv[j][i] = xsrow[j][(size_t)kslot(kb0, nk, i) * g.xs_k];
+                    xs_out[j][i] = xsrow[j][(size_t)kslot(kb0, nk, i) * g.xs_k];
             }
         }
     };
@@ -263,10 +272,13 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
     };
 
     // element e of a group's tile set -> (row tile r, m tile j, lane ln): that lane's 4 outputs
-    auto store_out = [&](int grp, int e, const f32x4& v) {
+    // A unit of output is an "item": row group grp x chunk c of 64 activation rows, numbered
+    // grp * m_chunks + c (with M <= 64 there is one chunk and item == grp).
+    auto store_out = [&](int item, int e, const f32x4& v) {
+        const int grp = item / p.m_chunks, chunk = item - grp * p.m_chunks;
         const int r = e / (MT * 64), j = (e >> 6) % MT, ln = e & 63;
         const int tile = grp * R + r;
-        const int m = j * 16 + (ln & 15), n = tile * 16 + (ln >> 4) * 4;
+        const int m = chunk * (MT * 16) + j * 16 + (ln & 15), n = tile * 16 + (ln >> 4) * 4;
         if(tile >= p.n_tiles || m >= g.M)
             return;
         uint16_t* dst = g.out + (size_t)m * g.N + n;
@@ -313,14 +325,15 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
             sum = w < nw ? sum + v[w] : sum;
         return sum;
     };
-    auto flush_group_split = [&](int grp, const f32x4* red) {
+    auto flush_group_split = [&](int grp /* item */, const f32x4* red) {
+        const size_t n_items = (size_t)p.n_groups * p.m_chunks;
         // The workgroups that share a row group run on different XCDs, whose L2 caches are not
         // coherent with each other; every access to the exchanged tiles therefore bypasses them
         // (sc1), and the stores are waited for before the ticket is taken.
         for(int e = t; e < E; e += (nw * 64))
         {
             const f32x4    s   = wave_sum(red, e);
-            const uint32_t off = (uint32_t)(((size_t)split * p.n_groups + grp) * E + e) * 16u;
+            const uint32_t off = (uint32_t)(((size_t)split * n_items + grp) * E + e) * 16u;
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, s), part_rsrc, off, 0, kCoherent);
         }
         __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): the stores above have reached memory
@@ -337,7 +350,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
             f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
             for(int sp = 0; sp < p.splits; ++sp) // split order, whoever arrived last
             {
-                const uint32_t off = (uint32_t)(((size_t)sp * p.n_groups + grp) * E + e) * 16u;
+                const uint32_t off = (uint32_t)(((size_t)sp * n_items + grp) * E + e) * 16u;
                 s += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, off, 0, kCoherent));
             }
             store_out(grp, e, s);
@@ -378,9 +391,9 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
             pslot ^= 1;
         }
     };
-    auto park_current = [&]() {
+    auto park_current = [&](int item) {
         park(pslot);
-        prev = grp;
+        prev = item;
     };
 
     if constexpr(SINGLE)
@@ -391,6 +404,90 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
         // load is still to fill would wait for that load)
         const int kb0 = kb_lo + wave * kStepKb;
         const int nk  = max(0, min(kStepKb, kb_hi - kb0));
+        if constexpr(CHUNKED)
+        {
+            {
+                // More than 64 activation rows: the weights of a row group are turned into
+                // fragments once and stay in registers while the workgroup walks the chunks
+                // of MT x 16 rows; each chunk's activations are requested while the previous chunk
+                // is multiplied, the next group's weights while the current group is walked.
+                u32x4 xraw[MT][kStepKb][2];
+                float xsn[MT][kStepKb];
+                auto  issue_chunk = [&](int chunk) {
+                    set_chunk(chunk * (MT * 16));
+                    issue_x(kb0, nk, xraw, xsn, 0, MT);
+                };
+                u32x4 raw[R][kStepKb][2];
+                float ws_next[R][kStepKb], ws_cur[R][kStepKb];
+                if(nk > 0)
+                {
+                    issue_w(grp, kb0, nk, raw, ws_next);
+                    issue_chunk(0);
+                }
+                for(; grp < p.n_groups; grp += stride)
+                {
+                    const bool more = grp + stride < p.n_groups;
+                    i32x8      aw[R][kStepKb];
+                    if(nk > 0)
+                    {
+#pragma unroll
+                        for(int r = 0; r < R; ++r)
+#pragma unroll
+                            for(int i = 0; i < kStepKb; ++i)
+                            {
+                                aw[r][i]     = SHUF ? as_fragment(raw[r][i]) : settle(raw[r][i]);
+                                ws_cur[r][i] = ws_next[r][i];
+                            }
+                    }
+                    for(int chunk = 0; chunk < p.m_chunks; ++chunk)
+                    {
+                        float xsc[MT][kStepKb];
+                        clear_acc();
+                        if(nk > 0)
+                        {
+                            settle_x(xraw);
+#pragma unroll
+                            for(int j = 0; j < MT; ++j)
+#pragma unroll
+                                for(int i = 0; i < kStepKb; ++i)
+                                    xsc[j][i] = xsn[j][i];
+                            // what the next item needs goes out before this one is multiplied;
+                            // the raw weight registers are free since the fragments were formed
+                            if(chunk + 1 < p.m_chunks)
+                                issue_chunk(chunk + 1);
+                            else if(more)
+                            {
+                                issue_w(grp + stride, kb0, nk, raw, ws_next);
+                                issue_chunk(0);
+                            }
+#pragma unroll
+                            for(int j = 0; j < MT; ++j)
+#pragma unroll
+                                for(int i = 0; i < kStepKb; ++i)
+                                {
+                                    if(FULL || i < nk)
+                                    {
+#pragma unroll
+                                        for(int r = 0; r < R; ++r)
+                                        {
+                                            const f32x4 part = mfma_16x16x128_fp8(aw[r][i], bx[j][i],
+                                                                                  f32x4{0.f, 0.f, 0.f, 0.f});
+                                            const float sc   = xsc[j][i] * ws_cur[r][i];
+#pragma unroll
+                                            for(int c = 0; c < 4; ++c)
+                                                acc[r][j][c] = __builtin_fmaf(part[c], sc, acc[r][j][c]);
+                                        }
+                                    }
+                                }
+                        }
+                        flush_prev();
+                        park_current(grp * p.m_chunks + chunk);
+                    }
+                }
+                flush_prev();
+                return;
+            }
+        }
         u32x4     raw_a[R][kStepKb][2], raw_b[R][kStepKb][2];
         float     ws_a[R][kStepKb], ws_b[R][kStepKb];
         {
@@ -409,7 +506,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                 {
                     // narrow activations leave registers to spare: the second group's weights
                     // are requested at once, behind the first group's and the activations
-                    issue_x(kb0, nk, xraw, 0, MT);
+                    issue_x(kb0, nk, xraw, xsv, 0, MT);
                     if(more)
                     {
                         issue_w(grp + stride, kb0, nk, raw_b, ws_b);
@@ -424,14 +521,14 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                 }
                 else
                 {
-                    issue_x(kb0, nk, xraw, 0, kHalf);
+                    issue_x(kb0, nk, xraw, xsv, 0, kHalf);
                     i32x8 aw[R][kStepKb];
 #pragma unroll
                     for(int r = 0; r < R; ++r)
 #pragma unroll
                         for(int i = 0; i < kStepKb; ++i)
                             aw[r][i] = SHUF ? as_fragment(raw_a[r][i]) : settle(raw_a[r][i]);
-                    issue_x(kb0, nk, xraw, kHalf, MT);
+                    issue_x(kb0, nk, xraw, xsv, kHalf, MT);
                     multiply_first(nk, aw, ws_a, xraw, 0, kHalf);
                     if(more) // the next group's weights, now that half of the raw registers are free
                     {
@@ -442,7 +539,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                         multiply_first(nk, aw, ws_a, xraw, kHalf, MT);
                 }
             }
-            park_current();
+            park_current(grp);
             grp += stride;
         }
         while(grp < p.n_groups) // raw_b holds this group
@@ -461,7 +558,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                 if(nk > 0)
                     multiply(nk, raw_b, ws_b);
             }
-            park_current();
+            park_current(grp);
             grp += stride;
             if(grp >= p.n_groups)
                 break;
@@ -479,37 +576,40 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                 if(nk > 0)
                     multiply(nk, raw_a, ws_a);
             }
-            park_current();
+            park_current(grp);
             grp += stride;
         }
     }
     else
     {
-        // long K: every wave takes several steps; activations are re-read per row group
+        // long K: every wave takes several steps; activations are re-read per item
         for(; grp < p.n_groups; grp += stride)
-        {
-            clear_acc();
-            bool flushed = false;
-            for(int kb0 = kb_lo + wave * kStepKb; kb0 < kb_hi; kb0 += nw * kStepKb)
+            for(int chunk = 0; chunk < p.m_chunks; ++chunk)
             {
-                const int nk = min(kStepKb, kb_hi - kb0);
-                u32x4     wraw[R][kStepKb][2];
-                u32x4     xraw[MT][kStepKb][2];
-                float     wsv[R][kStepKb];
-                issue_w(grp, kb0, nk, wraw, wsv);
-                issue_x(kb0, nk, xraw, 0, MT);
-                if(!flushed) // the previous group's sum, behind this group's first requests
+                if(p.m_chunks > 1)
+                    set_chunk(chunk * (MT * 16));
+                clear_acc();
+                bool flushed = false;
+                for(int kb0 = kb_lo + wave * kStepKb; kb0 < kb_hi; kb0 += nw * kStepKb)
                 {
-                    flush_prev();
-                    flushed = true;
+                    const int nk = min(kStepKb, kb_hi - kb0);
+                    u32x4     wraw[R][kStepKb][2];
+                    u32x4     xraw[MT][kStepKb][2];
+                    float     wsv[R][kStepKb];
+                    issue_w(grp, kb0, nk, wraw, wsv);
+                    issue_x(kb0, nk, xraw, xsv, 0, MT);
+                    if(!flushed) // the previous item's sum, behind this item's first requests
+                    {
+                        flush_prev();
+                        flushed = true;
+                    }
+                    settle_x(xraw);
+                    multiply(nk, wraw, wsv);
                 }
-                settle_x(xraw);
-                multiply(nk, wraw, wsv);
+                if(!flushed)
+                    flush_prev();
+                park_current(grp * p.m_chunks + chunk);
             }
-            if(!flushed)
-                flush_prev();
-            park_current();
-        }
     }
     flush_prev();
 }
@@ -580,10 +680,10 @@ int tuning_value(const char* tuning, const char* key)
     return 0;
 }
 
-template <int MT, int R, bool SINGLE, bool FULL, bool SHUF>
+template <int MT, int R, bool SINGLE, bool FULL, bool SHUF, bool CHUNKED = false>
 hipError_t launch_one(const DecodeParams& p, dim3 grid, int waves, size_t smem, hipStream_t stream)
 {
-    auto        kernel = gemm_decode_kernel<MT, R, SINGLE, FULL, SHUF>;
+    auto        kernel = gemm_decode_kernel<MT, R, SINGLE, FULL, SHUF, CHUNKED>;
     static bool raised[kMaxDevices]; // dynamic LDS above the default limit needs opting in, once
     int         dev = 0;
     (void)hipGetDevice(&dev);
@@ -603,6 +703,12 @@ template <int MT, int R, bool SHUF>
 hipError_t launch_mt_r(const DecodeParams& p, bool single, bool full, dim3 grid, int waves, size_t smem,
                        hipStream_t stream)
 {
+    if constexpr(MT == 2)
+    {
+        if(single && p.m_chunks > 1)
+            return full ? launch_one<MT, R, true, true, SHUF, true>(p, grid, waves, smem, stream)
+                        : launch_one<MT, R, true, false, SHUF, true>(p, grid, waves, smem, stream);
+    }
     if(single)
         return full ? launch_one<MT, R, true, true, SHUF>(p, grid, waves, smem, stream)
                     : launch_one<MT, R, true, false, SHUF>(p, grid, waves, smem, stream);
@@ -625,7 +731,7 @@ hipError_t launch_mt(const DecodeParams& p, int rows, bool single, bool full, di
 
 bool gemm_decode_supports(const GemmKernelParams& p)
 {
-    return p.M >= 1 && p.M <= 64 && p.kblocks >= 1;
+    return p.M >= 1 && p.M <= kDecodeMaxM && p.kblocks >= 1;
 }
 
 // split_k_log2 < 0: choose.  Otherwise 2^split_k_log2 K ranges (rounded to whole steps).
@@ -638,7 +744,7 @@ hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int spl
     p.bf16_out    = out_dtype == In16::bf16 ? 1 : 0;
     p.n_tiles     = (g.N + 15) / 16;
     p.xs_vec4     = (g.xs_k == 1 && (g.xs_m & 3) == 0 && ((uintptr_t)g.xs & 15) == 0) ? 1 : 0;
-    const int mt        = (g.M + 15) / 16;
+    int       mt        = g.M > 64 ? 4 : (g.M + 15) / 16; // m tiles a wave holds at a time
     const int max_waves = 4;
     const int steps     = (g.kblocks + kStepKb - 1) / kStepKb;
     const int kChipCus  = 256;
@@ -679,6 +785,11 @@ hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int spl
         waves = steps_per_split < max_waves ? steps_per_split : max_waves;
     const bool single = steps_per_split <= waves;
     const bool full   = (g.kblocks % kStepKb) == 0;
+    // more than 64 rows are walked in chunks: 32 rows at a time when the weights stay in registers
+    // across chunks (that path also stages the next chunk), else 64
+    if(g.M > 64 && single)
+        mt = 2;
+    p.m_chunks = g.M > 64 ? (g.M + mt * 16 - 1) / (mt * 16) : 1;
 
     int gx = tuning_value(tuning, "g");
     if(gx <= 0)
@@ -697,11 +808,11 @@ hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int spl
     const size_t tile_set = (size_t)rows * mt * 64 * 16; // bytes of one group's fp32 tile set
     if(splits > 1)
     {
-        const size_t bytes = (size_t)splits * p.n_groups * tile_set;
+        const size_t bytes = (size_t)splits * p.n_groups * p.m_chunks * tile_set;
         if(bytes >= ((size_t)1 << 31))
             return hipErrorInvalidValue;
         Workspace* w = nullptr;
-        hipError_t e = ensure_workspace(device_id, bytes, (size_t)p.n_groups, stream, &w);
+        hipError_t e = ensure_workspace(device_id, bytes, (size_t)p.n_groups * p.m_chunks, stream, &w);
         if(e != hipSuccess)
             return e;
         p.partial       = w->partial;

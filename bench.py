@@ -49,6 +49,9 @@ def parse_args():
                     help="'copy' is a plain 1 GiB device copy used to calibrate the rocprofv3 FETCH_SIZE / "
                     "WRITE_SIZE counters; it is not part of the path")
     ap.add_argument("--no-also", action="store_true", help="time only the primary workload")
+    ap.add_argument("--layout", default="plain", choices=["plain", "preshuffled"],
+                    help="GEMM workloads: row-major weights (gemm_a8w8_blockscale) or weights shuffled "
+                    "(16,16) with column-major x_scale (gemm_a8w8_blockscale_bpreshuffle)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     return ap.parse_args()
 
@@ -176,6 +179,8 @@ class QuantWorkload:
 
 
 class GemmWorkload:
+    layout = "plain"  # set from --layout before setup()
+
     def __init__(self, name, m, n, k, label):
         self.name, self.M, self.N, self.K, self.label = name, m, n, k, label
 
@@ -194,8 +199,9 @@ class GemmWorkload:
         if m >= 1024:
             ch = torch.randperm(k, generator=g, device=dev)[: max(1, k // 100)]
             x[:, ch] *= 50.0
+        pre = self.layout == "preshuffled"
         self.xq, self.xs = aiter_amd.get_hip_quant(aiter_amd.QuantType.per_1x128)(
-            x.bfloat16(), quant_dtype=dtypes.fp8)
+            x.bfloat16(), quant_dtype=dtypes.fp8, transpose_scale=pre)
         del x
 
         # Rotate the weights so that no call finds them in a cache: three buffers for the
@@ -204,6 +210,8 @@ class GemmWorkload:
         nbuf = 1 if (n * k) > (1 << 28) else 3
         pairs = [quant_weight_gpu(torch, dtypes.fp8, n, k, 10 + i, dev) for i in range(nbuf)]
         self.wqs = [p[0] for p in pairs]
+        if pre:
+            self.wqs = [aiter_amd.shuffle_weight(w.view(torch.uint8)).view(w.dtype) for w in self.wqs]
         self.ws = pairs[0][1]
         if m <= 64:
             want = -(-640_000_000 // (n * k))
@@ -214,13 +222,17 @@ class GemmWorkload:
 
     def step(self):
         self.i = (self.i + 1) % len(self.wqs)
-        self.aiter.gemm_a8w8_blockscale_ck(self.xq, self.wqs[self.i], self.xs, self.ws, self.out, splitK=-1)
+        if self.layout == "preshuffled":
+            self.aiter.gemm_a8w8_blockscale_bpreshuffle_ck(self.xq, self.wqs[self.i], self.xs, self.ws, self.out)
+        else:
+            self.aiter.gemm_a8w8_blockscale_ck(self.xq, self.wqs[self.i], self.xs, self.ws, self.out, splitK=-1)
 
     def flops(self):
         return 2.0 * self.M * self.N * self.K
 
     def describe(self):
-        return {"workload": self.label, "M": self.M, "N": self.N, "K": self.K, "kernel": "gemm_a8w8_blockscale"}
+        return {"workload": self.label, "M": self.M, "N": self.N, "K": self.K, "layout": self.layout,
+                "kernel": "gemm_a8w8_blockscale" + ("_bpreshuffle" if self.layout == "preshuffled" else "")}
 
     def result(self, sec):
         tf = self.flops() / sec / 1e12
@@ -236,6 +248,8 @@ class GemmWorkload:
     def cpu_baseline(self, torch):
         from oracle import torch_ref as tr
 
+        if self.layout == "preshuffled":
+            return None  # same arithmetic as the plain layout, whose run carries the CPU figure
         rows = min(self.M, 16)
         ncols = min(self.N, 4096)
         xq = self.xq[:rows].cpu()
@@ -428,6 +442,7 @@ def main():
     dev = "cuda:0"
     torch.cuda.set_device(0)
 
+    GemmWorkload.layout = args.layout
     wl = make_workload(args.workload)
     wl.setup(torch, dev)
     sec = time_steps(torch, wl.step, args.steps, args.warmup)

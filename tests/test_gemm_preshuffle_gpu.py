@@ -49,8 +49,9 @@ def test_matches_oracle_and_plain_layout(m, n, k, form):
 
 
 @pytest.mark.parametrize("kernel", ["tile_16x256", "tile_64x128", "tile_128x128", "prefill_256x256", "decode_stream"])
-def test_named_kernels(kernel):
-    m, n, k = (48, 1008, 1024) if kernel == "decode_stream" else (272, 1008, 1024)
+@pytest.mark.parametrize("m", [48, 272])
+def test_named_kernels(kernel, m):
+    n, k = 1008, 1024
     xq, wq, xs, ws = make_problem(m, n, k, seed=11, outliers=0.01)
     out = run_preshuffled(xq, wq, xs, ws, kernel=kernel)
     assert_close_to_f64(out, xq, wq, xs, ws, f"bpreshuffle {kernel}")
