@@ -49,6 +49,9 @@ def parse_args():
                     help="'copy' is a plain 1 GiB device copy used to calibrate the rocprofv3 FETCH_SIZE / "
                     "WRITE_SIZE counters; it is not part of the path")
     ap.add_argument("--no-also", action="store_true", help="time only the primary workload")
+    ap.add_argument("--rotate-mb", type=int, default=640,
+                    help="decode workloads: cycle through this many MB of weight copies (default 640, "
+                    "more than twice the last-level cache; 0 keeps three copies, which stay cached)")
     ap.add_argument("--layout", default="plain", choices=["plain", "preshuffled"],
                     help="GEMM workloads: row-major weights (gemm_a8w8_blockscale) or weights shuffled "
                     "(16,16) with column-major x_scale (gemm_a8w8_blockscale_bpreshuffle)")
@@ -180,6 +183,7 @@ class QuantWorkload:
 
 class GemmWorkload:
     layout = "plain"  # set from --layout before setup()
+    rotate_mb = 640   # set from --rotate-mb before setup()
 
     def __init__(self, name, m, n, k, label):
         self.name, self.M, self.N, self.K, self.label = name, m, n, k, label
@@ -214,7 +218,7 @@ class GemmWorkload:
             self.wqs = [aiter_amd.shuffle_weight(w.view(torch.uint8)).view(w.dtype) for w in self.wqs]
         self.ws = pairs[0][1]
         if m <= 64:
-            want = -(-640_000_000 // (n * k))
+            want = -(-self.rotate_mb * 1_000_000 // (n * k))
             self.wqs += [self.wqs[i % nbuf].clone() for i in range(max(0, want - nbuf))]
         self.weight_bytes_rotated = len(self.wqs) * n * k
         self.out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
@@ -443,6 +447,7 @@ def main():
     torch.cuda.set_device(0)
 
     GemmWorkload.layout = args.layout
+    GemmWorkload.rotate_mb = args.rotate_mb
     wl = make_workload(args.workload)
     wl.setup(torch, dev)
     sec = time_steps(torch, wl.step, args.steps, args.warmup)
