@@ -18,7 +18,12 @@ from .gemm_op_a8w8 import (
     gemm_kernel_names,
 )
 from .shuffle import shuffle_weight
-from .quant import dynamic_per_token_scaled_quant, get_hip_quant, per_group_quant_hip
+from .quant import (
+    dynamic_per_token_scaled_quant,
+    get_hip_quant,
+    per_group_quant_hip,
+    weight_per_128x128_quant,
+)
 from .rmsnorm import (
     add_rmsnorm,
     add_rmsnorm_quant,
@@ -33,6 +38,7 @@ __all__ = [
     "QuantType",
     "get_hip_quant",
     "shuffle_weight",
+    "weight_per_128x128_quant",
     "gemm_a8w8_blockscale_bpreshuffle",
     "gemm_a8w8_blockscale_bpreshuffle_ck",
     "per_group_quant_hip",

@@ -33,6 +33,7 @@ _SIGNATURES = {
     "add_rmsnorm_quant": [
         _TP, _TP, _TP, _TP, _TP, _TP, ctypes.c_float, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
     ],
+    "weight_per_128x128_quant": [_TP, _TP, _TP],
     "gemm_a8w8_blockscale": [_TP, _TP, _TP, _TP, _TP, ctypes.c_int64, ctypes.c_char_p],
     "gemm_a8w8_blockscale_bpreshuffle": [_TP, _TP, _TP, _TP, _TP, ctypes.c_char_p],
 }

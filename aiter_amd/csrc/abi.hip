@@ -543,6 +543,55 @@ int add_rmsnorm_quant(aiter_tensor_t* out, aiter_tensor_t* input, aiter_tensor_t
     });
 }
 
+int weight_per_128x128_quant(aiter_tensor_t* out, aiter_tensor_t* input, aiter_tensor_t* scales,
+                             aiter_stream_t stream)
+{
+    return guarded([&] {
+        const char* fn = "weight_per_128x128_quant";
+        check_tensor(fn, out, "out");
+        check_tensor(fn, input, "input");
+        check_tensor(fn, scales, "scales");
+        same_device(fn, {out, input, scales});
+        if(!is_f16_like(input->dtype_))
+            fail(fn, "input must be bf16 or fp16, got ", dtype_name(input->dtype_));
+        if(!is_fp8_like(out->dtype_))
+            fail(fn, "out must be fp8, got ", dtype_name(out->dtype_));
+        if(scales->dtype_ != AITER_DTYPE_fp32)
+            fail(fn, "scales must be fp32, got ", dtype_name(scales->dtype_));
+        if(input->ndim != 2 || out->ndim != 2)
+            fail(fn, "input and out must be 2-D [N, K]");
+        const int64_t N = input->shape[0], K = input->shape[1];
+        if(out->shape[0] != N || out->shape[1] != K)
+            fail(fn, "out must have the shape of input, [", N, ",", K, "]");
+        if(K % 128 != 0)
+            fail(fn, "K = ", K, " must be a multiple of 128");
+        if((K > 1 && input->strides[1] != 1) || (K > 1 && out->strides[1] != 1))
+            fail(fn, "input and out must be contiguous in K");
+        const int64_t ldw = N > 1 ? input->strides[0] : K, ldq = N > 1 ? out->strides[0] : K;
+        if(ldw < K || ldq < K || ldw % 8 != 0 || ldq % 16 != 0)
+            fail(fn, "row strides must be >= K and multiples of 16 bytes");
+        const int64_t nb = (N + 127) / 128, kb = K / 128;
+        if((int64_t)scales->numel_ != nb * kb || !contiguous(scales))
+            fail(fn, "scales must be contiguous [", nb, ",", kb, "], got ", scales->numel_, " elements");
+        if(N >= (1LL << 31) || K >= (1LL << 31) || nb > 65535)
+            fail(fn, "matrix too large");
+        check_aligned(fn, input, "input", 16);
+        check_aligned(fn, out, "out", 16);
+        check_aligned(fn, scales, "scales", 4);
+        fp8bs::WeightQuantArgs a{};
+        a.w     = input->ptr;
+        a.q     = (uint8_t*)out->ptr;
+        a.scale = (float*)scales->ptr;
+        a.N     = N;
+        a.K     = K;
+        a.ldw   = ldw;
+        a.ldq   = ldq;
+        a.dtype = in16_of(input->dtype_);
+        DeviceGuard guard(input->device_id);
+        check_hip(fn, fp8bs::launch_weight_block_quant(a, (hipStream_t)stream), nullptr);
+    });
+}
+
 int gemm_a8w8_blockscale(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t* x_scale,
                          aiter_tensor_t* w_scale, aiter_tensor_t* Out, int64_t splitK,
                          const char* kernelName, aiter_stream_t stream)

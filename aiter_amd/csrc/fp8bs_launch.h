@@ -28,6 +28,16 @@ struct QuantArgs
 };
 hipError_t launch_group_quant(const QuantArgs& a, hipStream_t stream);
 
+struct WeightQuantArgs
+{
+    const void* w;     // [N, K] 16-bit floats, row stride ldw elements
+    uint8_t*    q;     // [N, K] fp8 codes, row stride ldq elements
+    float*      scale; // [ceil(N/128), K/128]
+    int64_t     N, K, ldw, ldq;
+    In16        dtype;
+};
+hipError_t launch_weight_block_quant(const WeightQuantArgs& a, hipStream_t stream);
+
 struct NormArgs
 {
     const void* x;          // [rows, hidden] 16-bit, row stride x_stride (elements)

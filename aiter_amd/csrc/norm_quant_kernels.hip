@@ -151,15 +151,18 @@ __device__ __forceinline__ double wave_sum_f64(double v)
 // the scale; inf/inf is the default NaN, which has the sign bit set on x86.
 // Inlined on purpose: an out-of-line call would give the kernel a private (scratch) segment,
 // and waves that need scratch are dispatched far more slowly than the HBM stream can be fed.
-template <int LPG>
-__device__ __forceinline__ void quant16_slow(const float (&v)[16], u32x4& codes, float& scale)
+__device__ __forceinline__ uint32_t absmax_bits16(const float (&v)[16])
 {
     uint32_t mm = 0;
 #pragma unroll
     for(int i = 0; i < 16; ++i)
         mm = max(mm, __float_as_uint(v[i]) & 0x7fffffffu);
-    mm = group_max_u32<LPG>(mm); // as integers: NaN > inf > every finite magnitude
+    return mm; // as integers: NaN > inf > every finite magnitude
+}
 
+// mm: the group's largest |x| as an integer (absmax_bits16 reduced over the group)
+__device__ __forceinline__ void encode16_slow(const float (&v)[16], uint32_t mm, u32x4& codes, float& scale)
+{
     float s;
     if(mm > 0x7f800000u)
         s = __uint_as_float(mm | 0x00400000u);
@@ -189,8 +192,9 @@ __device__ __forceinline__ void quant16_slow(const float (&v)[16], u32x4& codes,
     scale = s;
 }
 
-template <int LPG>
-__device__ __forceinline__ void quant16(const float (&v)[16], u32x4& codes, float& scale)
+// largest |x| of 16 values as a float; a NaN (which fmaxf would drop) turns it into +inf, which
+// sends the group to the slow path
+__device__ __forceinline__ float amax16(const float (&v)[16])
 {
     float m  = 0.0f;
     bool  un = false;
@@ -200,32 +204,37 @@ __device__ __forceinline__ void quant16(const float (&v)[16], u32x4& codes, floa
         m = fmaxf(fmaxf(m, fabsf(v[i])), fabsf(v[i + 1]));
         un |= __builtin_isunordered(v[i], v[i + 1]);
     }
-    // a NaN would be dropped by fmaxf: send the group to the slow path through an infinite amax
-    m = un ? __builtin_inff() : m;
-    m = group_max_f32<LPG>(m);
+    return un ? __builtin_inff() : m;
+}
 
-    if(amax_allows_fast_path(__float_as_uint(m)))
-    {
-        const float s = m / 448.0f; // IEEE division
-        const float r = 1.0f / s;   // IEEE division: the correctly rounded reciprocal
-        uint32_t out[4];
+// m: the group's amax, for which amax_allows_fast_path holds
+__device__ __forceinline__ void encode16_fast(const float (&v)[16], float m, u32x4& codes, float& scale)
+{
+    const float s = m / 448.0f; // IEEE division
+    const float r = 1.0f / s;   // IEEE division: the correctly rounded reciprocal
+    uint32_t    out[4];
 #pragma unroll
-        for(int j = 0; j < 4; ++j)
-        {
-            int w = 0;
-            w = __builtin_amdgcn_cvt_pk_fp8_f32(div_by_scale(v[4 * j], s, r),
-                                                div_by_scale(v[4 * j + 1], s, r), w, false);
-            w = __builtin_amdgcn_cvt_pk_fp8_f32(div_by_scale(v[4 * j + 2], s, r),
-                                                div_by_scale(v[4 * j + 3], s, r), w, true);
-            out[j] = (uint32_t)w;
-        }
-        codes = u32x4{out[0], out[1], out[2], out[3]};
-        scale = s;
-    }
-    else
+    for(int j = 0; j < 4; ++j)
     {
-        quant16_slow<LPG>(v, codes, scale);
+        int w = 0;
+        w = __builtin_amdgcn_cvt_pk_fp8_f32(div_by_scale(v[4 * j], s, r), div_by_scale(v[4 * j + 1], s, r), w,
+                                            false);
+        w = __builtin_amdgcn_cvt_pk_fp8_f32(div_by_scale(v[4 * j + 2], s, r), div_by_scale(v[4 * j + 3], s, r),
+                                            w, true);
+        out[j] = (uint32_t)w;
     }
+    codes = u32x4{out[0], out[1], out[2], out[3]};
+    scale = s;
+}
+
+template <int LPG>
+__device__ __forceinline__ void quant16(const float (&v)[16], u32x4& codes, float& scale)
+{
+    const float m = group_max_f32<LPG>(amax16(v));
+    if(amax_allows_fast_path(__float_as_uint(m)))
+        encode16_fast(v, m, codes, scale);
+    else
+        encode16_slow(v, group_max_u32<LPG>(absmax_bits16(v)), codes, scale);
 }
 
 // ---------------------------------------------------------------- standalone group quant
@@ -340,6 +349,120 @@ hipError_t launch_group_quant(const QuantArgs& a, hipStream_t stream)
                   : launch_group_quant_t<In16::fp16, 32>(a, stream);
     default: return hipErrorInvalidValue;
     }
+}
+
+// ---------------------------------------------------------------- weight-side 128x128 block quant
+// One workgroup per 128x128 block of a [N, K] weight matrix: one scale per block, codes by the
+// same exact division as the activation quant.  Rows past N count as zeros (they do not move the
+// amax), as in the torch formulation that zero-pads ragged blocks
+// (op_tests/multigpu_tests/test_dispatch_combine.py:180-204 applies pertoken_quant,
+// aiter/ops/quant.py:64-94, to [n_blocks, 128*128] views).  An offline step: built for
+// exactness, not tuned.
+
+struct WeightQuantKernelParams
+{
+    const uint16_t* w;
+    uint8_t*        q;
+    float*          scale;
+    int32_t         N, K;
+    int64_t         ldw, ldq; // row strides in elements
+};
+
+template <class T, class Op>
+__device__ __forceinline__ T block256_reduce(T v, T* lds, Op op)
+{
+#pragma unroll
+    for(int off = 32; off >= 1; off >>= 1)
+        v = op(v, __shfl_xor(v, off, 64));
+    const int wave = threadIdx.x >> 6;
+    __syncthreads(); // lds may still be read from a previous reduction
+    if((threadIdx.x & 63) == 0)
+        lds[wave] = v;
+    __syncthreads();
+    return op(op(lds[0], lds[1]), op(lds[2], lds[3]));
+}
+
+template <In16 DT>
+__global__ __launch_bounds__(256) void weight_block_quant_kernel(WeightQuantKernelParams p)
+{
+    __shared__ float    red_f[4];
+    __shared__ uint32_t red_u[4];
+    const int t = threadIdx.x;
+    const int r = t >> 1, half = t & 1;      // block row, 64-element half of its 128 columns
+    const int n = blockIdx.y * 128 + r;
+    const int k0 = blockIdx.x * 128 + half * 64;
+    const bool live = n < p.N;
+
+    float v[4][16];
+#pragma unroll
+    for(int u = 0; u < 4; ++u)
+#pragma unroll
+        for(int i = 0; i < 16; ++i)
+            v[u][i] = 0.0f;
+    if(live)
+    {
+        const u32x4* src = (const u32x4*)(p.w + (size_t)n * p.ldw + k0);
+#pragma unroll
+        for(int u = 0; u < 4; ++u)
+        {
+            unpack8<DT>(src[2 * u], v[u]);
+            unpack8<DT>(src[2 * u + 1], v[u] + 8);
+        }
+    }
+    float m = 0.0f;
+#pragma unroll
+    for(int u = 0; u < 4; ++u)
+        m = fmaxf(m, amax16(v[u])); // +inf when the unit holds a NaN
+    m = block256_reduce(m, red_f, [](float a, float b) { return fmaxf(a, b); });
+
+    u32x4 codes[4];
+    float s = 1.0f;
+    if(amax_allows_fast_path(__float_as_uint(m)))
+    {
+#pragma unroll
+        for(int u = 0; u < 4; ++u)
+            encode16_fast(v[u], m, codes[u], s);
+    }
+    else
+    {
+        uint32_t mm = 0;
+#pragma unroll
+        for(int u = 0; u < 4; ++u)
+            mm = max(mm, absmax_bits16(v[u]));
+        mm = block256_reduce(mm, red_u, [](uint32_t a, uint32_t b) { return max(a, b); });
+#pragma unroll
+        for(int u = 0; u < 4; ++u)
+            encode16_slow(v[u], mm, codes[u], s);
+    }
+    if(live)
+    {
+        u32x4* dst = (u32x4*)(p.q + (size_t)n * p.ldq + k0);
+#pragma unroll
+        for(int u = 0; u < 4; ++u)
+            dst[u] = codes[u];
+    }
+    if(t == 0)
+        p.scale[(size_t)blockIdx.y * gridDim.x + blockIdx.x] = s;
+}
+
+hipError_t launch_weight_block_quant(const WeightQuantArgs& a, hipStream_t stream)
+{
+    if(a.N == 0 || a.K == 0)
+        return hipSuccess;
+    WeightQuantKernelParams p;
+    p.w     = (const uint16_t*)a.w;
+    p.q     = a.q;
+    p.scale = a.scale;
+    p.N     = (int32_t)a.N;
+    p.K     = (int32_t)a.K;
+    p.ldw   = a.ldw;
+    p.ldq   = a.ldq;
+    const dim3 grid((unsigned)(a.K / 128), (unsigned)((a.N + 127) / 128));
+    if(a.dtype == In16::bf16)
+        hipLaunchKernelGGL(weight_block_quant_kernel<In16::bf16>, grid, dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL(weight_block_quant_kernel<In16::fp16>, grid, dim3(256), 0, stream, p);
+    return hipGetLastError();
 }
 
 // ---------------------------------------------------------------- RMSNorm (+add) (+quant)

@@ -86,3 +86,20 @@ def get_hip_quant(qType):
         raise NotImplementedError(f"unsupported quant type {qType=}")
 
     return table.get(int(getattr(qType, "value", qType)), raise_NotImplementedError)
+
+
+def weight_per_128x128_quant(w: torch.Tensor, quant_dtype: torch.dtype = dtypes.fp8):
+    """[N, K] bf16/fp16 weights -> (fp8 codes [N, K], fp32 scales [ceil(N/128), K/128]).
+
+    The 128x128 block quantiser that produces the GEMM's ``WQ`` / ``w_scale``.  The reference
+    does this offline with torch ops (``pertoken_quant``, aiter/ops/quant.py:64-94, on
+    ``[n_blocks, 128*128]`` views, op_tests/multigpu_tests/test_dispatch_combine.py:180-204);
+    the result here is the same bit for bit.  K must be a multiple of 128; a ragged last row
+    block is quantised as if padded with zeros.
+    """
+    assert w.dim() == 2, "weight_per_128x128_quant expects a [N, K] matrix"
+    n, k = w.shape
+    wq = torch.empty(n, k, dtype=quant_dtype, device=w.device)
+    ws = torch.empty((n + 127) // 128, k // 128, dtype=torch.float32, device=w.device)
+    _ffi.call("weight_per_128x128_quant", wq, w, ws)
+    return wq, ws

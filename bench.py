@@ -108,16 +108,13 @@ def gemm_bytes(m, n, k):
 
 
 def quant_weight_gpu(torch, fp8, n, k, seed, dev):
-    """w ~ N(0, 0.02) quantised per 128x128 block on the GPU (setup only, never timed)."""
+    """w ~ N(0, 0.02) in bf16, quantised per 128x128 block by the library's own weight quantiser
+    (setup only, never timed)."""
+    import aiter_amd
+
     gw = torch.Generator(device=dev).manual_seed(seed)
-    nb, kb = (n + 127) // 128, k // 128
-    w = torch.zeros(nb * 128, k, device=dev)
-    w[:n] = torch.randn(n, k, generator=gw, device=dev) * 0.02
-    blocks = w.view(nb, 128, kb, 128)
-    amax = blocks.abs().amax(dim=(1, 3), keepdim=True)
-    scale = torch.where(amax == 0, torch.ones_like(amax), amax / 448.0)
-    wq = (blocks / scale).to(fp8).view(nb * 128, k)[:n].contiguous()
-    return wq, scale.view(nb, kb).contiguous()
+    w = (torch.randn(n, k, generator=gw, device=dev) * 0.02).bfloat16()
+    return aiter_amd.weight_per_128x128_quant(w, quant_dtype=fp8)
 
 
 # ---------------------------------------------------------------- workloads

@@ -122,6 +122,20 @@ int add_rmsnorm_quant(aiter_tensor_t* out, aiter_tensor_t* input, aiter_tensor_t
                       int shuffle_scale, int gemma_norm, aiter_stream_t stream);
 
 /*
+ * Weight-side quantiser: one fp32 scale per 128x128 block of a [N, K] weight matrix, fp8 codes by
+ * the same definition as the activation quant (scale = amax/448, zero block -> 1, code =
+ * e4m3fn(w / scale), true divisions).  The reference performs this offline step with torch ops,
+ * op_tests/multigpu_tests/test_dispatch_combine.py:180-204 (pertoken_quant,
+ * aiter/ops/quant.py:64-94, on [n_blocks, 128*128] views); this is the same arithmetic on the GPU.
+ *   input  bf16|fp16 [N, K], K % 128 == 0, row stride honoured; rows past N in the last block
+ *          count as zeros
+ *   out    fp8 [N, K], row stride honoured
+ *   scales fp32 [ceil(N/128), K/128] contiguous
+ */
+int weight_per_128x128_quant(aiter_tensor_t* out, aiter_tensor_t* input, aiter_tensor_t* scales,
+                             aiter_stream_t stream);
+
+/*
  * Block-scale FP8 GEMM.  Replaces gemm_a8w8_blockscale,
  * csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale.cu:82-114 (binding
  * aiter/ops/gemm_op_a8w8.py:285-298).
