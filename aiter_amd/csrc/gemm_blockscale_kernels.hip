@@ -159,7 +159,8 @@ static hipError_t launch_tile(const GemmKernelParams& p, hipStream_t stream)
     return hipGetLastError();
 }
 
-static const char* const kKernelNames = "tile_16x256,tile_64x128,tile_128x128,prefill_256x256,decode_stream";
+static const char* const kKernelNames =
+    "tile_16x256,tile_64x128,tile_128x128,mid_64x64,mid_64x128,mid_128x128,prefill_256x256,decode_stream";
 
 const char* gemm_kernel_names() { return kKernelNames; }
 
@@ -170,13 +171,16 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
     const char* name = (a.kernel_name && a.kernel_name[0]) ? a.kernel_name : nullptr;
     if(name == nullptr)
     {
-        // Up to 64 rows the weight-streaming kernel always wins.  Beyond that it re-reads the
-        // activations once per 32 weight rows, which pays only while the 256x256 tiling would
-        // leave most of the chip without a tile (measured crossover: about 48 tiles).
+        // Up to 64 activation rows the weight-streaming kernel wins everywhere.  Above that, the
+        // 256x256 tiling once it gives at least half of the compute units a tile, and the
+        // 128x128 / 64x64 tiling in between (measured crossovers on the DeepSeek shapes).
         const int64_t prefill_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
-        const bool    stream        = gemm_decode_supports(p) && (p.M <= 64 || prefill_tiles < 48);
-        if(stream)
+        if(p.M <= 64 && gemm_decode_supports(p))
             name = "decode_stream";
+        else if(prefill_tiles >= 128 && gemm_prefill_supports(p))
+            name = "prefill_256x256";
+        else if(gemm_mid_supports(p))
+            name = "mid_auto";
         else if(gemm_prefill_supports(p))
             name = "prefill_256x256";
         else
@@ -199,9 +203,28 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
         }
         return launch_gemm_decode(p, DT, a.split_k_log2, a.device_id, stream, tuning);
     }
+    if(strncmp(name, "mid_", 4) == 0)
+    {
+        const int tile = strcmp(name, "mid_128x128") == 0  ? 128
+                         : strcmp(name, "mid_64x128") == 0 ? 64128
+                         : strcmp(name, "mid_64x64") == 0  ? 64
+                         : strcmp(name, "mid_auto") == 0   ? 0
+                                                           : -1;
+        if(tile < 0)
+        {
+            *why = "unknown kernelName (see aiter_fp8bs_gemm_kernel_names())";
+            return hipErrorInvalidValue;
+        }
+        if(!gemm_mid_supports(p))
+        {
+            *why = "the mid_* kernels need operand matrices below 4 GiB";
+            return hipErrorInvalidValue;
+        }
+        return launch_gemm_mid(p, DT, a.split_k_log2, a.device_id, stream, tile);
+    }
     if(a.split_k_log2 > 0)
     {
-        *why = "splitK > 0 is only available with the decode_stream kernel (M <= 64)";
+        *why = "splitK > 0 is only available with the decode_stream and mid_* kernels";
         return hipErrorInvalidValue;
     }
     if(strcmp(name, "prefill_256x256") == 0)

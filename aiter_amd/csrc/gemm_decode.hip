@@ -729,6 +729,18 @@ hipError_t launch_mt(const DecodeParams& p, int rows, bool single, bool full, di
 
 } // namespace
 
+hipError_t gemm_split_workspace(int device_id, size_t partial_bytes, size_t n_tickets, hipStream_t stream,
+                                float** partial, uint32_t** tickets)
+{
+    Workspace* w = nullptr;
+    hipError_t e = ensure_workspace(device_id, partial_bytes, n_tickets, stream, &w);
+    if(e != hipSuccess)
+        return e;
+    *partial = w->partial;
+    *tickets = w->tickets;
+    return hipSuccess;
+}
+
 bool gemm_decode_supports(const GemmKernelParams& p)
 {
     return p.M >= 1 && p.M <= kDecodeMaxM && p.kblocks >= 1;

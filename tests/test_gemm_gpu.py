@@ -62,7 +62,8 @@ def test_config1_plumbing():
     assert np.all(np.abs(out.cpu().float().numpy() - o64) <= 2.0**-8 * np.abs(o64) + 1e-4)
 
 
-@pytest.mark.parametrize("kernel", [None, "tile_16x256", "tile_64x128", "tile_128x128", "prefill_256x256", "decode_stream"])
+@pytest.mark.parametrize("kernel", [None, "tile_16x256", "tile_64x128", "tile_128x128", "mid_64x64", "mid_64x128",
+                                    "mid_128x128", "prefill_256x256", "decode_stream"])
 @pytest.mark.parametrize(
     "m,n,k",
     [(1, 128, 128), (1, 2112, 512), (16, 256, 1024), (17, 384, 256), (64, 2112, 1024), (130, 520, 384), (257, 1000, 256)],
@@ -215,6 +216,22 @@ def test_decode_stream_more_than_64_rows(m, n, k, tuning):
     assert torch.equal(out.view(torch.int16), again.view(torch.int16))
     one = run_gpu(xq, wq, xs, ws, kernel="tile_128x128")
     assert (out.view(torch.int16) != one.view(torch.int16)).float().mean().item() < 0.02
+
+
+@pytest.mark.parametrize("m,n,k,splitk", [(128, 128, 128, 0), (200, 520, 1024, -1), (512, 2112, 7168, -1), (300, 1000, 2304, 2),
+                                            (1024, 4096, 1536, 0), (129, 130, 1024, 3), (256, 7168, 2048, -1)])
+@pytest.mark.parametrize("kernel", ["mid_64x64", "mid_64x128", "mid_128x128", "mid_auto"])
+def test_mid_kernel(kernel, m, n, k, splitk):
+    xq, wq, xs, ws = make_problem(m, n, k, seed=m + n + k + 2, outliers=0.01)
+    out = run_gpu(xq, wq, xs, ws, kernel=kernel, splitK=splitk)
+    assert_close_to_f64(out, xq, wq, xs, ws, f"{kernel} {m}x{n}x{k} splitK={splitk}")
+    again = run_gpu(xq, wq, xs, ws, kernel=kernel, splitK=splitk)
+    assert torch.equal(out.view(torch.int16), again.view(torch.int16))
+    tile = run_gpu(xq, wq, xs, ws, kernel="tile_128x128")
+    if splitk == 0:  # one K range: same products, same accumulation order as the generic tile kernel
+        assert torch.equal(out.view(torch.int16), tile.view(torch.int16))
+    else:
+        assert (out.view(torch.int16) != tile.view(torch.int16)).float().mean().item() < 0.02
 
 
 def test_decode_stream_rejects_more_than_512_rows():

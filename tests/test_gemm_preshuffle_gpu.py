@@ -48,7 +48,8 @@ def test_matches_oracle_and_plain_layout(m, n, k, form):
     assert (out.view(torch.int16) != plain.view(torch.int16)).float().mean().item() < 0.02
 
 
-@pytest.mark.parametrize("kernel", ["tile_16x256", "tile_64x128", "tile_128x128", "prefill_256x256", "decode_stream"])
+@pytest.mark.parametrize("kernel", ["tile_16x256", "tile_64x128", "tile_128x128", "mid_64x64", "mid_64x128", "mid_128x128", "prefill_256x256",
+                                    "decode_stream"])
 @pytest.mark.parametrize("m", [48, 272])
 def test_named_kernels(kernel, m):
     n, k = 1008, 1024
