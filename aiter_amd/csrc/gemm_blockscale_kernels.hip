@@ -13,6 +13,7 @@
 // one scalar per lane, xs[m,kb]*ws[nb,kb], and (b) its output 4 consecutive 16-bit values.
 #include "fp8bs_launch.h"
 #include "gemm_common.h"
+#include <cstdio>
 
 #include <string.h>
 
@@ -171,15 +172,16 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
     const char* name = (a.kernel_name && a.kernel_name[0]) ? a.kernel_name : nullptr;
     if(name == nullptr)
     {
-        // Up to 64 activation rows the weight-streaming kernel wins everywhere.  Above that, the
-        // 256x256 tiling once it gives at least half of the compute units a tile, and the
-        // 128x128 / 64x64 tiling in between (measured crossovers on the DeepSeek shapes).
+        // Up to 64 activation rows the weight-streaming kernel wins everywhere.  Above that,
+        // the 256x256 tiling or the mid_* tilings, whichever is modelled faster: a 256x256
+        // iteration over one K block takes about 1.8 us against 0.8 us for a quarter of the
+        // area, so it wins once its tiles cover enough of the chip (measured on the DeepSeek
+        // shapes: from about 128 tiles).
         const int64_t prefill_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
+        const float   prefill_us    = 12.f + (float)((prefill_tiles + 255) / 256) * (float)p.kblocks * 1.8f;
         if(p.M <= 64 && gemm_decode_supports(p))
             name = "decode_stream";
-        else if(prefill_tiles >= 128 && gemm_prefill_supports(p))
-            name = "prefill_256x256";
-        else if(gemm_mid_supports(p))
+        else if(gemm_mid_supports(p) && (!gemm_prefill_supports(p) || gemm_mid_estimate_us(p) < prefill_us))
             name = "mid_auto";
         else if(gemm_prefill_supports(p))
             name = "prefill_256x256";
@@ -205,12 +207,19 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
     }
     if(strncmp(name, "mid_", 4) == 0)
     {
-        const int tile = strcmp(name, "mid_128x128") == 0  ? 128
-                         : strcmp(name, "mid_64x128") == 0 ? 64128
-                         : strcmp(name, "mid_64x64") == 0  ? 64
-                         : strcmp(name, "mid_auto") == 0   ? 0
-                                                           : -1;
-        if(tile < 0)
+        // "mid_128x128" alone, or "mid_128x128:s=7" to pin the number of K ranges
+        const char* colon = strchr(name, ':');
+        const size_t len  = colon ? (size_t)(colon - name) : strlen(name);
+        auto is = [&](const char* s) { return strlen(s) == len && strncmp(name, s, len) == 0; };
+        const int tile = is("mid_128x128")  ? 128
+                         : is("mid_64x128") ? 64128
+                         : is("mid_64x64")  ? 64
+                         : is("mid_auto")   ? 0
+                                            : -1;
+        int splits = 0;
+        if(colon && (sscanf(colon, ":s=%d", &splits) != 1 || splits < 1 || splits > 64))
+            splits = -1;
+        if(tile < 0 || splits < 0)
         {
             *why = "unknown kernelName (see aiter_fp8bs_gemm_kernel_names())";
             return hipErrorInvalidValue;
@@ -220,7 +229,7 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
             *why = "the mid_* kernels need operand matrices below 4 GiB";
             return hipErrorInvalidValue;
         }
-        return launch_gemm_mid(p, DT, a.split_k_log2, a.device_id, stream, tile);
+        return launch_gemm_mid(p, DT, a.split_k_log2, a.device_id, stream, tile, splits);
     }
     if(a.split_k_log2 > 0)
     {

@@ -77,8 +77,10 @@ hipError_t launch_gemm_decode(const GemmKernelParams& p, In16 out_dtype, int spl
                               hipStream_t stream, const char* tuning = nullptr);
 bool       gemm_decode_supports(const GemmKernelParams& p);
 hipError_t launch_gemm_mid(const GemmKernelParams& p, In16 out_dtype, int split_k_log2, int device_id,
-                           hipStream_t stream, int tile = 0);
+                           hipStream_t stream, int tile = 0, int splits = 0);
 bool       gemm_mid_supports(const GemmKernelParams& p);
+// modelled duration (us) of the best mid_* tiling, for the choice between kernel families
+float      gemm_mid_estimate_us(const GemmKernelParams& p);
 // Per-device workspace for K split across workgroups (fp32 partial tiles + tickets that are zero
 // between launches), shared by the kernels that split K; grown on demand, kept for the life of
 // the process.  Calls that use it on one device must not overlap.

@@ -1,18 +1,16 @@
 // Mid-size block-scale FP8 GEMM: problems too tall for the weight-streaming kernel and too small
 // to cover the chip with 256x256 tiles.
 //
-// BM (m) x BN (n) output tile per workgroup, 128x128, 64x128 or 64x64, picked at launch so that
-// the tiles alone give every compute unit work: splitting K across workgroups instead costs an
-// fp32 round trip of the tile through memory, which measured far dearer than the extra operand
-// traffic of smaller tiles.  4 waves laid out 2 (n) x 2 (m).  Both operand slabs of a K block and
+// BM (m) x BN (n) output tile per workgroup, 128x128, 64x128 or 64x64, and a number of K ranges,
+// picked together at launch from a small cost model so that every compute unit has work.
+// 4 waves laid out 2 (n) x 2 (m).  Both operand slabs of a K block and
 // the block's x_scale column come in with direct global->LDS loads into a four-stage ring: three
 // K blocks are in flight while one is multiplied.  The 64x64 tile leaves room for two workgroups
 // per compute unit.
 //
-// K can still be split across workgroups (very few tiles, long K): fp32 partial tiles go to a
-// workspace (lane-major, 16-byte accesses that bypass the per-XCD L2) and the last workgroup to
-// finish a tile, found with an atomic ticket, adds them in split order, so results never depend
-// on timing.
+// K split across workgroups (few tiles, long K): each range's fp32 partial tile goes to a
+// workspace and a second, chip-wide launch adds the ranges in order and converts, so results never
+// depend on timing.
 //
 // The MFMAs of a K block and the FMAs that fold their products into the accumulators are an
 // explicit instruction stream, as in the 256x256 kernel: left to the compiler, every MFMA writes
@@ -35,9 +33,7 @@ struct MidParams
     int32_t   tiles_m, tiles_n;
     int32_t   splits, kb_per_split;
     int32_t   bf16_out;
-    float*    partial; // [splits][tiles][4 waves x TI*TJ tiles][64 lanes] x 4 fp32
-    uint32_t  partial_bytes;
-    uint32_t* tickets; // [tiles], zero between launches
+    float*    partial; // [splits][M][N] fp32
 };
 
 template <int BM, int BN>
@@ -81,6 +77,13 @@ __device__ __forceinline__ void fma4_asm(float (&acc)[4], const f32x4& product, 
     asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(acc[1]) : "v"(product[1]), "v"(s));
     asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(acc[2]) : "v"(product[2]), "v"(s));
     asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(acc[3]) : "v"(product[3]), "v"(s));
+}
+
+// 16-byte store that is written through to memory instead of lingering dirty in this XCD's L2:
+// the end of the kernel then has less to write back before the reduction launch can start
+__device__ __forceinline__ void store_through(float* dst, const f32x4& v)
+{
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
 }
 
 template <int BM, int BN, bool SHUF, int OCC>
@@ -332,51 +335,51 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
         return;
     }
 
-    // ---- K split across workgroups: park the partial tile set, take a ticket, last one in adds
-    // them up in split order.  The workgroups of one tile run on different XCDs, whose L2 caches
-    // are not coherent with each other, so every access to the exchanged data bypasses them (sc1)
-    // and the stores are waited for before the ticket is taken.
-    const __amdgpu_buffer_rsrc_t rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(p.partial, 0, (int)p.partial_bytes, 0x00020000);
-    constexpr int kCoherent = 16;
-    auto part_off = [&](int sp, int i, int j) -> uint32_t {
-        return (uint32_t)(((((size_t)sp * tiles + tile) * 4 + wave) * NQ + i * TJ + j) * 64 + lane) * 16u;
-    };
-#pragma unroll
-    for(int i = 0; i < TI; ++i)
-#pragma unroll
-        for(int j = 0; j < TJ; ++j)
-            __builtin_amdgcn_raw_buffer_store_b128(
-                u32x4{__float_as_uint(acc[i][j][0]), __float_as_uint(acc[i][j][1]), __float_as_uint(acc[i][j][2]),
-                      __float_as_uint(acc[i][j][3])},
-                rsrc,
-                                                   part_off(split, i, j), 0, kCoherent);
-    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0)); // the stores above have reached memory
-    __shared__ uint32_t s_ticket;
-    __syncthreads();
-    if(t == 0)
-        s_ticket = __hip_atomic_fetch_add(p.tickets + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if(s_ticket != (uint32_t)p.splits - 1)
-        return;
-    if(t == 0) // leave the ticket ready for the next launch
-        __hip_atomic_store(p.tickets + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // ---- K split across workgroups: this range's fp32 partial tile goes to the workspace,
+    // row-major [split][M][N]; the reduction kernel launched behind this one adds the ranges in
+    // order (results never depend on timing) and converts.  A second launch costs a few
+    // microseconds but spreads the sum over the whole chip: leaving it to the last workgroup of
+    // each tile serialises splits x tile bytes behind one compute unit's loads.
+    float* const part = p.partial + (size_t)split * (size_t)g.M * (size_t)g.N;
 #pragma unroll
     for(int j = 0; j < TJ; ++j)
 #pragma unroll
         for(int i = 0; i < TI; ++i)
         {
-            f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
-            for(int sp = 0; sp < p.splits; ++sp) // split order, whoever arrived last
-                s += __builtin_bit_cast(
-                    f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, part_off(sp, i, j), 0, kCoherent));
-            const float sum[4] = {s[0], s[1], s[2], s[3]};
-            store_tile(i, j, sum);
+            const int m = m0 + wm * (BM / 2) + j * 16 + l16;
+            const int n = n0 + wn * (BN / 2) + i * 16 + kg * 4;
+            if(m < g.M && n < g.N) // N % 4 == 0 on this path
+                store_through(part + (size_t)m * g.N + n, f32x4{acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]});
         }
 }
 
+// out[m][n .. n+3] = sum over the K ranges, in range order, of the fp32 partial tiles
+template <int SPLITS>
+__global__ __launch_bounds__(256) void gemm_mid_reduce_kernel(const float* __restrict__ partial,
+                                                              uint16_t* __restrict__ out, uint32_t quads,
+                                                              uint32_t splits, int bf16_out)
+{
+    const uint32_t q = blockIdx.x * 256u + threadIdx.x;
+    if(q >= quads)
+        return;
+    const f32x4* src = (const f32x4*)partial + q;
+    f32x4        v[SPLITS];
+#pragma unroll
+    for(int sp = 0; sp < SPLITS; ++sp)
+        v[sp] = src[(size_t)sp * quads];
+    f32x4 sum = v[0];
+#pragma unroll
+    for(int sp = 1; sp < SPLITS; ++sp)
+        sum += v[sp];
+    for(uint32_t sp = SPLITS; sp < splits; ++sp) // more ranges than the unrolled count
+        sum += src[(size_t)sp * quads];
+    const u32x2 o = bf16_out ? u32x2{pack2<In16::bf16>(sum[0], sum[1]), pack2<In16::bf16>(sum[2], sum[3])}
+                             : u32x2{pack2<In16::fp16>(sum[0], sum[1]), pack2<In16::fp16>(sum[2], sum[3])};
+    *((u32x2*)out + q) = o;
+}
+
 template <int BM, int BN>
-hipError_t launch_shape(MidParams& p, int split_k_log2, int device_id, hipStream_t stream)
+hipError_t launch_shape(MidParams& p, int split_k_log2, int want_splits, int device_id, hipStream_t stream)
 {
     using S = MidShape<BM, BN>;
     const GemmKernelParams& g = p.g;
@@ -385,15 +388,12 @@ hipError_t launch_shape(MidParams& p, int split_k_log2, int device_id, hipStream
     const int tiles = p.tiles_m * p.tiles_n;
 
     int splits = 1;
-    if(split_k_log2 >= 0)
+    if(want_splits > 0)
+        splits = want_splits;
+    else if(split_k_log2 >= 0)
         splits = 1 << split_k_log2;
-    else
-    {
-        // Splitting K costs an fp32 round trip of the tile through memory: taken only when even
-        // the smallest tile leaves most of the chip idle, and never below 8 K blocks per split.
-        while(tiles * splits * 2 <= 160 && g.kblocks / (splits * 2) >= 8)
-            splits *= 2;
-    }
+    if((g.N & 3) != 0 || ((uintptr_t)g.out & 7) != 0) // the reduction works on quads of n
+        splits = 1;
     if(splits > g.kblocks)
         splits = g.kblocks;
     p.kb_per_split = (g.kblocks + splits - 1) / splits;
@@ -402,13 +402,11 @@ hipError_t launch_shape(MidParams& p, int split_k_log2, int device_id, hipStream
 
     if(splits > 1)
     {
-        const size_t bytes = (size_t)splits * tiles * 4 * S::NQ * 64 * 16;
-        if(bytes >= ((size_t)1 << 31))
-            return hipErrorInvalidValue;
-        hipError_t e = gemm_split_workspace(device_id, bytes, (size_t)tiles, stream, &p.partial, &p.tickets);
+        const size_t bytes = (size_t)splits * (size_t)g.M * (size_t)g.N * 4;
+        uint32_t*    unused = nullptr;
+        hipError_t   e      = gemm_split_workspace(device_id, bytes, 1, stream, &p.partial, &unused);
         if(e != hipSuccess)
             return e;
-        p.partial_bytes = (uint32_t)bytes;
     }
 
     auto        kernel = g.w_shuffled ? gemm_mid_kernel<BM, BN, true, S::kOccupancy>
@@ -424,6 +422,21 @@ hipError_t launch_shape(MidParams& p, int split_k_log2, int device_id, hipStream
         raised[which][device_id] = true;
     }
     hipLaunchKernelGGL(kernel, dim3(tiles * splits), dim3(kThreads), S::kSmem, stream, p);
+    hipError_t e = hipGetLastError();
+    if(e != hipSuccess || splits == 1)
+        return e;
+    const uint32_t quads = (uint32_t)((size_t)g.M * (size_t)g.N / 4);
+    const dim3     rgrid((quads + 255) / 256);
+    switch(splits)
+    {
+    case 2: hipLaunchKernelGGL(gemm_mid_reduce_kernel<2>, rgrid, dim3(256), 0, stream, p.partial, g.out, quads, (uint32_t)splits, p.bf16_out); break;
+    case 3: hipLaunchKernelGGL(gemm_mid_reduce_kernel<3>, rgrid, dim3(256), 0, stream, p.partial, g.out, quads, (uint32_t)splits, p.bf16_out); break;
+    case 4: hipLaunchKernelGGL(gemm_mid_reduce_kernel<4>, rgrid, dim3(256), 0, stream, p.partial, g.out, quads, (uint32_t)splits, p.bf16_out); break;
+    case 5: hipLaunchKernelGGL(gemm_mid_reduce_kernel<5>, rgrid, dim3(256), 0, stream, p.partial, g.out, quads, (uint32_t)splits, p.bf16_out); break;
+    case 6: hipLaunchKernelGGL(gemm_mid_reduce_kernel<6>, rgrid, dim3(256), 0, stream, p.partial, g.out, quads, (uint32_t)splits, p.bf16_out); break;
+    case 7: hipLaunchKernelGGL(gemm_mid_reduce_kernel<7>, rgrid, dim3(256), 0, stream, p.partial, g.out, quads, (uint32_t)splits, p.bf16_out); break;
+    default: hipLaunchKernelGGL(gemm_mid_reduce_kernel<8>, rgrid, dim3(256), 0, stream, p.partial, g.out, quads, (uint32_t)splits, p.bf16_out); break;
+    }
     return hipGetLastError();
 }
 
@@ -436,27 +449,94 @@ bool gemm_mid_supports(const GemmKernelParams& p)
            (uint64_t)p.M * (uint64_t)p.lda < (1ull << 32) && (uint64_t)p.M * (uint64_t)p.kblocks < (1ull << 30);
 }
 
+// Rough duration (us) of one tiling on a 256-CU part, fitted to in-kernel timelines on the
+// DeepSeek-V3 projection shapes with the weights coming from HBM.  A launch costs a fixed share
+// (first wave running, first stage landing: about 2 us from HBM, output stores draining, end of
+// kernel) plus an iteration per K block whose cost is set by what a compute unit can pull in
+// (about 40 KB/us, so it hardly depends on how many workgroups run).  K ranges beyond the first
+// add the partial tiles' write-back and the reduction launch.  Only the order of the candidates
+// matters.
+struct MidPlan
+{
+    int   tile, splits;
+    float cost;
+};
+static MidPlan plan_cost(const GemmKernelParams& g, int tile, int splits)
+{
+    const int   bm = tile == 128 ? 128 : 64, bn = tile == 64 ? 64 : 128;
+    const int   occupancy = tile == 64 ? 2 : 1;
+    const float fixed     = tile == 64 ? 4.5f : tile == 64128 ? 5.7f : 6.9f;
+    const float iter0     = tile == 64 ? 0.56f : tile == 64128 ? 0.70f : 0.74f;
+    const float iter1     = tile == 64 ? 0.07f : tile == 64128 ? 0.05f : 0.06f;
+    const int   tiles     = ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
+    const int   wgs = tiles * splits, slots = 256 * occupancy;
+    const int   rounds    = (wgs + slots - 1) / slots;
+    const float per_cu    = (float)(wgs < slots ? wgs : slots) / 256.f;
+    const int   iters     = (g.kblocks + splits - 1) / splits;
+    float       cost      = fixed + (float)rounds * (float)iters * (iter0 + iter1 * per_cu) +
+                 (float)(rounds - 1) * (fixed - 2.4f);
+    if(splits > 1)
+    {
+        const float reduce = 1.7f + (float)splits * (float)g.M * (float)g.N * 4.f / 6.0e6f;
+        cost += 1.5f + (reduce < 4.8f ? 4.8f : reduce);
+    }
+    return MidPlan{tile, splits, cost};
+}
+static MidPlan best_plan(const GemmKernelParams& g, int tile)
+{
+    const int  tiles_to_try[3] = {128, 64128, 64};
+    const bool can_split       = (g.N & 3) == 0 && ((uintptr_t)g.out & 7) == 0;
+    MidPlan    best{0, 1, 1e30f};
+    for(int t : tiles_to_try)
+    {
+        if(tile != 0 && t != tile)
+            continue;
+        const int max_splits = can_split ? (g.kblocks / 4 < 16 ? g.kblocks / 4 : 16) : 1;
+        for(int sp = 1; sp <= (max_splits < 1 ? 1 : max_splits); ++sp)
+        {
+            const MidPlan c = plan_cost(g, t, sp);
+            if(c.cost < best.cost * 0.98f) // ties go to the earlier candidate (fewer ranges)
+                best = c;
+        }
+    }
+    return best;
+}
+
+float gemm_mid_estimate_us(const GemmKernelParams& g) { return best_plan(g, 0).cost; }
+
 // split_k_log2 < 0: choose.  tile: 0 = choose, else 128 (128x128), 64128 (64x128) or 64 (64x64).
+// splits > 0 pins the number of K ranges (any count, not only powers of two).
 hipError_t launch_gemm_mid(const GemmKernelParams& g, In16 out_dtype, int split_k_log2, int device_id,
-                           hipStream_t stream, int tile)
+                           hipStream_t stream, int tile, int splits)
 {
     MidParams p{};
     p.g        = g;
     p.bf16_out = out_dtype == In16::bf16 ? 1 : 0;
-    if(tile == 0)
+    if(tile != 0 && tile != 128 && tile != 64128 && tile != 64)
+        return hipErrorInvalidValue;
+    if(splits <= 0 && split_k_log2 >= 0)
+        splits = 1 << split_k_log2;
+    if(tile == 0 || splits <= 0)
     {
-        // 128x128 once that gives most compute units a workgroup, else 64x64 (measured: the
-        // iteration costs about the same for either tile, so few large tiles lose to many small
-        // ones until the chip is covered)
-        const int64_t big = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
-        tile              = big >= 160 ? 128 : 64;
+        MidPlan plan = splits > 0 ? MidPlan{0, splits, 0.f} : best_plan(g, tile);
+        if(splits > 0) // ranges pinned, tile free: best tile for that count
+        {
+            plan.cost = 1e30f;
+            for(int t : {128, 64128, 64})
+            {
+                const MidPlan c = plan_cost(g, t, splits);
+                if(c.cost < plan.cost)
+                    plan = c;
+            }
+        }
+        tile   = plan.tile;
+        splits = plan.splits;
     }
     switch(tile)
     {
-    case 128: return launch_shape<128, 128>(p, split_k_log2, device_id, stream);
-    case 64128: return launch_shape<64, 128>(p, split_k_log2, device_id, stream);
-    case 64: return launch_shape<64, 64>(p, split_k_log2, device_id, stream);
-    default: return hipErrorInvalidValue;
+    case 128: return launch_shape<128, 128>(p, -1, splits, device_id, stream);
+    case 64128: return launch_shape<64, 128>(p, -1, splits, device_id, stream);
+    default: return launch_shape<64, 64>(p, -1, splits, device_id, stream);
     }
 }
 

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the FP8 block-scale path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload quant|prefill|decode|decode9|fused]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload quant|prefill|decode|decode9|sweep|fused]
                     [--no-also] [--no-cpu]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
@@ -14,6 +14,8 @@ Workloads (BASELINE.json configs):
   decode   config 3  blockscale GEMM M=64 N=24576 K=1536 (the largest decode shape)
   decode9  config 3  all nine: M in {1,16,64} x (N,K) in {(7168,2048),(24576,1536),(2112,7168)};
                      weights rotate through 640 MB so that every call reads them from HBM
+  sweep    (beyond the configs) M in {128..4096} x four projection shapes, each beside the
+                     duration the reference's tuner recorded for it
   fused    config 5  RMSNorm + 1x128 quant on [2048,7168], then GEMM N=4096
 
 Timing uses HIP events recorded on the stream the kernels are launched on (torch's current
@@ -36,7 +38,7 @@ METRIC = "blockscale GEMM TFLOP/s (% FP8 MFMA peak); group-quant GB/s (% HBM pea
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 FP8_PEAK_TFLOPS = 5000.0       # MI355X dense FP8 MFMA
 # The reference's own tuner measurement for the prefill shape on gfx950 / 256 CUs
-# (aiter/configs/model_configs/a8w8_blockscale_tuned_gemm_ds_v3.csv:6382), quoted in BASELINE.md.
+# (aiter/configs/model_configs/a8w8_blockscale_tuned_gemm_ds_v3.csv:6382).
 REF_PREFILL_TFLOPS = 2108.5
 
 
@@ -45,7 +47,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="quant", choices=["quant", "prefill", "decode", "decode9", "fused", "copy"],
+    ap.add_argument("--workload", default="quant", choices=["quant", "prefill", "decode", "decode9", "sweep", "fused", "copy"],
                     help="'copy' is a plain 1 GiB device copy used to calibrate the rocprofv3 FETCH_SIZE / "
                     "WRITE_SIZE counters; it is not part of the path")
     ap.add_argument("--no-also", action="store_true", help="time only the primary workload")
@@ -193,6 +195,7 @@ class QuantWorkload:
 class GemmWorkload:
     layout = "plain"  # set from --layout before setup()
     rotate_mb = 640   # set from --rotate-mb before setup()
+    rotate_always = False
 
     def __init__(self, name, m, n, k, label):
         self.name, self.M, self.N, self.K, self.label = name, m, n, k, label
@@ -226,7 +229,7 @@ class GemmWorkload:
         if pre:
             self.wqs = [aiter_amd.shuffle_weight(w.view(torch.uint8)).view(w.dtype) for w in self.wqs]
         self.ws = pairs[0][1]
-        if m <= 64:
+        if m <= 64 or self.rotate_always:
             want = -(-self.rotate_mb * 1_000_000 // (n * k))
             self.wqs += [self.wqs[i % nbuf].clone() for i in range(max(0, want - nbuf))]
         self.weight_bytes_rotated = len(self.wqs) * n * k
@@ -421,7 +424,69 @@ class DecodeAllWorkload:
         return self.parts[-1].cpu_baseline(torch)
 
 
+# Durations (us) the reference's tuner recorded on gfx950 for these shapes
+# (aiter/configs/model_configs/a8w8_blockscale_tuned_gemm_ds_v3.csv, column "us").
+SWEEP_REFERENCE_US = {
+    (128, 7168, 2048): 9.4978, (256, 7168, 2048): 13.6951, (512, 7168, 2048): 20.7712,
+    (1024, 7168, 2048): 34.0461, (2048, 7168, 2048): 68.5722, (4096, 7168, 2048): 120.1982,
+    (128, 24576, 1536): 17.3757, (256, 24576, 1536): 27.2881, (512, 24576, 1536): 46.3688,
+    (1024, 24576, 1536): 84.1555, (2048, 24576, 1536): 153.4331, (4096, 24576, 1536): 282.6274,
+    (128, 2112, 7168): 21.1709, (256, 2112, 7168): 23.0603, (512, 2112, 7168): 32.0652,
+    (1024, 2112, 7168): 51.2969, (2048, 2112, 7168): 88.3043, (4096, 2112, 7168): 91.0323,
+    (128, 4096, 7168): 23.6181, (256, 4096, 7168): 24.9567, (512, 4096, 7168): 44.5905,
+    (1024, 4096, 7168): 63.9434, (2048, 4096, 7168): 114.7033, (4096, 4096, 7168): 209.3355,
+}
+
+
+class SweepWorkload:
+    """Token counts between decode and prefill (M = 128 ... 4096) on the four DeepSeek-V3 projection
+    shapes, each launch timed by graph replay with the weights cycled through --rotate-mb."""
+
+    name = "sweep"
+
+    def setup(self, torch, dev):
+        self.torch, self.dev = torch, dev
+        self.shapes = list(SWEEP_REFERENCE_US)
+        # the headline number of this workload is one shape; the table rides in per_shape
+        self.head = GemmWorkload("sweep", 1024, 4096, 7168, "sweep")
+        self.head.rotate_always = True
+        self.head.setup(torch, dev)
+
+    def step(self):
+        self.head.step()
+
+    def describe(self):
+        return {"workload": "blockscale GEMM, M = 128..4096 on (N,K) = (7168,2048), (24576,1536), (2112,7168), "
+                            "(4096,7168); headline value is (1024, 4096, 7168)",
+                "layout": GemmWorkload.layout, "kernel": "gemm_a8w8_blockscale (automatic kernel choice)"}
+
+    def result(self, sec):
+        tf = self.head.flops() / sec / 1e12
+        return tf, "TFLOP/s", {"bound": "mfma", "achieved": tf, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                               "frac": tf / FP8_PEAK_TFLOPS, "traffic": None}
+
+    def per_shape(self, torch, steps, warmup):
+        del self.head
+        out = []
+        for (m, n, k) in self.shapes:
+            torch.cuda.empty_cache()
+            w = GemmWorkload("sweep", m, n, k, "sweep")
+            w.rotate_always = True
+            w.setup(torch, self.dev)
+            s3 = time_launches(torch, w.step, steps, warmup)
+            ref = SWEEP_REFERENCE_US[(m, n, k)]
+            out.append({"M": m, "N": n, "K": k, "kernel_us": s3 * 1e6, "TFLOP/s": w.flops() / s3 / 1e12,
+                        "reference_tuned_us": ref, "reference_over_ours": ref / (s3 * 1e6)})
+            del w
+        return out
+
+    def cpu_baseline(self, torch):
+        return None
+
+
 def make_workload(name):
+    if name == "sweep":
+        return SweepWorkload()
     if name == "copy":
         return CopyCalibration()
     if name == "quant":
@@ -483,7 +548,7 @@ def main():
     }
     if args.workload == "prefill":
         line["vs_reference_tuned_csv"] = value / REF_PREFILL_TFLOPS
-    if args.workload == "decode9":
+    if args.workload in ("decode9", "sweep"):
         # shape after shape: steps + warmup launches each, in DECODE_SHAPES order
         line["per_shape"] = wl.per_shape(torch, args.steps, args.warmup)
         args.no_also = True

@@ -234,6 +234,23 @@ def test_mid_kernel(kernel, m, n, k, splitk):
         assert (out.view(torch.int16) != tile.view(torch.int16)).float().mean().item() < 0.02
 
 
+@pytest.mark.parametrize("name", ["mid_128x128:s=3", "mid_64x64:s=5", "mid_64x128:s=7", "mid_auto:s=2"])
+@pytest.mark.parametrize("m,n,k,dtype", [(200, 520, 2304, torch.bfloat16), (128, 2112, 7168, torch.float16)])
+def test_mid_kernel_pinned_k_ranges(name, m, n, k, dtype):
+    # any number of K ranges, not only powers of two; partial tiles summed in range order by a second launch
+    xq, wq, xs, ws = make_problem(m, n, k, seed=m + k, outliers=0.01)
+    out = run_gpu(xq, wq, xs, ws, dtype=dtype, kernel=name, splitK=-1)
+    assert_close_to_f64(out, xq, wq, xs, ws, f"{name} {m}x{n}x{k}")
+    again = run_gpu(xq, wq, xs, ws, dtype=dtype, kernel=name, splitK=-1)
+    assert torch.equal(out.view(torch.int16), again.view(torch.int16))
+
+
+def test_mid_kernel_rejects_malformed_range_count():
+    for name in ("mid_128x128:s=0", "mid_128x128:s=x", "mid_128x128:q=2", "mid_32x32"):
+        with pytest.raises(RuntimeError, match="unknown kernelName"):
+            run_gpu(*make_problem(128, 256, 256), kernel=name)
+
+
 def test_decode_stream_rejects_more_than_512_rows():
     with pytest.raises(RuntimeError, match="decode_stream handles"):
         run_gpu(*make_problem(513, 256, 256), kernel="decode_stream")
