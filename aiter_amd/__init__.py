@@ -18,6 +18,13 @@ from .gemm_op_a8w8 import (
     gemm_kernel_names,
 )
 from .shuffle import shuffle_weight
+from .fused_moe import (
+    ActivationType,
+    fmoe_fp8_blockscale_g1u1,
+    fused_moe_blockscale,
+    fused_topk,
+    moe_sorting,
+)
 from .quant import (
     dynamic_per_token_scaled_quant,
     get_hip_quant,
@@ -52,4 +59,9 @@ __all__ = [
     "add_rmsnorm_quant",
     "rmsnorm2d_fwd_with_dynamicquant",
     "rmsnorm2d_fwd_with_add_dynamicquant",
+    "ActivationType",
+    "fused_topk",
+    "moe_sorting",
+    "fmoe_fp8_blockscale_g1u1",
+    "fused_moe_blockscale",
 ]

@@ -18,7 +18,7 @@ LIB_NAME = "libaiter_fp8bs.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 
 SOURCES = ["abi.hip", "norm_quant_kernels.hip", "gemm_blockscale_kernels.hip", "gemm_prefill.hip", "gemm_decode.hip",
-           "gemm_mid.hip"]
+           "gemm_mid.hip", "moe_kernels.hip"]
 
 # -ffp-contract=off: the quantiser's rounding sequence must stay one IEEE operation per step.
 # The packed-fp32 target feature is switched off for device code on purpose; the host pass

@@ -7,6 +7,7 @@
 // (csrc/include/aiter_hip_common.h:538-552), work enqueued on the caller's stream.
 #include "../../include/aiter_fp8bs.h"
 #include "fp8bs_launch.h"
+#include "moe_launch.h"
 
 #include <exception>
 #include <sstream>
@@ -606,6 +607,306 @@ int gemm_a8w8_blockscale_bpreshuffle(aiter_tensor_t* XQ, aiter_tensor_t* WQ, ait
 {
     return gemm_blockscale_common("gemm_a8w8_blockscale_bpreshuffle", true, XQ, WQ, x_scale, w_scale, Out,
                                   -1, kernelName, stream);
+}
+
+// ---- mixture of experts -------------------------------------------------------------------
+
+int topk_softmax(aiter_tensor_t* topk_weights, aiter_tensor_t* topk_indices,
+                 aiter_tensor_t* token_expert_indices, aiter_tensor_t* gating_output, int need_renorm,
+                 aiter_stream_t stream)
+{
+    return guarded([&] {
+        const char* fn = "topk_softmax";
+        check_tensor(fn, topk_weights, "topk_weights");
+        check_tensor(fn, topk_indices, "topk_indices");
+        check_tensor(fn, gating_output, "gating_output");
+        if(token_expert_indices)
+            check_tensor(fn, token_expert_indices, "token_expert_indices");
+        same_device(fn, {topk_weights, topk_indices, token_expert_indices, gating_output});
+        if(gating_output->ndim != 2 || !contiguous(gating_output))
+            fail(fn, "gating_output must be a contiguous [tokens, experts] matrix");
+        const int64_t tokens = gating_output->shape[0], experts = gating_output->shape[1];
+        if(topk_weights->ndim != 2 || topk_indices->ndim != 2 || topk_weights->shape[0] != tokens ||
+           topk_indices->shape[0] != tokens || topk_weights->shape[1] != topk_indices->shape[1])
+            fail(fn, "topk_weights and topk_indices must both be [tokens, topk]");
+        const int64_t topk = topk_weights->shape[1];
+        if(experts < 1 || experts > 1024)
+            fail(fn, "experts = ", experts, " outside 1..1024");
+        if(topk < 1 || topk > 32 || topk > experts)
+            fail(fn, "topk = ", topk, " outside 1..min(32, experts)");
+        if(topk_weights->dtype_ != AITER_DTYPE_fp32 || topk_indices->dtype_ != AITER_DTYPE_i32)
+            fail(fn, "topk_weights must be fp32 and topk_indices int32");
+        if((topk > 1 && topk_weights->strides[1] != 1) || (topk > 1 && topk_indices->strides[1] != 1))
+            fail(fn, "topk_weights and topk_indices must be contiguous in their last dimension");
+        if(token_expert_indices &&
+           (token_expert_indices->dtype_ != AITER_DTYPE_i32 || !contiguous(token_expert_indices) ||
+            (int64_t)token_expert_indices->numel_ != tokens * topk))
+            fail(fn, "token_expert_indices must be contiguous int32 [tokens, topk]");
+        if(tokens >= (1LL << 24))
+            fail(fn, "too many tokens");
+        fp8bs::TopkSoftmaxArgs a{};
+        a.gating = gating_output->ptr;
+        switch(gating_output->dtype_)
+        {
+        case AITER_DTYPE_bf16: a.gating_dtype = 0; break;
+        case AITER_DTYPE_fp16: a.gating_dtype = 1; break;
+        case AITER_DTYPE_fp32: a.gating_dtype = 2; break;
+        default: fail(fn, "gating_output must be bf16, fp16 or fp32, got ", dtype_name(gating_output->dtype_));
+        }
+        a.weights   = (float*)topk_weights->ptr;
+        a.ids       = (int32_t*)topk_indices->ptr;
+        a.src_rows  = token_expert_indices ? (int32_t*)token_expert_indices->ptr : nullptr;
+        a.tokens    = (int32_t)tokens;
+        a.experts   = (int32_t)experts;
+        a.topk      = (int32_t)topk;
+        a.w_stride  = tokens > 1 ? topk_weights->strides[0] : topk;
+        a.id_stride = tokens > 1 ? topk_indices->strides[0] : topk;
+        a.renorm    = need_renorm != 0;
+        DeviceGuard guard(gating_output->device_id);
+        check_hip(fn, fp8bs::launch_topk_softmax(a, (hipStream_t)stream), nullptr);
+    });
+}
+
+int moe_sorting_fwd(aiter_tensor_t* topk_ids, aiter_tensor_t* topk_weights, aiter_tensor_t* sorted_token_ids,
+                    aiter_tensor_t* sorted_weights, aiter_tensor_t* sorted_expert_ids,
+                    aiter_tensor_t* num_valid_ids, aiter_tensor_t* moe_buf, int64_t num_experts,
+                    int64_t unit_size, aiter_tensor_t* local_expert_mask, aiter_tensor_t* num_local_tokens,
+                    int64_t dispatch_policy, aiter_stream_t stream)
+{
+    return guarded([&] {
+        const char* fn = "moe_sorting_fwd";
+        check_tensor(fn, topk_ids, "topk_ids");
+        check_tensor(fn, topk_weights, "topk_weights");
+        check_tensor(fn, sorted_token_ids, "sorted_token_ids");
+        check_tensor(fn, sorted_weights, "sorted_weights");
+        check_tensor(fn, sorted_expert_ids, "sorted_expert_ids");
+        check_tensor(fn, num_valid_ids, "num_valid_ids");
+        if(moe_buf)
+            check_tensor(fn, moe_buf, "moe_buf");
+        if(local_expert_mask)
+            check_tensor(fn, local_expert_mask, "local_expert_mask");
+        if(num_local_tokens)
+            check_tensor(fn, num_local_tokens, "num_local_tokens");
+        same_device(fn, {topk_ids, topk_weights, sorted_token_ids, sorted_weights, sorted_expert_ids, num_valid_ids,
+                         moe_buf, local_expert_mask, num_local_tokens});
+        (void)dispatch_policy; // a tuning hint of the reference's kernels
+        if(topk_ids->ndim != 2 || topk_weights->ndim != 2 || topk_ids->shape[0] != topk_weights->shape[0] ||
+           topk_ids->shape[1] != topk_weights->shape[1])
+            fail(fn, "topk_ids and topk_weights must both be [tokens, topk]");
+        const int64_t M = topk_ids->shape[0], topk = topk_ids->shape[1];
+        if(topk_ids->dtype_ != AITER_DTYPE_i32 || topk_weights->dtype_ != AITER_DTYPE_fp32)
+            fail(fn, "topk_ids must be int32 and topk_weights fp32");
+        if((topk > 1 && topk_ids->strides[1] != 1) || (topk > 1 && topk_weights->strides[1] != 1))
+            fail(fn, "topk_ids and topk_weights must be contiguous in their last dimension");
+        if(num_experts < 1 || num_experts > 1024)
+            fail(fn, "num_experts = ", num_experts, " outside 1..1024");
+        if(unit_size < 1 || unit_size > 1024)
+            fail(fn, "unit_size = ", unit_size, " outside 1..1024");
+        if(topk < 1 || topk > 255)
+            fail(fn, "topk = ", topk, " outside 1..255 (the sorted ids keep the slot in 8 bits)");
+        if(M >= (1LL << 24))
+            fail(fn, "tokens = ", M, " do not fit the 24 bits the sorted ids keep for them");
+        const int64_t max_padded = M * topk + num_experts * unit_size - topk;
+        const int64_t max_blocks = (max_padded + unit_size - 1) / unit_size;
+        if(sorted_token_ids->dtype_ != AITER_DTYPE_i32 || !contiguous(sorted_token_ids) ||
+           (int64_t)sorted_token_ids->numel_ < max_padded)
+            fail(fn, "sorted_token_ids must be contiguous int32 with at least ", max_padded, " elements");
+        if(sorted_weights->dtype_ != AITER_DTYPE_fp32 || !contiguous(sorted_weights) ||
+           (int64_t)sorted_weights->numel_ < max_padded)
+            fail(fn, "sorted_weights must be contiguous fp32 with at least ", max_padded, " elements");
+        if(sorted_expert_ids->dtype_ != AITER_DTYPE_i32 || !contiguous(sorted_expert_ids) ||
+           (int64_t)sorted_expert_ids->numel_ < max_blocks)
+            fail(fn, "sorted_expert_ids must be contiguous int32 with at least ", max_blocks, " elements");
+        if(num_valid_ids->dtype_ != AITER_DTYPE_i32 || num_valid_ids->numel_ < 2 || !contiguous(num_valid_ids))
+            fail(fn, "num_valid_ids must be contiguous int32 with 2 elements");
+        if(local_expert_mask && (local_expert_mask->dtype_ != AITER_DTYPE_i32 || !contiguous(local_expert_mask) ||
+                                 (int64_t)local_expert_mask->numel_ != num_experts))
+            fail(fn, "local_expert_mask must be contiguous int32 [num_experts]");
+        if(num_local_tokens && (num_local_tokens->dtype_ != AITER_DTYPE_i32 || num_local_tokens->numel_ < 1))
+            fail(fn, "num_local_tokens must be an int32 scalar on the device");
+        size_t buf_bytes = 0;
+        if(moe_buf && moe_buf->numel_)
+        {
+            if(!contiguous(moe_buf))
+                fail(fn, "moe_buf must be contiguous");
+            buf_bytes = moe_buf->numel_ * dtype_size(moe_buf->dtype_);
+            if(buf_bytes % 16 != 0)
+                fail(fn, "moe_buf must span a multiple of 16 bytes");
+            check_aligned(fn, moe_buf, "moe_buf", 16);
+        }
+        fp8bs::MoeSortArgs a{};
+        a.topk_ids          = (const int32_t*)topk_ids->ptr;
+        a.topk_weights      = (const float*)topk_weights->ptr;
+        a.expert_mask       = local_expert_mask ? (const int32_t*)local_expert_mask->ptr : nullptr;
+        a.num_local_tokens  = num_local_tokens ? (const int32_t*)num_local_tokens->ptr : nullptr;
+        a.sorted_ids        = (int32_t*)sorted_token_ids->ptr;
+        a.sorted_weights    = (float*)sorted_weights->ptr;
+        a.sorted_expert_ids = (int32_t*)sorted_expert_ids->ptr;
+        a.num_valid_ids     = (int32_t*)num_valid_ids->ptr;
+        a.moe_buf           = buf_bytes ? moe_buf->ptr : nullptr;
+        a.moe_buf_bytes     = buf_bytes;
+        a.M                 = (int32_t)M;
+        a.topk              = (int32_t)topk;
+        a.experts           = (int32_t)num_experts;
+        a.unit              = (int32_t)unit_size;
+        a.max_padded        = (int32_t)max_padded;
+        a.max_blocks        = (int32_t)max_blocks;
+        a.id_stride         = M > 1 ? topk_ids->strides[0] : topk;
+        a.w_stride          = M > 1 ? topk_weights->strides[0] : topk;
+        a.device_id         = topk_ids->device_id;
+        if(max_padded >= (1LL << 31))
+            fail(fn, "problem too large");
+        DeviceGuard guard(topk_ids->device_id);
+        check_hip(fn, fp8bs::launch_moe_sorting(a, (hipStream_t)stream), nullptr);
+    });
+}
+
+int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_tensor_t* gate, aiter_tensor_t* down,
+                             aiter_tensor_t* sorted_token_ids, aiter_tensor_t* sorted_weights,
+                             aiter_tensor_t* sorted_expert_ids, aiter_tensor_t* num_valid_ids, int64_t topk,
+                             aiter_tensor_t* input_scale, aiter_tensor_t* fc1_scale, aiter_tensor_t* fc2_scale,
+                             const char* kernel_name, int64_t fc_scale_blkn, int64_t fc_scale_blkk,
+                             aiter_tensor_t* fc2_smooth_scale, int64_t activation, int64_t block_size_M,
+                             aiter_stream_t stream)
+{
+    return guarded([&] {
+        const char* fn = "fmoe_fp8_blockscale_g1u1";
+        check_tensor(fn, out, "out");
+        check_tensor(fn, input, "input");
+        check_tensor(fn, gate, "gate");
+        check_tensor(fn, down, "down");
+        check_tensor(fn, sorted_token_ids, "sorted_token_ids");
+        check_tensor(fn, sorted_weights, "sorted_weights");
+        check_tensor(fn, sorted_expert_ids, "sorted_expert_ids");
+        check_tensor(fn, num_valid_ids, "num_valid_ids");
+        check_tensor(fn, fc1_scale, "fc1_scale");
+        check_tensor(fn, fc2_scale, "fc2_scale");
+        if(input_scale)
+            check_tensor(fn, input_scale, "input_scale");
+        same_device(fn, {out, input, gate, down, sorted_token_ids, sorted_weights, sorted_expert_ids, num_valid_ids,
+                         input_scale, fc1_scale, fc2_scale});
+        (void)kernel_name; // names the reference's tuned kernels; one implementation here
+        if(fc2_smooth_scale)
+            fail(fn, "fc2_smooth_scale is not supported");
+        if(fc_scale_blkn != 128 || fc_scale_blkk != 128)
+            fail(fn, "only 128 x 128 weight scale blocks are supported, got ", fc_scale_blkn, " x ", fc_scale_blkk);
+        if(block_size_M != 32)
+            fail(fn, "block_size_M must be 32, got ", block_size_M);
+        if(activation != 0 && activation != 1)
+            fail(fn, "activation must be 0 (silu) or 1 (gelu), got ", activation);
+        if(!is_f16_like(out->dtype_))
+            fail(fn, "out must be bf16 or fp16, got ", dtype_name(out->dtype_));
+        if(input->ndim != 2 || out->ndim != 2 || gate->ndim != 3 || down->ndim != 3)
+            fail(fn, "input/out must be 2-D [tokens, dim], gate/down 3-D [experts, n, k]");
+        const int64_t M = input->shape[0], dim = input->shape[1];
+        const int64_t E = gate->shape[0], inter = down->shape[2];
+        if(out->shape[0] != M || out->shape[1] != dim)
+            fail(fn, "out must be [", M, ",", dim, "]");
+        if(gate->shape[1] != 2 * inter || gate->shape[2] != dim)
+            fail(fn, "gate must be [experts, 2*inter_dim, dim] = [", E, ",", 2 * inter, ",", dim, "] (gate then up rows)");
+        if(down->shape[0] != E || down->shape[1] != dim)
+            fail(fn, "down must be [", E, ",", dim, ",", inter, "]");
+        if(!is_fp8_like(gate->dtype_) || !is_fp8_like(down->dtype_))
+            fail(fn, "gate and down must be fp8");
+        if(!contiguous(gate) || !contiguous(down))
+            fail(fn, "gate and down must be contiguous (pre-shuffled with layout (16,16))");
+        if(dim % 128 != 0 || inter % 128 != 0 || dim < 128 || inter < 128)
+            fail(fn, "dim = ", dim, " and inter_dim = ", inter, " must be positive multiples of 128");
+        if(dim % 256 != 0)
+            fail(fn, "dim = ", dim, " must be a multiple of 256");
+        if(topk < 1 || topk > 255)
+            fail(fn, "topk = ", topk, " outside 1..255");
+        if(M >= (1LL << 24) || E > 1024 || E < 1)
+            fail(fn, "tokens or experts out of range");
+        const int64_t kb1 = dim / 128, kb2 = inter / 128;
+        if(fc1_scale->dtype_ != AITER_DTYPE_fp32 || !contiguous(fc1_scale) ||
+           (int64_t)fc1_scale->numel_ != E * (2 * inter / 128) * kb1)
+            fail(fn, "fc1_scale must be contiguous fp32 with experts * (2*inter_dim/128) * (dim/128) = ",
+                 E * (2 * inter / 128) * kb1, " elements, got ", fc1_scale->numel_);
+        if(fc2_scale->dtype_ != AITER_DTYPE_fp32 || !contiguous(fc2_scale) ||
+           (int64_t)fc2_scale->numel_ != E * (dim / 128) * kb2)
+            fail(fn, "fc2_scale must be contiguous fp32 with experts * (dim/128) * (inter_dim/128) = ",
+                 E * (dim / 128) * kb2, " elements, got ", fc2_scale->numel_);
+        if(sorted_token_ids->dtype_ != AITER_DTYPE_i32 || sorted_expert_ids->dtype_ != AITER_DTYPE_i32 ||
+           num_valid_ids->dtype_ != AITER_DTYPE_i32 || sorted_weights->dtype_ != AITER_DTYPE_fp32)
+            fail(fn, "sorted_token_ids / sorted_expert_ids / num_valid_ids must be int32, sorted_weights fp32");
+        if(!contiguous(sorted_token_ids) || !contiguous(sorted_expert_ids) || !contiguous(sorted_weights) ||
+           num_valid_ids->numel_ < 1)
+            fail(fn, "the sorted arrays must be contiguous");
+        const int64_t max_blocks = (int64_t)sorted_expert_ids->numel_;
+        const int64_t max_padded = max_blocks * 32;
+        if((int64_t)sorted_token_ids->numel_ < max_padded - 31 || (int64_t)sorted_weights->numel_ < max_padded - 31)
+            fail(fn, "sorted_token_ids and sorted_weights must cover the ", max_blocks,
+                 " blocks of sorted_expert_ids");
+        // the kernels read whole blocks: the last block may only be addressed if it is backed
+        const int64_t backed = (int64_t)sorted_token_ids->numel_ < (int64_t)sorted_weights->numel_
+                                   ? (int64_t)sorted_token_ids->numel_
+                                   : (int64_t)sorted_weights->numel_;
+        const int64_t use_blocks = backed / 32 < max_blocks ? backed / 32 : max_blocks;
+        if(max_padded >= (1LL << 31) || max_padded * dim >= (1LL << 40))
+            fail(fn, "problem too large");
+
+        fp8bs::MoeArgs a{};
+        if(is_fp8_like(input->dtype_))
+        {
+            if(!input_scale)
+                fail(fn, "fp8 input needs input_scale");
+            if(input_scale->dtype_ != AITER_DTYPE_fp32 || !contiguous(input_scale) ||
+               (int64_t)input_scale->numel_ != M * kb1)
+                fail(fn, "input_scale must be contiguous fp32 [dim/128, tokens] = [", kb1, ",", M, "]");
+            if(input_scale->ndim == 2 && M > 1 && kb1 > 1 &&
+               !(input_scale->shape[0] == kb1 && input_scale->shape[1] == M))
+                fail(fn, "input_scale must be laid out [dim/128, tokens] (the transposed scale of the 1x128 quant)");
+            if(dim > 1 && input->strides[1] != 1)
+                fail(fn, "input must be contiguous in its last dimension");
+            a.lda = M > 1 ? input->strides[0] : dim;
+            if(a.lda < dim || a.lda % 16 != 0)
+                fail(fn, "input row stride must be >= dim and a multiple of 16");
+            check_aligned(fn, input, "input", 16);
+            a.xq = (const uint8_t*)input->ptr;
+            a.xs = (const float*)input_scale->ptr;
+        }
+        else if(is_f16_like(input->dtype_))
+        {
+            if(!contiguous(input))
+                fail(fn, "16-bit input must be contiguous");
+            check_aligned(fn, input, "input", 16);
+            a.x16       = input->ptr;
+            a.x16_dtype = in16_of(input->dtype_);
+            a.lda       = dim;
+        }
+        else
+            fail(fn, "input must be fp8 (with input_scale) or bf16/fp16, got ", dtype_name(input->dtype_));
+        if(dim > 1 && out->strides[1] != 1)
+            fail(fn, "out must be contiguous in its last dimension");
+        a.out_stride = M > 1 ? out->strides[0] : dim;
+        if(a.out_stride < dim || a.out_stride % 4 != 0)
+            fail(fn, "out row stride must be >= dim and a multiple of 4");
+        check_aligned(fn, out, "out", 8);
+        check_aligned(fn, gate, "gate", 16);
+        check_aligned(fn, down, "down", 16);
+        a.w1                = (const uint8_t*)gate->ptr;
+        a.w1_scale          = (const float*)fc1_scale->ptr;
+        a.w2                = (const uint8_t*)down->ptr;
+        a.w2_scale          = (const float*)fc2_scale->ptr;
+        a.sorted_ids        = (const int32_t*)sorted_token_ids->ptr;
+        a.sorted_weights    = (const float*)sorted_weights->ptr;
+        a.sorted_expert_ids = (const int32_t*)sorted_expert_ids->ptr;
+        a.num_valid         = (const int32_t*)num_valid_ids->ptr;
+        a.out               = out->ptr;
+        a.out_dtype         = in16_of(out->dtype_);
+        a.M                 = (int32_t)M;
+        a.dim               = (int32_t)dim;
+        a.inter             = (int32_t)inter;
+        a.experts           = (int32_t)E;
+        a.topk              = (int32_t)topk;
+        a.max_blocks        = (int32_t)use_blocks;
+        a.max_padded        = (int32_t)(use_blocks * 32);
+        a.activation        = (int32_t)activation;
+        a.device_id         = input->device_id;
+        DeviceGuard guard(input->device_id);
+        check_hip(fn, fp8bs::launch_fmoe_blockscale(a, (hipStream_t)stream), nullptr);
+    });
 }
 
 } // extern "C"

@@ -1,0 +1,832 @@
+// Block-scale FP8 mixture-of-experts: routing (softmax top-k), sorting of the routed
+// (token, expert) pairs into per-expert blocks, and the two grouped GEMMs of a gated expert
+//   h = act(x W_gate^T) * (x W_up^T),   y = h W_down^T,   out[token] += sum_k weight_k * y_k
+// with fp8 e4m3fn operands, 1x128 activation scales and 128x128 weight scales.
+//
+// Semantics follow aiter/fused_moe.py (moe_sorting :341-416, fused_topk :4058-4130),
+// op_tests/test_moe_sorting.py:44-105 (the sorted layout) and op_tests/test_moe_blockscale.py
+// (torch_moe_blockscale :19-101, the arithmetic; asm_moe_test :130-162, the call).
+//
+// Layout of the sorted arrays: per expert, its (token, slot) pairs in ascending (token, slot)
+// order as `slot << 24 | token`, padded with `topk << 24 | M` to a multiple of the block size;
+// sorted_expert_ids holds one expert id per block; num_valid_ids = {padded total, M}.
+//
+// The GEMMs stream pre-shuffled (16,16) weights straight into MFMA operand registers: a 16-row
+// tile's K block is 2 KiB of contiguous memory in fragment order, so no LDS staging is needed.
+// A workgroup owns one block of 32 sorted rows (one expert).  First GEMM: 32 gate + 32 up
+// columns, its 4 waves split K and add their partial tiles through LDS, the activation is applied
+// and the product written as bf16; the 1x128 quantiser of the dense path then turns it into fp8.
+// Second GEMM: 4 waves x 64 columns, K = inter_dim; rows are written per sorted slot (one writer
+// per element, fp32 while that fits 1 GiB, else bf16), and a last kernel adds each token's slots
+// in slot order, weighted, into `out`: deterministic, unlike atomic accumulation.
+#include "gemm_common.h"
+#include "moe_launch.h"
+
+namespace fp8bs {
+
+namespace {
+
+constexpr int kSortChunk = 4096; // (token, slot) pairs per workgroup of the large sort
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for(int o = 32; o > 0; o >>= 1)
+        v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for(int o = 32; o > 0; o >>= 1)
+        v += __shfl_xor(v, o);
+    return v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// softmax + top-k, one wave per token.  Ties go to the lower expert index.
+template <typename T>
+__global__ __launch_bounds__(256) void topk_softmax_kernel(const T* __restrict__ gating, float* __restrict__ weights,
+                                                           int32_t* __restrict__ ids, int32_t* __restrict__ src_rows,
+                                                           int32_t tokens, int32_t experts, int32_t topk,
+                                                           int64_t w_stride, int64_t id_stride, int renorm)
+{
+    constexpr int kMaxPerLane = 16; // experts <= 1024
+    const int     lane = threadIdx.x & 63;
+    const int     tok  = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if(tok >= tokens)
+        return;
+    const T* row = gating + (size_t)tok * experts;
+    float    v[kMaxPerLane];
+    float    mx = -INFINITY;
+#pragma unroll
+    for(int i = 0; i < kMaxPerLane; ++i)
+    {
+        const int e = i * 64 + lane;
+        v[i]        = e < experts ? (float)row[e] : -INFINITY;
+        mx          = fmaxf(mx, v[i]);
+    }
+    mx        = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for(int i = 0; i < kMaxPerLane; ++i)
+    {
+        v[i] = (i * 64 + lane) < experts ? expf(v[i] - mx) : -1.f; // -1: never selected
+        sum += v[i] > 0.f ? v[i] : 0.f;
+    }
+    sum               = wave_sum(sum);
+    const float inv   = 1.f / sum;
+    float       picked = 0.f, my_w = 0.f;
+    int         my_id = 0;
+    for(int k = 0; k < topk; ++k)
+    {
+        float best = -1.f;
+        int   bi   = 0x7fffffff;
+#pragma unroll
+        for(int i = 0; i < kMaxPerLane; ++i)
+            if(v[i] > best) // ascending i = ascending expert index within a lane
+            {
+                best = v[i];
+                bi   = i * 64 + lane;
+            }
+#pragma unroll
+        for(int o = 32; o > 0; o >>= 1)
+        {
+            const float ob = __shfl_xor(best, o);
+            const int   oi = __shfl_xor(bi, o);
+            if(ob > best || (ob == best && oi < bi))
+            {
+                best = ob;
+                bi   = oi;
+            }
+        }
+        if((bi & 63) == lane)
+        {
+#pragma unroll
+            for(int i = 0; i < kMaxPerLane; ++i)
+                if(i == (bi >> 6))
+                    v[i] = -1.f;
+        }
+        if(lane == k)
+        {
+            my_w  = best * inv;
+            my_id = bi;
+        }
+        picked += best * inv;
+    }
+    if(lane < topk)
+    {
+        weights[(size_t)tok * w_stride + lane] = renorm ? my_w / picked : my_w;
+        ids[(size_t)tok * id_stride + lane]    = my_id;
+        if(src_rows)
+            src_rows[(size_t)tok * topk + lane] = lane * tokens + tok;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Sorting.  Three launches: per-chunk histograms; one workgroup that turns them into per-chunk
+// write positions, block -> expert ids and the totals; a stable scatter in which thread e walks
+// the chunk (held in LDS) for expert e, so that pairs keep their (token, slot) order.
+struct SortParams
+{
+    const int32_t* topk_ids;     // [M][topk], row stride id_stride
+    const float*   topk_weights; // [M][topk], row stride w_stride
+    const int32_t* expert_mask;  // optional [experts], 0 = not local
+    const int32_t* num_local_tokens; // optional device scalar: rows of topk_ids to sort
+    int32_t*       sorted_ids;
+    float*         sorted_weights;
+    int32_t*       sorted_expert_ids;
+    int32_t*       num_valid_ids;
+    int32_t*       counts; // workspace [chunks][experts]: counts, then positions
+    int32_t*       expert_begin; // workspace [experts + 1]: start of each expert's padded run
+    int32_t        M, topk, experts, unit, chunks;
+    int32_t        max_padded, max_blocks;
+    int64_t        id_stride, w_stride;
+};
+
+__device__ __forceinline__ int32_t sort_rows(const SortParams& p)
+{
+    int32_t rows = p.M;
+    if(p.num_local_tokens)
+    {
+        const int32_t r = *p.num_local_tokens;
+        rows            = r < 0 ? 0 : (r < rows ? r : rows);
+    }
+    return rows;
+}
+
+__global__ __launch_bounds__(1024) void moe_sort_count_kernel(SortParams p)
+{
+    extern __shared__ int32_t hist[];
+    for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
+        hist[e] = 0;
+    __syncthreads();
+    const int64_t n = (int64_t)sort_rows(p) * p.topk;
+    const int64_t lo = (int64_t)blockIdx.x * kSortChunk;
+    for(int i = threadIdx.x; i < kSortChunk; i += blockDim.x)
+    {
+        const int64_t f = lo + i;
+        if(f >= n)
+            break;
+        const int32_t e = p.topk_ids[(f / p.topk) * p.id_stride + (f % p.topk)];
+        if(e >= 0 && e < p.experts)
+            atomicAdd(&hist[e], 1);
+    }
+    __syncthreads();
+    for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
+        p.counts[(size_t)blockIdx.x * p.experts + e] = hist[e];
+}
+
+__global__ __launch_bounds__(1024) void moe_sort_scan_kernel(SortParams p)
+{
+    extern __shared__ int32_t sh[]; // [experts] padded totals -> exclusive starts, [experts] local ids
+    int32_t* padded = sh;
+    int32_t* local  = sh + p.experts;
+    for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
+    {
+        int32_t run = 0;
+        for(int c = 0; c < p.chunks; ++c)
+        {
+            const int32_t n                       = p.counts[(size_t)c * p.experts + e];
+            p.counts[(size_t)c * p.experts + e] = run; // position inside the expert's run
+            run += n;
+        }
+        const bool masked = p.expert_mask && p.expert_mask[e] == 0;
+        padded[e]         = masked ? -1 : (run + p.unit - 1) / p.unit * p.unit;
+        // the unpadded count rides in expert_begin until the starts are known
+        p.expert_begin[e] = run;
+    }
+    __syncthreads();
+    if(threadIdx.x == 0)
+    {
+        int32_t at = 0, lid = 0;
+        for(int e = 0; e < p.experts; ++e)
+        {
+            const int32_t len = padded[e];
+            padded[e]         = len < 0 ? -1 : at;
+            local[e]          = lid;
+            if(len >= 0)
+            {
+                at += len;
+                ++lid;
+            }
+        }
+        p.num_valid_ids[0] = at;
+        p.num_valid_ids[1] = sort_rows(p);
+        sh[2 * p.experts]  = at;
+    }
+    __syncthreads();
+    const int32_t total = sh[2 * p.experts];
+    const int32_t pad_id = (p.topk << 24) | p.M;
+    for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
+    {
+        const int32_t begin = padded[e], count = p.expert_begin[e];
+        p.expert_begin[e]   = begin;
+        if(begin < 0)
+            continue;
+        const int32_t len = (count + p.unit - 1) / p.unit * p.unit;
+        for(int b = 0; b < len / p.unit; ++b)
+            p.sorted_expert_ids[begin / p.unit + b] = local[e];
+        for(int i = count; i < len; ++i)
+        {
+            p.sorted_ids[begin + i]     = pad_id;
+            p.sorted_weights[begin + i] = 0.f;
+        }
+    }
+    for(int b = total / p.unit + threadIdx.x; b < p.max_blocks; b += blockDim.x)
+        p.sorted_expert_ids[b] = -1;
+    for(int i = total + threadIdx.x; i < p.max_padded; i += blockDim.x)
+    {
+        p.sorted_ids[i]     = pad_id;
+        p.sorted_weights[i] = 0.f;
+    }
+}
+
+__global__ __launch_bounds__(1024) void moe_sort_scatter_kernel(SortParams p)
+{
+    __shared__ int32_t ids[kSortChunk];
+    const int64_t      n  = (int64_t)sort_rows(p) * p.topk;
+    const int64_t      lo = (int64_t)blockIdx.x * kSortChunk;
+    const int          cnt = (int)((n - lo) < kSortChunk ? (n - lo > 0 ? n - lo : 0) : kSortChunk);
+    for(int i = threadIdx.x; i < cnt; i += blockDim.x)
+    {
+        const int64_t f = lo + i;
+        ids[i]          = p.topk_ids[(f / p.topk) * p.id_stride + (f % p.topk)];
+    }
+    __syncthreads();
+    for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
+    {
+        const int32_t begin = p.expert_begin[e];
+        if(begin < 0)
+            continue;
+        int32_t at = begin + p.counts[(size_t)blockIdx.x * p.experts + e];
+        for(int i = 0; i < cnt; ++i)
+            if(ids[i] == e)
+            {
+                const int64_t f     = lo + i;
+                const int32_t token = (int32_t)(f / p.topk), slot = (int32_t)(f % p.topk);
+                p.sorted_ids[at]     = (slot << 24) | token;
+                p.sorted_weights[at] = p.topk_weights[(size_t)token * p.w_stride + slot];
+                ++at;
+            }
+    }
+}
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(u32x4* __restrict__ dst, size_t vecs)
+{
+    for(size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < vecs; i += (size_t)gridDim.x * 256)
+        dst[i] = u32x4{0u, 0u, 0u, 0u};
+}
+
+__global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* __restrict__ dst, size_t n, int32_t v)
+{
+    for(size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
+        dst[i] = v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// The two grouped GEMMs.
+struct MoeGemmParams
+{
+    const uint8_t* xq;   // first GEMM: [M][K] fp8 tokens (row stride lda); second: [slots][K] by sorted slot
+    const float*   xs;   // first: [K/128][M]; second: [slots][K/128]
+    const uint8_t* w;    // [experts][N][K] fp8, pre-shuffled (16,16) per expert
+    const float*   wsc;  // [experts][N/128][K/128]
+    const int32_t* sorted_ids;
+    const int32_t* sorted_expert_ids;
+    const int32_t* num_valid;
+    uint16_t*      out;  // first: [slots][inter] bf16; second: [slots][N] bf16 or fp32
+    int32_t        M, K, N, inter, kblocks, n_groups, max_blocks, experts, activation;
+    int32_t        out_f32; // second GEMM only: rows kept in fp32
+    int64_t        lda;
+};
+
+// fragment of a pre-shuffled weight tile's K block: 2 KiB, lane (l16, kg) takes the 16 bytes at
+// kg*512 + l16*16 and the 16 bytes 256 further on
+__device__ __forceinline__ i32x8 load_w_fragment(const uint8_t* tile_kb, int l16, int kg)
+{
+    const i32x4 lo = *(const i32x4*)(tile_kb + kg * 512 + l16 * 16);
+    const i32x4 hi = *(const i32x4*)(tile_kb + kg * 512 + 256 + l16 * 16);
+    return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+}
+// fragment of a row-major activation row's K block: 32 contiguous bytes at kg*32
+__device__ __forceinline__ i32x8 load_x_fragment(const uint8_t* row_kb, int kg)
+{
+    const i32x4 lo = *(const i32x4*)(row_kb + kg * 32);
+    const i32x4 hi = *(const i32x4*)(row_kb + kg * 32 + 16);
+    return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+}
+
+__device__ __forceinline__ float activate(float g, int activation)
+{
+    if(activation == 0) // silu
+        return g / (1.f + expf(-g));
+    return 0.5f * g * (1.f + erff(g * 0.70710678118654752f)); // gelu (erf form)
+}
+
+// First GEMM + activation.  Workgroup = (block of 32 sorted rows, group of 32 inter columns);
+// the 4 waves take every fourth K block each.  MFMA roles as in the dense kernels: weight rows
+// are the "A" operand, activation rows the "B" operand, so a lane ends up with 4 consecutive
+// columns of one row.
+__global__ __launch_bounds__(256) void moe_gate_up_kernel(MoeGemmParams p)
+{
+    __shared__ __attribute__((aligned(16))) float red[4][8][64][4]; // [wave][m tile * 4 + n tile][lane][c]
+    const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
+    if(blk * 32 >= p.num_valid[0])
+        return;
+    const int expert = p.sorted_expert_ids[blk];
+    if(expert < 0 || expert >= p.experts)
+        return;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
+
+    // rows of the two m tiles this lane feeds as the "B" operand
+    const uint8_t* xrow[2];
+    int            tok[2];
+#pragma unroll
+    for(int j = 0; j < 2; ++j)
+    {
+        const int id = p.sorted_ids[blk * 32 + j * 16 + l16] & 0xffffff;
+        tok[j]       = id < p.M ? id : 0; // padding rows compute on token 0 and are never read
+        xrow[j]      = p.xq + (size_t)tok[j] * p.lda;
+    }
+    // weight tiles: n tiles 0,1 = gate columns grp*32 .. +31, n tiles 2,3 = the matching up columns
+    const size_t   wexp = (size_t)expert * (size_t)p.N * (size_t)p.K;
+    const uint8_t* wt[4];
+#pragma unroll
+    for(int i = 0; i < 4; ++i)
+    {
+        const int row0 = (i < 2 ? 0 : p.inter) + grp * 32 + (i & 1) * 16;
+        wt[i]          = p.w + wexp + (size_t)(row0 >> 4) * 16 * (size_t)p.K;
+    }
+    const float* ws_gate = p.wsc + ((size_t)expert * (p.N / 128) + (grp * 32) / 128) * p.kblocks;
+    const float* ws_up   = p.wsc + ((size_t)expert * (p.N / 128) + (p.inter + grp * 32) / 128) * p.kblocks;
+
+    f32x4 acc[2][4];
+#pragma unroll
+    for(int j = 0; j < 2; ++j)
+#pragma unroll
+        for(int i = 0; i < 4; ++i)
+            acc[j][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    struct Operands
+    {
+        i32x8 w[4], x[2];
+        float xs[2], wg, wu;
+    };
+    auto fetch = [&](int kb, Operands& o) {
+#pragma unroll
+        for(int i = 0; i < 4; ++i)
+            o.w[i] = load_w_fragment(wt[i] + (size_t)kb * 2048, l16, kg);
+#pragma unroll
+        for(int j = 0; j < 2; ++j)
+        {
+            o.x[j]  = load_x_fragment(xrow[j] + (size_t)kb * 128, kg);
+            o.xs[j] = p.xs[(size_t)kb * p.M + tok[j]];
+        }
+        o.wg = ws_gate[kb];
+        o.wu = ws_up[kb];
+    };
+    auto multiply = [&](const Operands& o) {
+#pragma unroll
+        for(int j = 0; j < 2; ++j)
+#pragma unroll
+            for(int i = 0; i < 4; ++i)
+            {
+                const f32x4 prod = mfma_16x16x128_fp8(o.w[i], o.x[j], f32x4{0.f, 0.f, 0.f, 0.f});
+                const float s    = o.xs[j] * (i < 2 ? o.wg : o.wu);
+#pragma unroll
+                for(int c = 0; c < 4; ++c)
+                    acc[j][i][c] = __builtin_fmaf(prod[c], s, acc[j][i][c]);
+            }
+    };
+    // two operand sets, filled alternately: the next K block travels while this one is multiplied
+    Operands a, b;
+    int      kb = wave;
+    if(kb < p.kblocks)
+        fetch(kb, a);
+    while(kb < p.kblocks)
+    {
+        if(kb + 4 < p.kblocks)
+            fetch(kb + 4, b);
+        multiply(a);
+        kb += 4;
+        if(kb >= p.kblocks)
+            break;
+        if(kb + 4 < p.kblocks)
+            fetch(kb + 4, a);
+        multiply(b);
+        kb += 4;
+    }
+
+#pragma unroll
+    for(int j = 0; j < 2; ++j)
+#pragma unroll
+        for(int i = 0; i < 4; ++i)
+            *(f32x4*)red[wave][j * 4 + i][lane] = acc[j][i];
+    __syncthreads();
+    // wave w' finishes the pair (m tile w'>>1, gate tile w'&1 with up tile 2 + (w'&1))
+    const int j = wave >> 1, i = wave & 1;
+    f32x4     g = f32x4{0.f, 0.f, 0.f, 0.f}, u = g;
+#pragma unroll
+    for(int w = 0; w < 4; ++w) // wave order: the sum does not depend on timing
+    {
+        g += *(const f32x4*)red[w][j * 4 + i][lane];
+        u += *(const f32x4*)red[w][j * 4 + 2 + i][lane];
+    }
+    float h[4];
+#pragma unroll
+    for(int c = 0; c < 4; ++c)
+        h[c] = activate(g[c], p.activation) * u[c];
+    const int slot = blk * 32 + j * 16 + l16;
+    const int col  = grp * 32 + i * 16 + kg * 4;
+    *(u32x2*)(p.out + (size_t)slot * p.inter + col) =
+        u32x2{pack2<In16::bf16>(h[0], h[1]), pack2<In16::bf16>(h[2], h[3])};
+}
+
+// Second GEMM.  Workgroup = (block of 32 sorted rows, 256 output columns), wave = 64 columns.
+__global__ __launch_bounds__(256) void moe_down_kernel(MoeGemmParams p)
+{
+    const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
+    if(blk * 32 >= p.num_valid[0])
+        return;
+    const int expert = p.sorted_expert_ids[blk];
+    if(expert < 0 || expert >= p.experts)
+        return;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
+    const int n0 = grp * 256 + wave * 64;
+    if(n0 >= p.N)
+        return;
+    const uint8_t* xrow[2];
+    const float*   xsr[2];
+#pragma unroll
+    for(int j = 0; j < 2; ++j)
+    {
+        const size_t slot = (size_t)blk * 32 + j * 16 + l16;
+        xrow[j]           = p.xq + slot * p.lda;
+        xsr[j]            = p.xs + slot * p.kblocks;
+    }
+    const uint8_t* wt  = p.w + (size_t)expert * (size_t)p.N * (size_t)p.K + (size_t)(n0 >> 4) * 16 * (size_t)p.K;
+    const float*   wsr = p.wsc + ((size_t)expert * (p.N / 128) + n0 / 128) * p.kblocks;
+
+    f32x4 acc[2][4];
+#pragma unroll
+    for(int j = 0; j < 2; ++j)
+#pragma unroll
+        for(int i = 0; i < 4; ++i)
+            acc[j][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for(int kb = 0; kb < p.kblocks; ++kb)
+    {
+        i32x8 w[4], x[2];
+#pragma unroll
+        for(int i = 0; i < 4; ++i)
+            w[i] = load_w_fragment(wt + (size_t)i * 16 * (size_t)p.K + (size_t)kb * 2048, l16, kg);
+        float s[2];
+        const float wsv = wsr[kb];
+#pragma unroll
+        for(int j = 0; j < 2; ++j)
+        {
+            x[j] = load_x_fragment(xrow[j] + (size_t)kb * 128, kg);
+            s[j] = xsr[j][kb] * wsv;
+        }
+#pragma unroll
+        for(int j = 0; j < 2; ++j)
+#pragma unroll
+            for(int i = 0; i < 4; ++i)
+            {
+                const f32x4 prod = mfma_16x16x128_fp8(w[i], x[j], f32x4{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+                for(int c = 0; c < 4; ++c)
+                    acc[j][i][c] = __builtin_fmaf(prod[c], s[j], acc[j][i][c]);
+            }
+    }
+#pragma unroll
+    for(int j = 0; j < 2; ++j)
+#pragma unroll
+        for(int i = 0; i < 4; ++i)
+        {
+            const size_t slot = (size_t)blk * 32 + j * 16 + l16;
+            const int    col  = n0 + i * 16 + kg * 4;
+            if(p.out_f32)
+                *(f32x4*)((float*)p.out + slot * p.N + col) = acc[j][i];
+            else
+                *(u32x2*)(p.out + slot * p.N + col) = u32x2{pack2<In16::bf16>(acc[j][i][0], acc[j][i][1]),
+                                                            pack2<In16::bf16>(acc[j][i][2], acc[j][i][3])};
+        }
+}
+
+// where each (token, slot) pair sits in the sorted order (-1: not routed to a local expert)
+__global__ __launch_bounds__(256) void moe_invert_kernel(const int32_t* __restrict__ sorted_ids,
+                                                         const int32_t* __restrict__ num_valid,
+                                                         int32_t* __restrict__ where, int32_t M, int32_t topk,
+                                                         int32_t max_padded)
+{
+    const int32_t n = num_valid[0] < max_padded ? num_valid[0] : max_padded;
+    for(int32_t i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256)
+    {
+        const int32_t id = sorted_ids[i], token = id & 0xffffff, slot = (id >> 24) & 0xff;
+        if(token < M && slot < topk)
+            where[(size_t)token * topk + slot] = i;
+    }
+}
+
+// out[token] += sum over the token's slots, in slot order, of weight * y[sorted position]
+template <In16 DT, bool Y32>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const void* __restrict__ y, const float* __restrict__ sorted_weights,
+                                                          const int32_t* __restrict__ where, uint16_t* __restrict__ out,
+                                                          int32_t M, int32_t topk, int32_t dim, int64_t out_stride)
+{
+    const int quads = dim / 4;
+    const int token = blockIdx.x;
+    const int q     = blockIdx.y * 256 + threadIdx.x;
+    if(q >= quads)
+        return;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for(int k = 0; k < topk; ++k)
+    {
+        const int32_t at = where[(size_t)token * topk + k];
+        if(at < 0)
+            continue;
+        const float w = sorted_weights[at];
+        if constexpr(Y32)
+        {
+            const f32x4 v = *(const f32x4*)((const float*)y + (size_t)at * dim + (size_t)q * 4);
+#pragma unroll
+            for(int c = 0; c < 4; ++c)
+                acc[c] = __builtin_fmaf(w, v[c], acc[c]);
+        }
+        else
+        {
+            const u32x2 v = *(const u32x2*)((const uint16_t*)y + (size_t)at * dim + (size_t)q * 4);
+            acc[0] = __builtin_fmaf(w, __uint_as_float(v[0] << 16), acc[0]);
+            acc[1] = __builtin_fmaf(w, __uint_as_float(v[0] & 0xffff0000u), acc[1]);
+            acc[2] = __builtin_fmaf(w, __uint_as_float(v[1] << 16), acc[2]);
+            acc[3] = __builtin_fmaf(w, __uint_as_float(v[1] & 0xffff0000u), acc[3]);
+        }
+    }
+    uint16_t*   dst  = out + (size_t)token * out_stride + (size_t)q * 4;
+    const u32x2 prev = *(const u32x2*)dst;
+    float       o[4];
+    if constexpr(DT == In16::bf16)
+    {
+        o[0] = __uint_as_float(prev[0] << 16);
+        o[1] = __uint_as_float(prev[0] & 0xffff0000u);
+        o[2] = __uint_as_float(prev[1] << 16);
+        o[3] = __uint_as_float(prev[1] & 0xffff0000u);
+    }
+    else
+    {
+        o[0] = (float)__builtin_bit_cast(_Float16, (unsigned short)(prev[0] & 0xffffu));
+        o[1] = (float)__builtin_bit_cast(_Float16, (unsigned short)(prev[0] >> 16));
+        o[2] = (float)__builtin_bit_cast(_Float16, (unsigned short)(prev[1] & 0xffffu));
+        o[3] = (float)__builtin_bit_cast(_Float16, (unsigned short)(prev[1] >> 16));
+    }
+    *(u32x2*)dst = u32x2{pack2<DT>(o[0] + acc[0], o[1] + acc[1]), pack2<DT>(o[2] + acc[2], o[3] + acc[3])};
+}
+
+// per-device scratch, grown on demand and kept for the life of the process
+struct Scratch
+{
+    void*  ptr   = nullptr;
+    size_t bytes = 0;
+};
+Scratch g_scratch[64];
+
+hipError_t scratch_for(int device_id, size_t bytes, hipStream_t stream, uint8_t** out)
+{
+    if(device_id < 0 || device_id >= 64)
+        return hipErrorInvalidDevice;
+    Scratch& s = g_scratch[device_id];
+    if(s.bytes < bytes)
+    {
+        if(s.ptr)
+        {
+            // work already enqueued may still use the old buffer
+            hipError_t e = hipStreamSynchronize(stream);
+            if(e != hipSuccess)
+                return e;
+            e = hipFree(s.ptr);
+            if(e != hipSuccess)
+                return e;
+            s.ptr   = nullptr;
+            s.bytes = 0;
+        }
+        const size_t want = bytes + bytes / 4;
+        hipError_t   e    = hipMalloc(&s.ptr, want);
+        if(e != hipSuccess)
+            return e;
+        s.bytes = want;
+    }
+    *out = (uint8_t*)s.ptr;
+    return hipSuccess;
+}
+
+size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// The second GEMM's rows wait in memory for the per-token sum: in fp32 while that costs at most
+// 1 GiB (bf16 rounding of rows that largely cancel in the sum is then avoided), in bf16 beyond.
+bool rows_in_f32(const MoeArgs& a) { return (size_t)a.max_padded * a.dim * 4 <= ((size_t)1 << 30); }
+
+} // namespace
+
+hipError_t launch_topk_softmax(const TopkSoftmaxArgs& a, hipStream_t stream)
+{
+    if(a.tokens == 0)
+        return hipSuccess;
+    const dim3 grid((unsigned)((a.tokens + 3) / 4));
+    switch(a.gating_dtype)
+    {
+    case 0:
+        hipLaunchKernelGGL(topk_softmax_kernel<__bf16>, grid, dim3(256), 0, stream, (const __bf16*)a.gating, a.weights,
+                           a.ids, a.src_rows, a.tokens, a.experts, a.topk, a.w_stride, a.id_stride, a.renorm ? 1 : 0);
+        break;
+    case 1:
+        hipLaunchKernelGGL(topk_softmax_kernel<_Float16>, grid, dim3(256), 0, stream, (const _Float16*)a.gating,
+                           a.weights, a.ids, a.src_rows, a.tokens, a.experts, a.topk, a.w_stride, a.id_stride,
+                           a.renorm ? 1 : 0);
+        break;
+    default:
+        hipLaunchKernelGGL(topk_softmax_kernel<float>, grid, dim3(256), 0, stream, (const float*)a.gating, a.weights,
+                           a.ids, a.src_rows, a.tokens, a.experts, a.topk, a.w_stride, a.id_stride, a.renorm ? 1 : 0);
+        break;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_moe_sorting(const MoeSortArgs& a, hipStream_t stream)
+{
+    SortParams p{};
+    p.topk_ids          = a.topk_ids;
+    p.topk_weights      = a.topk_weights;
+    p.expert_mask       = a.expert_mask;
+    p.num_local_tokens  = a.num_local_tokens;
+    p.sorted_ids        = a.sorted_ids;
+    p.sorted_weights    = a.sorted_weights;
+    p.sorted_expert_ids = a.sorted_expert_ids;
+    p.num_valid_ids     = a.num_valid_ids;
+    p.M                 = a.M;
+    p.topk              = a.topk;
+    p.experts           = a.experts;
+    p.unit              = a.unit;
+    p.max_padded        = a.max_padded;
+    p.max_blocks        = a.max_blocks;
+    p.id_stride         = a.id_stride;
+    p.w_stride          = a.w_stride;
+    const int64_t n     = (int64_t)a.M * a.topk;
+    p.chunks            = (int32_t)((n + kSortChunk - 1) / kSortChunk);
+    if(p.chunks < 1)
+        p.chunks = 1;
+    uint8_t*     scratch = nullptr;
+    const size_t counts_bytes = align_up((size_t)p.chunks * a.experts * 4);
+    hipError_t   e = scratch_for(a.device_id, counts_bytes + align_up(((size_t)a.experts + 1) * 4), stream, &scratch);
+    if(e != hipSuccess)
+        return e;
+    p.counts       = (int32_t*)scratch;
+    p.expert_begin = (int32_t*)(scratch + counts_bytes);
+
+    if(a.moe_buf && a.moe_buf_bytes)
+    {
+        const size_t vecs = a.moe_buf_bytes / 16;
+        unsigned     g    = (unsigned)((vecs + 255) / 256);
+        g                 = g > 4096 ? 4096 : (g < 1 ? 1 : g);
+        hipLaunchKernelGGL(fill_zero_kernel, dim3(g), dim3(256), 0, stream, (u32x4*)a.moe_buf, vecs);
+    }
+    hipLaunchKernelGGL(moe_sort_count_kernel, dim3(p.chunks), dim3(1024), (size_t)a.experts * 4, stream, p);
+    hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(1), dim3(1024), ((size_t)a.experts * 2 + 1) * 4, stream, p);
+    hipLaunchKernelGGL(moe_sort_scatter_kernel, dim3(p.chunks), dim3(1024), 0, stream, p);
+    return hipGetLastError();
+}
+
+size_t moe_workspace_bytes(const MoeArgs& a)
+{
+    const size_t slots = (size_t)a.max_padded;
+    size_t       b     = 0;
+    b += align_up(slots * a.inter * 2);          // activation product, bf16
+    b += align_up(slots * a.inter);              // the same as fp8
+    b += align_up(slots * (a.inter / 128) * 4);  // its scales
+    b += align_up(slots * a.dim * (rows_in_f32(a) ? 4 : 2)); // second GEMM's rows
+    b += align_up((size_t)a.M * a.topk * 4);     // sorted position of each (token, slot)
+    if(a.x16)
+    {
+        b += align_up((size_t)a.M * a.dim);             // quantised tokens
+        b += align_up((size_t)a.M * (a.dim / 128) * 4); // their scales
+    }
+    return b;
+}
+
+hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
+{
+    if(a.M == 0 || a.max_padded == 0)
+        return hipSuccess;
+    uint8_t*   ws = nullptr;
+    hipError_t e  = scratch_for(a.device_id, moe_workspace_bytes(a), stream, &ws);
+    if(e != hipSuccess)
+        return e;
+    const size_t slots = (size_t)a.max_padded;
+    uint16_t*    h16   = (uint16_t*)ws;
+    ws += align_up(slots * a.inter * 2);
+    uint8_t* hq = ws;
+    ws += align_up(slots * a.inter);
+    float* hs = (float*)ws;
+    ws += align_up(slots * (a.inter / 128) * 4);
+    const bool y32 = rows_in_f32(a);
+    uint16_t*  y   = (uint16_t*)ws;
+    ws += align_up(slots * a.dim * (y32 ? 4 : 2));
+    int32_t* where = (int32_t*)ws;
+    ws += align_up((size_t)a.M * a.topk * 4);
+
+    const uint8_t* xq = a.xq;
+    const float*   xs = a.xs;
+    if(a.x16) // 16-bit tokens: quantise them 1x128 first, scales transposed
+    {
+        uint8_t* q = ws;
+        ws += align_up((size_t)a.M * a.dim);
+        float* s = (float*)ws;
+        QuantArgs qa{};
+        qa.x               = a.x16;
+        qa.y               = q;
+        qa.scale           = s;
+        qa.rows            = a.M;
+        qa.groups_per_row  = a.dim / 128;
+        qa.group           = 128;
+        qa.transpose_scale = true;
+        qa.num_rows        = nullptr;
+        qa.num_rows_factor = 1;
+        qa.dtype           = a.x16_dtype;
+        e                  = launch_group_quant(qa, stream);
+        if(e != hipSuccess)
+            return e;
+        xq = q;
+        xs = s;
+    }
+
+    {
+        const size_t n = (size_t)a.M * a.topk;
+        unsigned     g = (unsigned)((n + 255) / 256);
+        g              = g > 2048 ? 2048 : g;
+        hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, stream, where, n, -1);
+        unsigned g2 = (unsigned)((slots + 255) / 256);
+        g2          = g2 > 2048 ? 2048 : g2;
+        hipLaunchKernelGGL(moe_invert_kernel, dim3(g2), dim3(256), 0, stream, a.sorted_ids, a.num_valid, where, a.M,
+                           a.topk, a.max_padded);
+    }
+
+    MoeGemmParams p{};
+    p.xq                = xq;
+    p.xs                = xs;
+    p.w                 = a.w1;
+    p.wsc               = a.w1_scale;
+    p.sorted_ids        = a.sorted_ids;
+    p.sorted_expert_ids = a.sorted_expert_ids;
+    p.num_valid         = a.num_valid;
+    p.out               = h16;
+    p.M                 = a.M;
+    p.K                 = a.dim;
+    p.N                 = 2 * a.inter;
+    p.inter             = a.inter;
+    p.kblocks           = a.dim / 128;
+    p.n_groups          = a.inter / 32;
+    p.max_blocks        = a.max_blocks;
+    p.experts           = a.experts;
+    p.activation        = a.activation;
+    p.lda               = a.x16 ? a.dim : a.lda;
+    hipLaunchKernelGGL(moe_gate_up_kernel, dim3((unsigned)((size_t)a.max_blocks * p.n_groups)), dim3(256), 0, stream, p);
+
+    QuantArgs qa{};
+    qa.x               = h16;
+    qa.y               = hq;
+    qa.scale           = hs;
+    qa.rows            = (int64_t)slots;
+    qa.groups_per_row  = a.inter / 128;
+    qa.group           = 128;
+    qa.transpose_scale = false;
+    qa.num_rows        = a.num_valid; // only the rows that exist
+    qa.num_rows_factor = 1;
+    qa.dtype           = In16::bf16;
+    e                  = launch_group_quant(qa, stream);
+    if(e != hipSuccess)
+        return e;
+
+    MoeGemmParams d = p;
+    d.xq            = hq;
+    d.xs            = hs;
+    d.w             = a.w2;
+    d.wsc           = a.w2_scale;
+    d.out           = y;
+    d.K             = a.inter;
+    d.N             = a.dim;
+    d.kblocks       = a.inter / 128;
+    d.n_groups      = (a.dim + 255) / 256;
+    d.lda           = a.inter;
+    d.out_f32       = y32 ? 1 : 0;
+    hipLaunchKernelGGL(moe_down_kernel, dim3((unsigned)((size_t)a.max_blocks * d.n_groups)), dim3(256), 0, stream, d);
+
+    const dim3 cgrid((unsigned)a.M, (unsigned)((a.dim / 4 + 255) / 256));
+    auto combine = a.out_dtype == In16::bf16
+                       ? (y32 ? moe_combine_kernel<In16::bf16, true> : moe_combine_kernel<In16::bf16, false>)
+                       : (y32 ? moe_combine_kernel<In16::fp16, true> : moe_combine_kernel<In16::fp16, false>);
+    hipLaunchKernelGGL(combine, cgrid, dim3(256), 0, stream, (const void*)y, a.sorted_weights, where,
+                       (uint16_t*)a.out, a.M, a.topk, a.dim, a.out_stride);
+    return hipGetLastError();
+}
+
+} // namespace fp8bs

@@ -1,0 +1,62 @@
+// Internal interface between the C-ABI entry points and the mixture-of-experts launchers.
+#pragma once
+
+#include "fp8bs_launch.h"
+
+namespace fp8bs {
+
+struct TopkSoftmaxArgs
+{
+    const void* gating; // [tokens][experts], contiguous
+    int         gating_dtype; // 0 bf16, 1 fp16, 2 fp32
+    float*      weights; // [tokens][topk], row stride w_stride
+    int32_t*    ids;     // [tokens][topk], row stride id_stride
+    int32_t*    src_rows; // optional [tokens][topk]: slot * tokens + token
+    int32_t     tokens, experts, topk;
+    int64_t     w_stride, id_stride;
+    bool        renorm;
+};
+hipError_t launch_topk_softmax(const TopkSoftmaxArgs& a, hipStream_t stream);
+
+struct MoeSortArgs
+{
+    const int32_t* topk_ids;
+    const float*   topk_weights;
+    const int32_t* expert_mask;      // optional [experts]
+    const int32_t* num_local_tokens; // optional device scalar
+    int32_t*       sorted_ids;        // [max_padded]
+    float*         sorted_weights;    // [max_padded]
+    int32_t*       sorted_expert_ids; // [max_blocks]
+    int32_t*       num_valid_ids;     // [2]
+    void*          moe_buf;           // zeroed (may be null)
+    size_t         moe_buf_bytes;     // multiple of 16
+    int32_t        M, topk, experts, unit, max_padded, max_blocks;
+    int64_t        id_stride, w_stride;
+    int            device_id;
+};
+hipError_t launch_moe_sorting(const MoeSortArgs& a, hipStream_t stream);
+
+struct MoeArgs
+{
+    const uint8_t* xq;  // [M][dim] fp8 (row stride lda), or null when x16 is given
+    const float*   xs;  // [dim/128][M]
+    const void*    x16; // [M][dim] bf16/fp16 contiguous: quantised inside
+    In16           x16_dtype;
+    const uint8_t* w1;       // [experts][2*inter][dim] fp8, shuffled (16,16)
+    const float*   w1_scale; // [experts][2*inter/128][dim/128]
+    const uint8_t* w2;       // [experts][dim][inter] fp8, shuffled (16,16)
+    const float*   w2_scale; // [experts][dim/128][inter/128]
+    const int32_t* sorted_ids;
+    const float*   sorted_weights;
+    const int32_t* sorted_expert_ids;
+    const int32_t* num_valid;
+    void*          out; // [M][dim] 16-bit, row stride out_stride; accumulated into
+    In16           out_dtype;
+    int32_t        M, dim, inter, experts, topk, max_padded, max_blocks;
+    int32_t        activation; // 0 silu, 1 gelu
+    int64_t        lda, out_stride;
+    int            device_id;
+};
+hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream);
+
+} // namespace fp8bs

@@ -175,6 +175,68 @@ int gemm_a8w8_blockscale_bpreshuffle(aiter_tensor_t* XQ, aiter_tensor_t* WQ, ait
  * csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale_instance.py:73-117). */
 const char* aiter_fp8bs_gemm_kernel_names(void);
 
+/*
+ * ---- block-scale mixture of experts (gated experts, fp8 e4m3fn, 1x128 / 128x128 scales) ----
+ *
+ * Softmax over the experts, top-k, optional renormalisation of the k weights.
+ * Replaces aiter::topk_softmax as bound by aiter/ops/moe_op.py:29-66 (used by fused_topk,
+ * aiter/fused_moe.py:4058-4130).
+ *   topk_weights fp32 [tokens, topk]; topk_indices int32 [tokens, topk] (rows may be strided);
+ *   token_expert_indices optional int32 [tokens, topk] (slot * tokens + token);
+ *   gating_output bf16|fp16|fp32 [tokens, experts] contiguous, experts <= 1024, topk <= 32.
+ * Ties go to the lower expert index.
+ */
+int topk_softmax(aiter_tensor_t* topk_weights, aiter_tensor_t* topk_indices,
+                 aiter_tensor_t* token_expert_indices, aiter_tensor_t* gating_output, int need_renorm,
+                 aiter_stream_t stream);
+
+/*
+ * Sort the routed (token, slot) pairs by expert into blocks of unit_size rows and zero moe_buf.
+ * Replaces moe_sorting_fwd, csrc/include/moe_sorting.h:6-17 as bound by
+ * aiter/ops/moe_sorting.py:11-25; layout as in op_tests/test_moe_sorting.py:44-105:
+ *   sorted_token_ids  int32 [tokens*topk + num_experts*unit_size - topk]: per local expert its
+ *                     pairs as (slot << 24 | token), ascending, padded with (topk << 24 | tokens)
+ *   sorted_weights    fp32, same length: the pairs' routing weights
+ *   sorted_expert_ids int32 [ceil(that length / unit_size)]: local expert id per block, -1 beyond
+ *   num_valid_ids     int32 [2]: {padded total, tokens sorted}
+ *   moe_buf           optional, any dtype, contiguous: set to zero
+ *   local_expert_mask optional int32 [num_experts]: experts with 0 are skipped and the others
+ *                     renumbered; num_local_tokens optional int32 device scalar: only that many
+ *                     rows of topk_ids take part.  dispatch_policy is accepted and ignored.
+ */
+int moe_sorting_fwd(aiter_tensor_t* topk_ids, aiter_tensor_t* topk_weights, aiter_tensor_t* sorted_token_ids,
+                    aiter_tensor_t* sorted_weights, aiter_tensor_t* sorted_expert_ids,
+                    aiter_tensor_t* num_valid_ids, aiter_tensor_t* moe_buf, int64_t num_experts,
+                    int64_t unit_size, aiter_tensor_t* local_expert_mask, aiter_tensor_t* num_local_tokens,
+                    int64_t dispatch_policy, aiter_stream_t stream);
+
+/*
+ * Gated experts on sorted tokens: out[token] += sum_k weight_k * down_e(act(gate_e x) * up_e x).
+ * Replaces fmoe_fp8_blockscale_g1u1, csrc/py_itfs_cu/asm_fmoe.cu:893-958 as bound by
+ * aiter/ops/moe_op.py:224-244 and called by op_tests/test_moe_blockscale.py:130-162.
+ *   out    bf16|fp16 [tokens, dim], accumulated into (moe_sorting_fwd zeroes it)
+ *   input  fp8 [tokens, dim] with input_scale fp32 [dim/128, tokens] (the transposed scales of
+ *          the 1x128 quant), or bf16|fp16 [tokens, dim] with input_scale NULL (quantised inside)
+ *   gate   fp8 [experts, 2*inter_dim, dim]: gate rows then up rows, each expert pre-shuffled
+ *          with layout (16,16) (aiter/ops/shuffle.py:192-205); fc1_scale fp32
+ *          [experts, 2*inter_dim/128 * dim/128]
+ *   down   fp8 [experts, dim, inter_dim], pre-shuffled likewise; fc2_scale fp32
+ *          [experts, dim/128 * inter_dim/128]
+ *   the four sorted arrays as moe_sorting_fwd writes them with unit_size 32
+ *   activation 0 = silu, 1 = gelu; fc_scale_blkn = fc_scale_blkk = 128; block_size_M = 32;
+ *   fc2_smooth_scale must be NULL; kernel_name is accepted and ignored.
+ * The product of the first GEMM is quantised 1x128 to fp8 for the second.  Each token's k
+ * contributions are added in slot order: results do not depend on timing.  Scratch memory is
+ * allocated by the library on first use and grown on demand.
+ */
+int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_tensor_t* gate, aiter_tensor_t* down,
+                             aiter_tensor_t* sorted_token_ids, aiter_tensor_t* sorted_weights,
+                             aiter_tensor_t* sorted_expert_ids, aiter_tensor_t* num_valid_ids, int64_t topk,
+                             aiter_tensor_t* input_scale, aiter_tensor_t* fc1_scale, aiter_tensor_t* fc2_scale,
+                             const char* kernel_name, int64_t fc_scale_blkn, int64_t fc_scale_blkk,
+                             aiter_tensor_t* fc2_smooth_scale, int64_t activation, int64_t block_size_M,
+                             aiter_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -128,3 +128,101 @@ def make_activation(m, k, seed=0, outlier_frac=0.0, outlier_gain=50.0):
 def make_weight(n, k, seed=1, std=0.02):
     g = torch.Generator().manual_seed(seed)
     return (torch.randn(n, k, generator=g) * std).bfloat16()
+
+
+# ---------------------------------------------------------------------------------------------
+# mixture of experts
+
+
+def fused_topk_ref(gating_output: torch.Tensor, topk: int, renormalize: bool):
+    """What aiter/fused_moe.py:4058-4130 asks of topk_softmax: softmax over the experts in fp32,
+    the k largest (ties to the lower expert index), optionally renormalised to sum 1."""
+    probs = torch.softmax(gating_output.to(torch.float32), dim=-1)
+    # stable descending sort = ties to the lower index
+    order = torch.sort(probs, dim=-1, descending=True, stable=True).indices[:, :topk]
+    weights = torch.gather(probs, 1, order)
+    if renormalize:
+        weights = weights / weights.sum(dim=-1, keepdim=True)
+    return weights, order.to(torch.int32)
+
+
+def moe_sorting_ref(topk_ids, topk_weights, num_experts, block_size=32, expert_mask=None, num_local_tokens=None):
+    """op_tests/test_moe_sorting.py:44-105 (run_torch_moe_sorting).
+
+    Returns (sorted_ids, sorted_weights, sorted_expert_ids, num_tokens_post_pad); entries of
+    sorted_weights that the reference leaves uninitialised are returned as NaN."""
+    m, topk = topk_ids.shape
+    max_num_tokens_padded = topk_ids.numel() + num_experts * block_size - topk
+    max_num_m_blocks = (max_num_tokens_padded + block_size - 1) // block_size
+    init_val = topk << 24 | m
+    sorted_ids = torch.full((max_num_tokens_padded,), init_val, dtype=torch.int32)
+    sorted_weights = torch.full((max_num_tokens_padded,), float("nan"), dtype=torch.float32)
+    sorted_expert_ids = torch.full((max_num_m_blocks,), -1, dtype=torch.int32)
+    if num_local_tokens is not None:
+        topk_ids = topk_ids[: int(num_local_tokens)]
+    begin = 0
+    blk = 0
+    skipped = 0
+    for e in range(num_experts):
+        if expert_mask is not None and int(expert_mask[e]) == 0:
+            skipped += 1
+            continue
+        token_id, topk_id = torch.where(topk_ids == e)
+        n = token_id.numel()
+        nblk = (n + block_size - 1) // block_size
+        sorted_ids[begin : begin + n] = (topk_id << 24 | token_id).to(torch.int32)
+        sorted_weights[begin : begin + n] = topk_weights[token_id, topk_id]
+        begin += nblk * block_size
+        sorted_expert_ids[blk : blk + nblk] = e - skipped
+        blk += nblk
+    post_pad = torch.tensor([begin, topk_ids.shape[0]], dtype=torch.int32)
+    return sorted_ids, sorted_weights, sorted_expert_ids, post_pad
+
+
+def moe_blockscale_ref(a_q, w1_q, w2_q, topk_weights, topk_ids, a_scale, fc1_scale, fc2_scale,
+                       block=(128, 128), activation="silu", expert_mask=None, compute=torch.float32,
+                       a2_quant=False):
+    """op_tests/test_moe_blockscale.py:19-101 (torch_moe_blockscale), g1u1 case.
+
+    a2_quant=True adds what the reference's kernels do between the two GEMMs and its stage-wise
+    oracles model (aiter/fused_moe.py:3330-3337 quant_func on the first stage's 16-bit output,
+    torch_moe_stage2 :3732-3745): the activation product is rounded to bf16, quantised 1x128 to
+    fp8 by the torch definition, and dequantised for the second GEMM.
+
+    a_q [tokens, dim] fp8 with a_scale [tokens, dim/128]; w1_q [E, 2*inter, dim] (gate rows then
+    up rows) with fc1_scale [E, (2*inter/128)*(dim/128)]; w2_q [E, dim, inter] with fc2_scale
+    [E, (dim/128)*(inter/128)].  Everything is dequantised to `compute` and evaluated expert by
+    expert; the result is returned in `compute` (the reference casts to the model dtype)."""
+    blk_n, blk_k = block
+    tokens, topk = topk_ids.shape
+    E, dim, inter = w2_q.shape
+    x = a_q.to(compute).view(tokens, -1, blk_k) * a_scale.to(compute).unsqueeze(-1)
+    x = x.view(tokens, dim)
+    s1 = fc1_scale.to(compute).view(E, 2 * inter // blk_n, dim // blk_k)
+    s1 = s1.repeat_interleave(blk_n, dim=1).repeat_interleave(blk_k, dim=2)
+    s2 = fc2_scale.to(compute).view(E, dim // blk_n, inter // blk_k)
+    s2 = s2.repeat_interleave(blk_n, dim=1).repeat_interleave(blk_k, dim=2)
+    ids = topk_ids.to(torch.int64)
+    if expert_mask is not None:
+        local = expert_mask.to(torch.int64).cumsum(0) - 1
+        local[expert_mask == 0] = -1
+        ids = local[ids]
+    out = torch.zeros(tokens, topk, dim, dtype=compute)
+    for e in range(E):
+        mask = ids == e
+        if not mask.any():
+            continue
+        w1 = w1_q[e].to(compute) * s1[e]
+        w2 = w2_q[e].to(compute) * s2[e]
+        t_idx, k_idx = torch.where(mask)
+        act_in = x[t_idx] @ w1.t()
+        gate, up = act_in.split([inter, inter], dim=-1)
+        if activation == "silu":
+            act = F.silu(gate) * up
+        else:
+            act = F.gelu(gate) * up
+        if a2_quant:
+            q, sc = per_1x128_quant(act.to(torch.bfloat16), group=blk_k)
+            act = (q.to(compute).view(act.shape[0], -1, blk_k) * sc.to(compute).unsqueeze(-1)).view(act.shape)
+        out[t_idx, k_idx] = act @ w2.t()
+    return (out * topk_weights.to(compute).view(tokens, topk, 1)).sum(dim=1)
