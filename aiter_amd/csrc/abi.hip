@@ -9,6 +9,8 @@
 #include "fp8bs_launch.h"
 #include "moe_launch.h"
 
+#include <cstdlib>
+#include <cstring>
 #include <exception>
 #include <sstream>
 #include <stdexcept>
@@ -785,7 +787,6 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
             check_tensor(fn, input_scale, "input_scale");
         same_device(fn, {out, input, gate, down, sorted_token_ids, sorted_weights, sorted_expert_ids, num_valid_ids,
                          input_scale, fc1_scale, fc2_scale});
-        (void)kernel_name; // names the reference's tuned kernels; one implementation here
         if(fc2_smooth_scale)
             fail(fn, "fc2_smooth_scale is not supported");
         if(fc_scale_blkn != 128 || fc_scale_blkk != 128)
@@ -903,6 +904,11 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
         a.max_blocks        = (int32_t)use_blocks;
         a.max_padded        = (int32_t)(use_blocks * 32);
         a.activation        = (int32_t)activation;
+        // the reference's names pick among its tuned kernels; here "nt=1|2|4" pins the first GEMM's
+        // columns per workgroup and anything else means choose
+        a.gate_tiles = 0;
+        if(kernel_name && strncmp(kernel_name, "nt=", 3) == 0)
+            a.gate_tiles = atoi(kernel_name + 3);
         a.device_id         = input->device_id;
         DeviceGuard guard(input->device_id);
         check_hip(fn, fp8bs::launch_fmoe_blockscale(a, (hipStream_t)stream), nullptr);

@@ -242,9 +242,45 @@ __global__ __launch_bounds__(1024) void moe_sort_scan_kernel(SortParams p)
     }
 }
 
+
+// Stable scatter of one chunk of (token, slot) pairs held in LDS, by one wave: 64 pairs at a time,
+// a pair's rank among the earlier pairs of its expert comes from ballots over the bits of the
+// expert id, and `running[e]` (LDS) carries the expert's fill level from one step to the next.
+__device__ __forceinline__ void scatter_chunk(const SortParams& p, const int32_t* ids, const float* wts,
+                                              const int32_t* begin, int32_t* running, int cnt, int64_t first)
+{
+    const int lane = threadIdx.x & 63;
+    for(int base = 0; base < cnt; base += 64)
+    {
+        const int  i  = base + lane;
+        const int  e  = i < cnt ? ids[i] : -1;
+        const bool in = e >= 0 && e < p.experts && begin[e] >= 0;
+        uint64_t   same = __ballot(in);
+#pragma unroll
+        for(int b = 0; b < 10; ++b)
+        {
+            const uint64_t bal = __ballot((e >> b) & 1);
+            same &= ((e >> b) & 1) ? bal : ~bal;
+        }
+        if(in)
+        {
+            const int     rank = __popcll(same & ((1ull << lane) - 1ull));
+            const int     n    = __popcll(same);
+            const int32_t fill = running[e];
+            const int32_t at   = begin[e] + fill + rank;
+            const int64_t f    = first + i;
+            p.sorted_ids[at]     = ((int32_t)(f % p.topk) << 24) | (int32_t)(f / p.topk);
+            p.sorted_weights[at] = wts[i];
+            if(rank == n - 1)
+                running[e] = fill + n;
+        }
+    }
+}
+
 __global__ __launch_bounds__(1024) void moe_sort_scatter_kernel(SortParams p)
 {
     __shared__ int32_t ids[kSortChunk];
+    __shared__ float   wts[kSortChunk];
     const int64_t      n  = (int64_t)sort_rows(p) * p.topk;
     const int64_t      lo = (int64_t)blockIdx.x * kSortChunk;
     const int          cnt = (int)((n - lo) < kSortChunk ? (n - lo > 0 ? n - lo : 0) : kSortChunk);
@@ -252,23 +288,106 @@ __global__ __launch_bounds__(1024) void moe_sort_scatter_kernel(SortParams p)
     {
         const int64_t f = lo + i;
         ids[i]          = p.topk_ids[(f / p.topk) * p.id_stride + (f % p.topk)];
+        wts[i]          = p.topk_weights[(f / p.topk) * p.w_stride + (f % p.topk)];
+    }
+    __shared__ int32_t begin[1024], running[1024];
+    for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
+    {
+        begin[e]   = p.expert_begin[e];
+        running[e] = p.counts[(size_t)blockIdx.x * p.experts + e];
+    }
+    __syncthreads();
+    if(threadIdx.x < 64)
+        scatter_chunk(p, ids, wts, begin, running, cnt, lo);
+}
+
+// All of it in one workgroup, for up to kSortChunk pairs (the decode regime): histogram in LDS,
+// a serial scan over the experts, then thread e walks the pairs for expert e.
+__global__ __launch_bounds__(1024) void moe_sort_single_kernel(SortParams p)
+{
+    __shared__ int32_t ids[kSortChunk];
+    __shared__ float   wts[kSortChunk];
+    __shared__ int32_t count[1024], begin[1024], local[1024];
+    __shared__ int32_t s_total;
+    const int rows = sort_rows(p);
+    const int cnt  = rows * p.topk; // <= kSortChunk, checked at launch
+    for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
+        count[e] = 0;
+    __syncthreads();
+    for(int i = threadIdx.x; i < cnt; i += blockDim.x)
+    {
+        const int     r = i / p.topk, k = i - r * p.topk;
+        const int32_t e = p.topk_ids[(size_t)r * p.id_stride + k];
+        ids[i]          = e;
+        wts[i]          = p.topk_weights[(size_t)r * p.w_stride + k];
+        if(e >= 0 && e < p.experts)
+            atomicAdd(&count[e], 1);
+    }
+    __syncthreads();
+    {
+        // exclusive scan over the experts of (padded length, 1 if local), one expert per thread
+        const int  e      = threadIdx.x;
+        const bool live   = e < p.experts && !(p.expert_mask && p.expert_mask[e] == 0);
+        const int  len    = live ? (count[e] + p.unit - 1) / p.unit * p.unit : 0;
+        int64_t    packed = ((int64_t)(live ? 1 : 0) << 40) | (int64_t)len;
+        const int64_t mine = packed;
+#pragma unroll
+        for(int o = 1; o < 64; o <<= 1)
+        {
+            const int64_t up = __shfl_up(packed, o);
+            if((threadIdx.x & 63) >= o)
+                packed += up;
+        }
+        __shared__ int64_t wave_total[16];
+        if((threadIdx.x & 63) == 63)
+            wave_total[threadIdx.x >> 6] = packed;
+        __syncthreads();
+        int64_t base = 0;
+        for(int w = 0; w < (int)(threadIdx.x >> 6); ++w)
+            base += wave_total[w];
+        const int64_t excl = base + packed - mine;
+        if(e < p.experts)
+        {
+            begin[e] = live ? (int32_t)(excl & 0xffffffffffll) : -1;
+            local[e] = (int32_t)(excl >> 40);
+        }
+        if(threadIdx.x == 1023)
+        {
+            const int32_t at   = (int32_t)((base + packed) & 0xffffffffffll);
+            s_total            = at;
+            p.num_valid_ids[0] = at;
+            p.num_valid_ids[1] = rows;
+        }
+    }
+    __syncthreads();
+    const int32_t total  = s_total;
+    const int32_t pad_id = (p.topk << 24) | p.M;
+    for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
+    {
+        const int32_t b0 = begin[e];
+        if(b0 < 0)
+            continue;
+        const int32_t len = (count[e] + p.unit - 1) / p.unit * p.unit;
+        for(int b = 0; b < len / p.unit; ++b)
+            p.sorted_expert_ids[b0 / p.unit + b] = local[e];
+        for(int32_t at = b0 + count[e]; at < b0 + len; ++at)
+        {
+            p.sorted_ids[at]     = pad_id;
+            p.sorted_weights[at] = 0.f;
+        }
     }
     __syncthreads();
     for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
+        local[e] = 0; // from here on: the expert's fill level
+    __syncthreads();
+    if(threadIdx.x < 64)
+        scatter_chunk(p, ids, wts, begin, local, cnt, 0);
+    for(int b = total / p.unit + threadIdx.x; b < p.max_blocks; b += blockDim.x)
+        p.sorted_expert_ids[b] = -1;
+    for(int i = total + threadIdx.x; i < p.max_padded; i += blockDim.x)
     {
-        const int32_t begin = p.expert_begin[e];
-        if(begin < 0)
-            continue;
-        int32_t at = begin + p.counts[(size_t)blockIdx.x * p.experts + e];
-        for(int i = 0; i < cnt; ++i)
-            if(ids[i] == e)
-            {
-                const int64_t f     = lo + i;
-                const int32_t token = (int32_t)(f / p.topk), slot = (int32_t)(f % p.topk);
-                p.sorted_ids[at]     = (slot << 24) | token;
-                p.sorted_weights[at] = p.topk_weights[(size_t)token * p.w_stride + slot];
-                ++at;
-            }
+        p.sorted_ids[i]     = pad_id;
+        p.sorted_weights[i] = 0.f;
     }
 }
 
@@ -298,6 +417,8 @@ struct MoeGemmParams
     uint16_t*      out;  // first: [slots][inter] bf16; second: [slots][N] bf16 or fp32
     int32_t        M, K, N, inter, kblocks, n_groups, max_blocks, experts, activation;
     int32_t        out_f32; // second GEMM only: rows kept in fp32
+    int32_t        topk;
+    int32_t*       where;   // first GEMM only: [M][topk] sorted position of each (token, slot) pair
     int64_t        lda;
 };
 
@@ -324,127 +445,231 @@ __device__ __forceinline__ float activate(float g, int activation)
     return 0.5f * g * (1.f + erff(g * 0.70710678118654752f)); // gelu (erf form)
 }
 
-// First GEMM + activation.  Workgroup = (block of 32 sorted rows, group of 32 inter columns);
-// the 4 waves take every fourth K block each.  MFMA roles as in the dense kernels: weight rows
-// are the "A" operand, activation rows the "B" operand, so a lane ends up with 4 consecutive
-// columns of one row.
+// First GEMM + activation.  Workgroup = (block of 32 sorted rows, NT x 16 inter columns): NT
+// gate tiles and the NT matching up tiles; NT is picked at launch (small units when few (expert,
+// block) pairs exist, so that the last units to finish do not set the kernel's duration; wide
+// units otherwise, which re-read the activations less often).  The 4 waves take every fourth K
+// block each and add their partial tiles through LDS in wave order.  One operand set per wave:
+// several workgroups share a compute unit and cover each other's load latency.  A block whose
+// second half is padding (the usual case when few tokens are routed) multiplies one 16-row tile
+// only.  MFMA roles as in the dense kernels: weight rows are the "A" operand, activation rows
+// the "B" operand, so a lane ends up with 4 consecutive columns of one row.
+template <int MT, int NT>
+__device__ __forceinline__ void gate_up_body(const MoeGemmParams& p, float* red, int blk, int grp, int expert)
+{
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
+    const uint8_t* xrow[MT];
+    const float*   xsr[MT];
+#pragma unroll
+    for(int j = 0; j < MT; ++j)
+    {
+        const int id  = p.sorted_ids[blk * 32 + j * 16 + l16] & 0xffffff;
+        const int tok = id < p.M ? id : 0; // padding rows compute on token 0 and are never read
+        xrow[j]       = p.xq + (size_t)tok * p.lda;
+        xsr[j]        = p.xs + tok;
+    }
+    const size_t   tile_stride = (size_t)16 * (size_t)p.K;
+    const size_t   wexp = (size_t)expert * (size_t)p.N * (size_t)p.K;
+    const uint8_t* wg   = p.w + wexp + (size_t)(grp * NT) * tile_stride;
+    const uint8_t* wu   = p.w + wexp + (size_t)((p.inter >> 4) + grp * NT) * tile_stride;
+    const float*   ws_gate = p.wsc + ((size_t)expert * (p.N / 128) + (grp * NT * 16) / 128) * p.kblocks;
+    const float*   ws_up   = p.wsc + ((size_t)expert * (p.N / 128) + (p.inter + grp * NT * 16) / 128) * p.kblocks;
+
+    f32x4 acc[MT][2 * NT];
+#pragma unroll
+    for(int j = 0; j < MT; ++j)
+#pragma unroll
+        for(int i = 0; i < 2 * NT; ++i)
+            acc[j][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for(int kb = wave; kb < p.kblocks; kb += 4)
+    {
+        i32x8 w[2 * NT], x[MT];
+        float xs[MT];
+#pragma unroll
+        for(int i = 0; i < NT; ++i)
+        {
+            w[i]      = load_w_fragment(wg + i * tile_stride + (size_t)kb * 2048, l16, kg);
+            w[NT + i] = load_w_fragment(wu + i * tile_stride + (size_t)kb * 2048, l16, kg);
+        }
+#pragma unroll
+        for(int j = 0; j < MT; ++j)
+        {
+            x[j]  = load_x_fragment(xrow[j] + (size_t)kb * 128, kg);
+            xs[j] = xsr[j][(size_t)kb * p.M];
+        }
+        const float sg = ws_gate[kb], su = ws_up[kb];
+#pragma unroll
+        for(int j = 0; j < MT; ++j)
+#pragma unroll
+            for(int i = 0; i < 2 * NT; ++i)
+            {
+                const f32x4 prod = mfma_16x16x128_fp8(w[i], x[j], f32x4{0.f, 0.f, 0.f, 0.f});
+                const float sc   = xs[j] * (i < NT ? sg : su);
+#pragma unroll
+                for(int c = 0; c < 4; ++c)
+                    acc[j][i][c] = __builtin_fmaf(prod[c], sc, acc[j][i][c]);
+            }
+    }
+
+    // red[wave][n tile][lane][c], one m tile at a time
+#pragma unroll
+    for(int j = 0; j < MT; ++j)
+    {
+        if(j > 0)
+            __syncthreads();
+#pragma unroll
+        for(int i = 0; i < 2 * NT; ++i)
+            *(f32x4*)(red + (((size_t)wave * (2 * NT) + i) * 64 + lane) * 4) = acc[j][i];
+        __syncthreads();
+        if(wave < NT) // wave i finishes the pair (gate tile i, up tile NT + i)
+        {
+            const int i = wave;
+            f32x4     g = f32x4{0.f, 0.f, 0.f, 0.f}, u = g;
+#pragma unroll
+            for(int w = 0; w < 4; ++w) // wave order: the sum does not depend on timing
+            {
+                g += *(const f32x4*)(red + (((size_t)w * (2 * NT) + i) * 64 + lane) * 4);
+                u += *(const f32x4*)(red + (((size_t)w * (2 * NT) + NT + i) * 64 + lane) * 4);
+            }
+            float h[4];
+#pragma unroll
+            for(int c = 0; c < 4; ++c)
+                h[c] = activate(g[c], p.activation) * u[c];
+            const int slot = blk * 32 + j * 16 + l16;
+            const int col  = (grp * NT + i) * 16 + kg * 4;
+            *(u32x2*)(p.out + (size_t)slot * p.inter + col) =
+                u32x2{pack2<In16::bf16>(h[0], h[1]), pack2<In16::bf16>(h[2], h[3])};
+        }
+    }
+}
+
+template <int NT>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(MoeGemmParams p)
 {
-    __shared__ __attribute__((aligned(16))) float red[4][8][64][4]; // [wave][m tile * 4 + n tile][lane][c]
+    __shared__ __attribute__((aligned(16))) float red_dyn[4 * 2 * NT * 64 * 4];
     const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
     if(blk * 32 >= p.num_valid[0])
         return;
     const int expert = p.sorted_expert_ids[blk];
     if(expert < 0 || expert >= p.experts)
         return;
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
-
-    // rows of the two m tiles this lane feeds as the "B" operand
-    const uint8_t* xrow[2];
-    int            tok[2];
-#pragma unroll
-    for(int j = 0; j < 2; ++j)
+    if(grp == 0 && threadIdx.x < 32) // record where each (token, slot) pair sits, for the final sum
     {
-        const int id = p.sorted_ids[blk * 32 + j * 16 + l16] & 0xffffff;
-        tok[j]       = id < p.M ? id : 0; // padding rows compute on token 0 and are never read
-        xrow[j]      = p.xq + (size_t)tok[j] * p.lda;
+        const int at = blk * 32 + threadIdx.x;
+        const int id = p.sorted_ids[at], token = id & 0xffffff, slot = (id >> 24) & 0xff;
+        if(token < p.M && slot < p.topk)
+            p.where[(size_t)token * p.topk + slot] = at;
     }
-    // weight tiles: n tiles 0,1 = gate columns grp*32 .. +31, n tiles 2,3 = the matching up columns
-    const size_t   wexp = (size_t)expert * (size_t)p.N * (size_t)p.K;
-    const uint8_t* wt[4];
-#pragma unroll
-    for(int i = 0; i < 4; ++i)
-    {
-        const int row0 = (i < 2 ? 0 : p.inter) + grp * 32 + (i & 1) * 16;
-        wt[i]          = p.w + wexp + (size_t)(row0 >> 4) * 16 * (size_t)p.K;
-    }
-    const float* ws_gate = p.wsc + ((size_t)expert * (p.N / 128) + (grp * 32) / 128) * p.kblocks;
-    const float* ws_up   = p.wsc + ((size_t)expert * (p.N / 128) + (p.inter + grp * 32) / 128) * p.kblocks;
-
-    f32x4 acc[2][4];
-#pragma unroll
-    for(int j = 0; j < 2; ++j)
-#pragma unroll
-        for(int i = 0; i < 4; ++i)
-            acc[j][i] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    struct Operands
-    {
-        i32x8 w[4], x[2];
-        float xs[2], wg, wu;
-    };
-    auto fetch = [&](int kb, Operands& o) {
-#pragma unroll
-        for(int i = 0; i < 4; ++i)
-            o.w[i] = load_w_fragment(wt[i] + (size_t)kb * 2048, l16, kg);
-#pragma unroll
-        for(int j = 0; j < 2; ++j)
-        {
-            o.x[j]  = load_x_fragment(xrow[j] + (size_t)kb * 128, kg);
-            o.xs[j] = p.xs[(size_t)kb * p.M + tok[j]];
-        }
-        o.wg = ws_gate[kb];
-        o.wu = ws_up[kb];
-    };
-    auto multiply = [&](const Operands& o) {
-#pragma unroll
-        for(int j = 0; j < 2; ++j)
-#pragma unroll
-            for(int i = 0; i < 4; ++i)
-            {
-                const f32x4 prod = mfma_16x16x128_fp8(o.w[i], o.x[j], f32x4{0.f, 0.f, 0.f, 0.f});
-                const float s    = o.xs[j] * (i < 2 ? o.wg : o.wu);
-#pragma unroll
-                for(int c = 0; c < 4; ++c)
-                    acc[j][i][c] = __builtin_fmaf(prod[c], s, acc[j][i][c]);
-            }
-    };
-    // two operand sets, filled alternately: the next K block travels while this one is multiplied
-    Operands a, b;
-    int      kb = wave;
-    if(kb < p.kblocks)
-        fetch(kb, a);
-    while(kb < p.kblocks)
-    {
-        if(kb + 4 < p.kblocks)
-            fetch(kb + 4, b);
-        multiply(a);
-        kb += 4;
-        if(kb >= p.kblocks)
-            break;
-        if(kb + 4 < p.kblocks)
-            fetch(kb + 4, a);
-        multiply(b);
-        kb += 4;
-    }
-
-#pragma unroll
-    for(int j = 0; j < 2; ++j)
-#pragma unroll
-        for(int i = 0; i < 4; ++i)
-            *(f32x4*)red[wave][j * 4 + i][lane] = acc[j][i];
-    __syncthreads();
-    // wave w' finishes the pair (m tile w'>>1, gate tile w'&1 with up tile 2 + (w'&1))
-    const int j = wave >> 1, i = wave & 1;
-    f32x4     g = f32x4{0.f, 0.f, 0.f, 0.f}, u = g;
-#pragma unroll
-    for(int w = 0; w < 4; ++w) // wave order: the sum does not depend on timing
-    {
-        g += *(const f32x4*)red[w][j * 4 + i][lane];
-        u += *(const f32x4*)red[w][j * 4 + 2 + i][lane];
-    }
-    float h[4];
-#pragma unroll
-    for(int c = 0; c < 4; ++c)
-        h[c] = activate(g[c], p.activation) * u[c];
-    const int slot = blk * 32 + j * 16 + l16;
-    const int col  = grp * 32 + i * 16 + kg * 4;
-    *(u32x2*)(p.out + (size_t)slot * p.inter + col) =
-        u32x2{pack2<In16::bf16>(h[0], h[1]), pack2<In16::bf16>(h[2], h[3])};
+    // rows of a block are real pairs first, padding after: the second 16 rows matter only if row 16 is real
+    const bool second_half = (p.sorted_ids[blk * 32 + 16] & 0xffffff) < p.M;
+    if(second_half)
+        gate_up_body<2, NT>(p, red_dyn, blk, grp, expert);
+    else
+        gate_up_body<1, NT>(p, red_dyn, blk, grp, expert);
 }
 
-// Second GEMM.  Workgroup = (block of 32 sorted rows, 256 output columns), wave = 64 columns.
+// Second GEMM.  Workgroup = (block of 32 sorted rows, 512 output columns), wave = 128 columns =
+// 8 weight tiles walked two at a time with the next two already requested; the block's
+// activation rows (K = inter_dim, at most 4 K blocks on this path) stay in registers.
+template <int MT, int KB>
+__device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int grp, int expert)
+{
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
+    const int n0 = grp * 512 + wave * 128;
+    if(n0 >= p.N)
+        return;
+    i32x8 x[MT][KB];
+    float xs[MT][KB];
+    bool  real[MT]; // padding rows are multiplied along but not stored
+#pragma unroll
+    for(int j = 0; j < MT; ++j)
+    {
+        const size_t slot = (size_t)blk * 32 + j * 16 + l16;
+        real[j]           = (p.sorted_ids[slot] & 0xffffff) < p.M;
+#pragma unroll
+        for(int kb = 0; kb < KB; ++kb)
+        {
+            x[j][kb]  = load_x_fragment(p.xq + slot * p.lda + (size_t)kb * 128, kg);
+            xs[j][kb] = p.xs[slot * KB + kb];
+        }
+    }
+    const size_t   tile_stride = (size_t)16 * (size_t)p.K;
+    const uint8_t* wt  = p.w + (size_t)expert * (size_t)p.N * (size_t)p.K + (size_t)(n0 >> 4) * tile_stride;
+    const float*   wsr = p.wsc + (size_t)expert * (p.N / 128) * KB;
+    const int      pairs = (p.N - n0) / 32 < 4 ? (p.N - n0) / 32 : 4; // N is a multiple of 256
+
+    auto fetch = [&](int pair, i32x8 (&w)[2][KB]) {
+#pragma unroll
+        for(int i = 0; i < 2; ++i)
+#pragma unroll
+            for(int kb = 0; kb < KB; ++kb)
+                w[i][kb] = load_w_fragment(wt + (size_t)(pair * 2 + i) * tile_stride + (size_t)kb * 2048, l16, kg);
+    };
+    auto finish = [&](int pair, const i32x8 (&w)[2][KB]) {
+#pragma unroll
+        for(int i = 0; i < 2; ++i)
+        {
+            const int    n   = n0 + (pair * 2 + i) * 16;
+            const float* wsn = wsr + (size_t)(n / 128) * KB;
+#pragma unroll
+            for(int j = 0; j < MT; ++j)
+            {
+                f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for(int kb = 0; kb < KB; ++kb)
+                {
+                    const f32x4 prod = mfma_16x16x128_fp8(w[i][kb], x[j][kb], f32x4{0.f, 0.f, 0.f, 0.f});
+                    const float sc   = xs[j][kb] * wsn[kb];
+#pragma unroll
+                    for(int c = 0; c < 4; ++c)
+                        acc[c] = __builtin_fmaf(prod[c], sc, acc[c]);
+                }
+                const size_t slot = (size_t)blk * 32 + j * 16 + l16;
+                const int    col  = n + kg * 4;
+                if(!real[j])
+                    continue;
+                if(p.out_f32)
+                    *(f32x4*)((float*)p.out + slot * p.N + col) = acc;
+                else
+                    *(u32x2*)(p.out + slot * p.N + col) =
+                        u32x2{pack2<In16::bf16>(acc[0], acc[1]), pack2<In16::bf16>(acc[2], acc[3])};
+            }
+        }
+    };
+    i32x8 wa[2][KB], wb[2][KB];
+    fetch(0, wa);
+    for(int pair = 0; pair < pairs; pair += 2)
+    {
+        if(pair + 1 < pairs)
+            fetch(pair + 1, wb);
+        finish(pair, wa);
+        if(pair + 1 >= pairs)
+            break;
+        if(pair + 2 < pairs)
+            fetch(pair + 2, wa);
+        finish(pair + 1, wb);
+    }
+}
+
+template <int KB>
 __global__ __launch_bounds__(256) void moe_down_kernel(MoeGemmParams p)
+{
+    const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
+    if(blk * 32 >= p.num_valid[0])
+        return;
+    const int expert = p.sorted_expert_ids[blk];
+    if(expert < 0 || expert >= p.experts)
+        return;
+    const bool second_half = (p.sorted_ids[blk * 32 + 16] & 0xffffff) < p.M;
+    if(second_half)
+        down_body<2, KB>(p, blk, grp, expert);
+    else
+        down_body<1, KB>(p, blk, grp, expert);
+}
+
+// The same for any K: workgroup = (block, 256 columns), wave = 64 columns, K blocks walked in turn.
+__global__ __launch_bounds__(256) void moe_down_long_k_kernel(MoeGemmParams p)
 {
     const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
     if(blk * 32 >= p.num_valid[0])
@@ -458,12 +683,14 @@ __global__ __launch_bounds__(256) void moe_down_kernel(MoeGemmParams p)
         return;
     const uint8_t* xrow[2];
     const float*   xsr[2];
+    bool           real[2];
 #pragma unroll
     for(int j = 0; j < 2; ++j)
     {
         const size_t slot = (size_t)blk * 32 + j * 16 + l16;
         xrow[j]           = p.xq + slot * p.lda;
         xsr[j]            = p.xs + slot * p.kblocks;
+        real[j]           = (p.sorted_ids[slot] & 0xffffff) < p.M;
     }
     const uint8_t* wt  = p.w + (size_t)expert * (size_t)p.N * (size_t)p.K + (size_t)(n0 >> 4) * 16 * (size_t)p.K;
     const float*   wsr = p.wsc + ((size_t)expert * (p.N / 128) + n0 / 128) * p.kblocks;
@@ -480,13 +707,13 @@ __global__ __launch_bounds__(256) void moe_down_kernel(MoeGemmParams p)
 #pragma unroll
         for(int i = 0; i < 4; ++i)
             w[i] = load_w_fragment(wt + (size_t)i * 16 * (size_t)p.K + (size_t)kb * 2048, l16, kg);
-        float s[2];
+        float       sc[2];
         const float wsv = wsr[kb];
 #pragma unroll
         for(int j = 0; j < 2; ++j)
         {
-            x[j] = load_x_fragment(xrow[j] + (size_t)kb * 128, kg);
-            s[j] = xsr[j][kb] * wsv;
+            x[j]  = load_x_fragment(xrow[j] + (size_t)kb * 128, kg);
+            sc[j] = xsr[j][kb] * wsv;
         }
 #pragma unroll
         for(int j = 0; j < 2; ++j)
@@ -496,7 +723,7 @@ __global__ __launch_bounds__(256) void moe_down_kernel(MoeGemmParams p)
                 const f32x4 prod = mfma_16x16x128_fp8(w[i], x[j], f32x4{0.f, 0.f, 0.f, 0.f});
 #pragma unroll
                 for(int c = 0; c < 4; ++c)
-                    acc[j][i][c] = __builtin_fmaf(prod[c], s[j], acc[j][i][c]);
+                    acc[j][i][c] = __builtin_fmaf(prod[c], sc[j], acc[j][i][c]);
             }
     }
 #pragma unroll
@@ -506,27 +733,14 @@ __global__ __launch_bounds__(256) void moe_down_kernel(MoeGemmParams p)
         {
             const size_t slot = (size_t)blk * 32 + j * 16 + l16;
             const int    col  = n0 + i * 16 + kg * 4;
+            if(!real[j])
+                continue;
             if(p.out_f32)
                 *(f32x4*)((float*)p.out + slot * p.N + col) = acc[j][i];
             else
                 *(u32x2*)(p.out + slot * p.N + col) = u32x2{pack2<In16::bf16>(acc[j][i][0], acc[j][i][1]),
                                                             pack2<In16::bf16>(acc[j][i][2], acc[j][i][3])};
         }
-}
-
-// where each (token, slot) pair sits in the sorted order (-1: not routed to a local expert)
-__global__ __launch_bounds__(256) void moe_invert_kernel(const int32_t* __restrict__ sorted_ids,
-                                                         const int32_t* __restrict__ num_valid,
-                                                         int32_t* __restrict__ where, int32_t M, int32_t topk,
-                                                         int32_t max_padded)
-{
-    const int32_t n = num_valid[0] < max_padded ? num_valid[0] : max_padded;
-    for(int32_t i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256)
-    {
-        const int32_t id = sorted_ids[i], token = id & 0xffffff, slot = (id >> 24) & 0xff;
-        if(token < M && slot < topk)
-            where[(size_t)token * topk + slot] = i;
-    }
 }
 
 // out[token] += sum over the token's slots, in slot order, of weight * y[sorted position]
@@ -690,6 +904,11 @@ hipError_t launch_moe_sorting(const MoeSortArgs& a, hipStream_t stream)
         g                 = g > 4096 ? 4096 : (g < 1 ? 1 : g);
         hipLaunchKernelGGL(fill_zero_kernel, dim3(g), dim3(256), 0, stream, (u32x4*)a.moe_buf, vecs);
     }
+    if(n <= kSortChunk)
+    {
+        hipLaunchKernelGGL(moe_sort_single_kernel, dim3(1), dim3(1024), 0, stream, p);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(moe_sort_count_kernel, dim3(p.chunks), dim3(1024), (size_t)a.experts * 4, stream, p);
     hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(1), dim3(1024), ((size_t)a.experts * 2 + 1) * 4, stream, p);
     hipLaunchKernelGGL(moe_sort_scatter_kernel, dim3(p.chunks), dim3(1024), 0, stream, p);
@@ -731,8 +950,14 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     const bool y32 = rows_in_f32(a);
     uint16_t*  y   = (uint16_t*)ws;
     ws += align_up(slots * a.dim * (y32 ? 4 : 2));
-    int32_t* where = (int32_t*)ws;
+    int32_t* where = (int32_t*)ws; // sorted position of each (token, slot) pair, -1 = not routed here
     ws += align_up((size_t)a.M * a.topk * 4);
+    {
+        const size_t n = (size_t)a.M * a.topk;
+        unsigned     g = (unsigned)((n + 255) / 256);
+        g              = g > 2048 ? 2048 : g;
+        hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, stream, where, n, -1);
+    }
 
     const uint8_t* xq = a.xq;
     const float*   xs = a.xs;
@@ -759,17 +984,6 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
         xs = s;
     }
 
-    {
-        const size_t n = (size_t)a.M * a.topk;
-        unsigned     g = (unsigned)((n + 255) / 256);
-        g              = g > 2048 ? 2048 : g;
-        hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, stream, where, n, -1);
-        unsigned g2 = (unsigned)((slots + 255) / 256);
-        g2          = g2 > 2048 ? 2048 : g2;
-        hipLaunchKernelGGL(moe_invert_kernel, dim3(g2), dim3(256), 0, stream, a.sorted_ids, a.num_valid, where, a.M,
-                           a.topk, a.max_padded);
-    }
-
     MoeGemmParams p{};
     p.xq                = xq;
     p.xs                = xs;
@@ -784,12 +998,29 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     p.N                 = 2 * a.inter;
     p.inter             = a.inter;
     p.kblocks           = a.dim / 128;
-    p.n_groups          = a.inter / 32;
+
+    p.topk              = a.topk;
+    p.where             = where;
     p.max_blocks        = a.max_blocks;
     p.experts           = a.experts;
     p.activation        = a.activation;
     p.lda               = a.x16 ? a.dim : a.lda;
-    hipLaunchKernelGGL(moe_gate_up_kernel, dim3((unsigned)((size_t)a.max_blocks * p.n_groups)), dim3(256), 0, stream, p);
+    {
+        // (expert, block) pairs to expect: every expert that can be hit once, plus the full blocks
+        const int64_t pairs = (int64_t)a.M * a.topk;
+        const int64_t est_blocks = (pairs < a.experts ? pairs : a.experts) + pairs / 32;
+        int           nt = a.gate_tiles;
+        if(nt != 1 && nt != 2 && nt != 4)
+            nt = est_blocks * (a.inter / 64) >= 1024 ? 4 : est_blocks * (a.inter / 32) >= 1024 ? 2 : 1;
+        p.n_groups = a.inter / (16 * nt);
+        const dim3 grid((unsigned)((size_t)a.max_blocks * p.n_groups));
+        switch(nt)
+        {
+        case 4: hipLaunchKernelGGL(moe_gate_up_kernel<4>, grid, dim3(256), 0, stream, p); break;
+        case 2: hipLaunchKernelGGL(moe_gate_up_kernel<2>, grid, dim3(256), 0, stream, p); break;
+        default: hipLaunchKernelGGL(moe_gate_up_kernel<1>, grid, dim3(256), 0, stream, p); break;
+        }
+    }
 
     QuantArgs qa{};
     qa.x               = h16;
@@ -815,10 +1046,26 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     d.K             = a.inter;
     d.N             = a.dim;
     d.kblocks       = a.inter / 128;
-    d.n_groups      = (a.dim + 255) / 256;
     d.lda           = a.inter;
     d.out_f32       = y32 ? 1 : 0;
-    hipLaunchKernelGGL(moe_down_kernel, dim3((unsigned)((size_t)a.max_blocks * d.n_groups)), dim3(256), 0, stream, d);
+    if(d.kblocks <= 4)
+    {
+        d.n_groups      = (a.dim + 511) / 512;
+        const dim3 grid((unsigned)((size_t)a.max_blocks * d.n_groups));
+        switch(d.kblocks)
+        {
+        case 1: hipLaunchKernelGGL(moe_down_kernel<1>, grid, dim3(256), 0, stream, d); break;
+        case 2: hipLaunchKernelGGL(moe_down_kernel<2>, grid, dim3(256), 0, stream, d); break;
+        case 3: hipLaunchKernelGGL(moe_down_kernel<3>, grid, dim3(256), 0, stream, d); break;
+        default: hipLaunchKernelGGL(moe_down_kernel<4>, grid, dim3(256), 0, stream, d); break;
+        }
+    }
+    else
+    {
+        d.n_groups = (a.dim + 255) / 256;
+        hipLaunchKernelGGL(moe_down_long_k_kernel, dim3((unsigned)((size_t)a.max_blocks * d.n_groups)), dim3(256), 0,
+                           stream, d);
+    }
 
     const dim3 cgrid((unsigned)a.M, (unsigned)((a.dim / 4 + 255) / 256));
     auto combine = a.out_dtype == In16::bf16

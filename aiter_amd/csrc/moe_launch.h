@@ -54,6 +54,7 @@ struct MoeArgs
     In16           out_dtype;
     int32_t        M, dim, inter, experts, topk, max_padded, max_blocks;
     int32_t        activation; // 0 silu, 1 gelu
+    int32_t        gate_tiles; // first GEMM: 16-column tiles per workgroup (1, 2, 4), 0 = choose
     int64_t        lda, out_stride;
     int            device_id;
 };

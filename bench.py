@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the FP8 block-scale path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload quant|prefill|decode|decode9|sweep|fused]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload quant|prefill|decode|decode9|sweep|moe|fused]
                     [--no-also] [--no-cpu]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
@@ -16,6 +16,7 @@ Workloads (BASELINE.json configs):
                      weights rotate through 640 MB so that every call reads them from HBM
   sweep    (beyond the configs) M in {128..4096} x four projection shapes, each beside the
                      duration the reference's tuner recorded for it
+  moe      (beyond the configs) block-scale expert layer of DeepSeek-V3, 1..1024 tokens
   fused    config 5  RMSNorm + 1x128 quant on [2048,7168], then GEMM N=4096
 
 Timing uses HIP events recorded on the stream the kernels are launched on (torch's current
@@ -47,7 +48,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="quant", choices=["quant", "prefill", "decode", "decode9", "sweep", "fused", "copy"],
+    ap.add_argument("--workload", default="quant", choices=["quant", "prefill", "decode", "decode9", "sweep", "moe", "fused", "copy"],
                     help="'copy' is a plain 1 GiB device copy used to calibrate the rocprofv3 FETCH_SIZE / "
                     "WRITE_SIZE counters; it is not part of the path")
     ap.add_argument("--no-also", action="store_true", help="time only the primary workload")
@@ -58,6 +59,7 @@ def parse_args():
                     help="GEMM workloads: row-major weights (gemm_a8w8_blockscale) or weights shuffled "
                     "(16,16) with column-major x_scale (gemm_a8w8_blockscale_bpreshuffle)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--kernel-name", default="", help="kernelName handed to the expert kernel of --workload moe")
     return ap.parse_args()
 
 
@@ -484,7 +486,107 @@ class SweepWorkload:
         return None
 
 
+# Durations (us) the reference's tuner recorded on a 256-CU part for the DeepSeek-V3 expert layer
+# (dim 7168, inter 256, 256 routed + 1 shared expert, top-8 + shared, fp8 per_1x128):
+# aiter/configs/model_configs/a8w8_blockscale_tuned_fmoe_ds_v3.csv, column "us" (both GEMM stages).
+MOE_REFERENCE_US = {1: 77.49, 16: 112.68, 32: 158.48, 64: 212.99, 128: 241.60, 256: 249.58, 512: 260.97, 1024: 359.48}
+
+
+class MoeWorkload:
+    """Block-scale expert layer of DeepSeek-V3 at one GPU's share: tokens x (8 of 256 routed experts
+    + the shared one), dim 7168, inter 256.  Timed: fmoe_fp8_blockscale_g1u1 on sorted tokens; the
+    routing is redrawn for every launch of a replayed graph so that weights come from HBM."""
+
+    name = "moe"
+    DIM, INTER, ROUTED, TOPK = 7168, 256, 256, 8
+    kernel_name = ""  # set from --kernel-name before setup()
+
+    def setup(self, torch, dev):
+        import aiter_amd
+        from aiter_amd import dtypes
+
+        self.torch, self.dev, self.aiter, self.fp8 = torch, dev, aiter_amd, dtypes.fp8
+        E = self.ROUTED + 1
+        g = torch.Generator(device=dev).manual_seed(0)
+        w1 = (torch.randn(E * 2 * self.INTER, self.DIM, generator=g, device=dev) * 0.1).bfloat16()
+        self.w1q, w1s = aiter_amd.weight_per_128x128_quant(w1)
+        del w1
+        w2 = (torch.randn(E * self.DIM, self.INTER, generator=g, device=dev) * 0.1).bfloat16()
+        self.w2q, w2s = aiter_amd.weight_per_128x128_quant(w2)
+        del w2
+        self.w1q = aiter_amd.shuffle_weight(self.w1q.view(E, 2 * self.INTER, self.DIM).view(torch.uint8)).view(dtypes.fp8)
+        self.w2q = aiter_amd.shuffle_weight(self.w2q.view(E, self.DIM, self.INTER).view(torch.uint8)).view(dtypes.fp8)
+        self.w1s, self.w2s = w1s.view(E, -1).contiguous(), w2s.view(E, -1).contiguous()
+        self.gen = g
+        self.prepare(32)
+
+    def prepare(self, tokens, routings=8):
+        torch, dev, aiter_amd = self.torch, self.dev, self.aiter
+        E = self.ROUTED + 1
+        x = torch.randn(tokens, self.DIM, generator=self.gen, device=dev).bfloat16()
+        self.xq, self.xs = aiter_amd.get_hip_quant(aiter_amd.QuantType.per_1x128)(
+            x, quant_dtype=self.fp8, transpose_scale=True)
+        self.xs = self.xs.view(self.DIM // 128, tokens)
+        self.tokens = tokens
+        self.sorted = []
+        self.experts_hit = 0
+        for _ in range(routings):
+            score = torch.randn(tokens, self.ROUTED, generator=self.gen, device=dev)
+            tw, ti = aiter_amd.fused_topk(x, score, self.TOPK, True)
+            ti = torch.cat([ti, torch.full((tokens, 1), self.ROUTED, dtype=ti.dtype, device=dev)], dim=1)
+            tw = torch.cat([tw, torch.ones(tokens, 1, dtype=tw.dtype, device=dev)], dim=1)
+            self.sorted.append(aiter_amd.moe_sorting(ti.contiguous(), tw.contiguous(), E, self.DIM, torch.bfloat16))
+            self.experts_hit += ti.unique().numel()
+        self.experts_hit /= routings
+        self.ids_for_sort = (ti.contiguous(), tw.contiguous())
+        self.i = 0
+
+    def step(self):
+        self.i = (self.i + 1) % len(self.sorted)
+        s_ids, s_w, s_e, nv, out = self.sorted[self.i]
+        self.aiter.fmoe_fp8_blockscale_g1u1(out, self.xq, self.w1q, self.w2q, s_ids, s_w, s_e, nv, self.TOPK + 1,
+                                            self.xs, self.w1s, self.w2s, self.kernel_name)
+
+    def step_sort(self):
+        self.aiter.moe_sorting(self.ids_for_sort[0], self.ids_for_sort[1], self.ROUTED + 1, self.DIM,
+                               self.torch.bfloat16)
+
+    def bytes(self):
+        # weights of the experts that are hit (read once), tokens and scales in, output out
+        per_expert = 3 * self.INTER * self.DIM + 4 * (3 * self.INTER // 128) * (self.DIM // 128)
+        return self.experts_hit * per_expert + self.tokens * self.DIM * (1 + 2) + 4 * self.tokens * self.DIM // 128
+
+    def flops(self):
+        return 2.0 * self.tokens * (self.TOPK + 1) * 3 * self.INTER * self.DIM
+
+    def describe(self):
+        return {"workload": "block-scale expert layer, dim 7168, inter 256, 256 routed + 1 shared expert, top-8 + "
+                            "shared; headline value is 32 tokens",
+                "kernel": "fmoe_fp8_blockscale_g1u1 (sorting timed separately)"}
+
+    def result(self, sec):
+        gbs = self.bytes() / sec / 1e9
+        return gbs, "GB/s", {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": gbs / HBM_PEAK_GBS, "traffic": None}
+
+    def per_shape(self, torch, steps, warmup):
+        out = []
+        for tokens, ref in MOE_REFERENCE_US.items():
+            self.prepare(tokens)
+            s = time_launches(torch, self.step, steps, warmup)
+            ss = time_launches(torch, self.step_sort, steps, warmup)
+            out.append({"tokens": tokens, "experts_hit": self.experts_hit, "kernel_us": s * 1e6,
+                        "sorting_us": ss * 1e6, "GB/s": self.bytes() / s / 1e9, "TFLOP/s": self.flops() / s / 1e12,
+                        "reference_tuned_us": ref, "reference_over_ours": ref / (s * 1e6)})
+        return out
+
+    def cpu_baseline(self, torch):
+        return None
+
+
 def make_workload(name):
+    if name == "moe":
+        return MoeWorkload()
     if name == "sweep":
         return SweepWorkload()
     if name == "copy":
@@ -522,6 +624,7 @@ def main():
 
     GemmWorkload.layout = args.layout
     GemmWorkload.rotate_mb = args.rotate_mb
+    MoeWorkload.kernel_name = args.kernel_name
     wl = make_workload(args.workload)
     wl.setup(torch, dev)
     sec = time_steps(torch, wl.step, args.steps, args.warmup)
@@ -548,7 +651,7 @@ def main():
     }
     if args.workload == "prefill":
         line["vs_reference_tuned_csv"] = value / REF_PREFILL_TFLOPS
-    if args.workload in ("decode9", "sweep"):
+    if args.workload in ("decode9", "sweep", "moe"):
         # shape after shape: steps + warmup launches each, in DECODE_SHAPES order
         line["per_shape"] = wl.per_shape(torch, args.steps, args.warmup)
         args.no_also = True
