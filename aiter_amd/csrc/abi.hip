@@ -664,6 +664,8 @@ int topk_softmax(aiter_tensor_t* topk_weights, aiter_tensor_t* topk_indices,
         a.w_stride  = tokens > 1 ? topk_weights->strides[0] : topk;
         a.id_stride = tokens > 1 ? topk_indices->strides[0] : topk;
         a.renorm    = need_renorm != 0;
+        if(tokens == 0)
+            return;
         DeviceGuard guard(gating_output->device_id);
         check_hip(fn, fp8bs::launch_topk_softmax(a, (hipStream_t)stream), nullptr);
     });
@@ -910,6 +912,8 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
         if(kernel_name && strncmp(kernel_name, "nt=", 3) == 0)
             a.gate_tiles = atoi(kernel_name + 3);
         a.device_id         = input->device_id;
+        if(M == 0)
+            return; // nothing to do, and no device needed to say so
         DeviceGuard guard(input->device_id);
         check_hip(fn, fp8bs::launch_fmoe_blockscale(a, (hipStream_t)stream), nullptr);
     });

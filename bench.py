@@ -695,6 +695,29 @@ def main():
                         "weight_MB_rotated": w3.weight_bytes_rotated / 1e6})
             del w3
         also["decode"] = dec
+        mid = []
+        for (m, n, k) in [(256, 4096, 7168), (512, 7168, 2048), (1024, 4096, 7168)]:
+            w4 = GemmWorkload("sweep", m, n, k, "sweep")
+            w4.rotate_always = True
+            w4.setup(torch, dev)
+            s4 = time_launches(torch, w4.step, 30, 5)
+            mid.append({"M": m, "N": n, "K": k, "kernel_us": s4 * 1e6, "TFLOP/s": w4.flops() / s4 / 1e12,
+                        "reference_tuned_us": SWEEP_REFERENCE_US[(m, n, k)],
+                        "reference_over_ours": SWEEP_REFERENCE_US[(m, n, k)] / (s4 * 1e6)})
+            del w4
+            torch.cuda.empty_cache()
+        also["mid_m"] = mid
+        w5 = MoeWorkload()
+        w5.setup(torch, dev)
+        moe = []
+        for tokens in (32, 128):
+            w5.prepare(tokens)
+            s5 = time_launches(torch, w5.step, 16, 3)
+            moe.append({"tokens": tokens, "kernel_us": s5 * 1e6, "GB/s": w5.bytes() / s5 / 1e9,
+                        "reference_tuned_us": MOE_REFERENCE_US[tokens],
+                        "reference_over_ours": MOE_REFERENCE_US[tokens] / (s5 * 1e6)})
+        del w5
+        also["moe"] = moe
         line["also"] = also
 
     print(json.dumps(line))

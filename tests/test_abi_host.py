@@ -139,6 +139,62 @@ def test_gemm_validation(lib):
     assert rc == 0 and msg is None
 
 
+def test_moe_validation(lib):
+    R = ctypes.byref
+    g = lambda t: R(fake_gpu(t))
+    f8 = lambda *sh: torch.zeros(*sh, dtype=torch.uint8).view(dtypes.fp8)
+    i32 = lambda *sh: torch.zeros(*sh, dtype=torch.int32)
+    # routing
+    rc, msg = call_raw(lib, "topk_softmax", g(torch.zeros(4, 2)), g(i32(4, 2)), None, g(torch.zeros(4, 2000)), 1, None)
+    assert rc == -1 and "experts = 2000" in msg
+    rc, msg = call_raw(lib, "topk_softmax", g(torch.zeros(4, 9)), g(i32(4, 9)), None, g(torch.zeros(4, 8)), 1, None)
+    assert rc == -1 and "topk = 9" in msg
+    rc, msg = call_raw(lib, "topk_softmax", g(torch.zeros(4, 2)), g(i32(4, 2).long()), None, g(torch.zeros(4, 8)), 1, None)
+    assert rc == -1 and "int32" in msg
+    # sorting: buffers sized as aiter/fused_moe.py:209-215 sizes them
+    ids, w = i32(4, 2), torch.zeros(4, 2)
+    padded = 4 * 2 + 8 * 32 - 2
+    ok = (g(ids), g(w), g(i32(padded)), g(torch.zeros(padded)), g(i32((padded + 31) // 32)), g(i32(2)))
+    rc, msg = call_raw(lib, "moe_sorting_fwd", *ok[:2], g(i32(padded - 1)), *ok[3:], None, 8, 32, None, None, 0, None)
+    assert rc == -1 and "sorted_token_ids" in msg and str(padded) in msg
+    rc, msg = call_raw(lib, "moe_sorting_fwd", *ok, None, 2000, 32, None, None, 0, None)
+    assert rc == -1 and "num_experts" in msg
+    rc, msg = call_raw(lib, "moe_sorting_fwd", *ok, None, 8, 32, g(i32(7)), None, 0, None)
+    assert rc == -1 and "local_expert_mask" in msg
+    # experts
+    E, dim, inter, M = 4, 256, 128, 4
+    args = dict(out=torch.zeros(M, dim, dtype=torch.bfloat16), inp=f8(M, dim), gate=f8(E, 2 * inter, dim),
+                down=f8(E, dim, inter), sids=i32(padded), sw=torch.zeros(padded), se=i32((padded + 31) // 32),
+                nv=i32(2), xs=torch.zeros(dim // 128, M), s1=torch.zeros(E, 2 * inter // 128 * dim // 128),
+                s2=torch.zeros(E, dim // 128 * inter // 128))
+
+    def fmoe(topk=2, blkn=128, blkk=128, act=0, block_m=32, **over):
+        a = dict(args, **over)
+        opt = lambda t: g(t) if t is not None else None
+        return call_raw(lib, "fmoe_fp8_blockscale_g1u1", g(a["out"]), g(a["inp"]), g(a["gate"]), g(a["down"]),
+                        g(a["sids"]), g(a["sw"]), g(a["se"]), g(a["nv"]), topk, opt(a["xs"]), g(a["s1"]), g(a["s2"]),
+                        b"", blkn, blkk, None, act, block_m, None)
+
+    rc, msg = fmoe(gate=f8(E, inter, dim))
+    assert rc == -1 and "gate must be [experts, 2*inter_dim, dim]" in msg
+    rc, msg = fmoe(blkn=64)
+    assert rc == -1 and "128 x 128" in msg
+    rc, msg = fmoe(block_m=16)
+    assert rc == -1 and "block_size_M" in msg
+    rc, msg = fmoe(act=7)
+    assert rc == -1 and "activation" in msg
+    rc, msg = fmoe(xs=None)
+    assert rc == -1 and "input_scale" in msg
+    rc, msg = fmoe(xs=torch.zeros(M, dim // 128))
+    assert rc == -1 and "[dim/128, tokens]" in msg
+    rc, msg = fmoe(s2=torch.zeros(E, 3))
+    assert rc == -1 and "fc2_scale" in msg
+    rc, msg = fmoe(out=torch.zeros(M, dim))
+    assert rc == -1 and "bf16 or fp16" in msg
+    rc, msg = fmoe(inp=f8(0, dim), out=torch.zeros(0, dim, dtype=torch.bfloat16), xs=torch.zeros(dim // 128, 0))
+    assert rc == 0 and msg is None  # nothing to do: returns before any HIP call
+
+
 def test_rmsnorm_validation(lib):
     R = ctypes.byref
     x = torch.zeros(4, 1024, dtype=torch.bfloat16)
