@@ -14,7 +14,7 @@
 // The GEMMs stream pre-shuffled (16,16) weights straight into MFMA operand registers: a 16-row
 // tile's K block is 2 KiB of contiguous memory in fragment order, so no LDS staging is needed.
 // A workgroup owns one block of 32 sorted rows (one expert).  First GEMM: 32 gate + 32 up
-// columns, its 4 waves split K and add their partial tiles through LDS, the activation is applied
+// columns, its 8 waves split K and add their partial tiles through LDS, the activation is applied
 // and the product written as bf16; the 1x128 quantiser of the dense path then turns it into fp8.
 // Second GEMM: 4 waves x 64 columns, K = inter_dim; rows are written per sorted slot (one writer
 // per element, fp32 while that fits 1 GiB, else bf16), and a last kernel adds each token's slots
@@ -418,6 +418,7 @@ struct MoeGemmParams
     int32_t        M, K, N, inter, kblocks, n_groups, max_blocks, experts, activation;
     int32_t        out_f32; // second GEMM only: rows kept in fp32
     int32_t        topk;
+    int32_t        waves;   // second GEMM only: waves per workgroup, 128 columns each
     int32_t*       where;   // first GEMM only: [M][topk] sorted position of each (token, slot) pair
     int64_t        lda;
 };
@@ -448,12 +449,17 @@ __device__ __forceinline__ float activate(float g, int activation)
 // First GEMM + activation.  Workgroup = (block of 32 sorted rows, NT x 16 inter columns): NT
 // gate tiles and the NT matching up tiles; NT is picked at launch (small units when few (expert,
 // block) pairs exist, so that the last units to finish do not set the kernel's duration; wide
-// units otherwise, which re-read the activations less often).  The 4 waves take every fourth K
+// units otherwise, which re-read the activations less often).  The waves take every eighth K
 // block each and add their partial tiles through LDS in wave order.  One operand set per wave:
 // several workgroups share a compute unit and cover each other's load latency.  A block whose
 // second half is padding (the usual case when few tokens are routed) multiplies one 16-row tile
 // only.  MFMA roles as in the dense kernels: weight rows are the "A" operand, activation rows
 // the "B" operand, so a lane ends up with 4 consecutive columns of one row.
+// waves per workgroup of the first GEMM: each keeps one K block of its tiles in flight, and a
+// workgroup that has a compute unit to itself (the last units of a launch) should still stream at
+// the unit's share of HBM
+constexpr int kGateUpWaves = 8;
+
 template <int MT, int NT>
 __device__ __forceinline__ void gate_up_body(const MoeGemmParams& p, float* red, int blk, int grp, int expert)
 {
@@ -482,7 +488,7 @@ __device__ __forceinline__ void gate_up_body(const MoeGemmParams& p, float* red,
         for(int i = 0; i < 2 * NT; ++i)
             acc[j][i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    for(int kb = wave; kb < p.kblocks; kb += 4)
+    for(int kb = wave; kb < p.kblocks; kb += kGateUpWaves)
     {
         i32x8 w[2 * NT], x[MT];
         float xs[MT];
@@ -527,7 +533,7 @@ __device__ __forceinline__ void gate_up_body(const MoeGemmParams& p, float* red,
             const int i = wave;
             f32x4     g = f32x4{0.f, 0.f, 0.f, 0.f}, u = g;
 #pragma unroll
-            for(int w = 0; w < 4; ++w) // wave order: the sum does not depend on timing
+            for(int w = 0; w < kGateUpWaves; ++w) // wave order: the sum does not depend on timing
             {
                 g += *(const f32x4*)(red + (((size_t)w * (2 * NT) + i) * 64 + lane) * 4);
                 u += *(const f32x4*)(red + (((size_t)w * (2 * NT) + NT + i) * 64 + lane) * 4);
@@ -545,9 +551,9 @@ __device__ __forceinline__ void gate_up_body(const MoeGemmParams& p, float* red,
 }
 
 template <int NT>
-__global__ __launch_bounds__(256) void moe_gate_up_kernel(MoeGemmParams p)
+__global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmParams p)
 {
-    __shared__ __attribute__((aligned(16))) float red_dyn[4 * 2 * NT * 64 * 4];
+    __shared__ __attribute__((aligned(16))) float red_dyn[kGateUpWaves * 2 * NT * 64 * 4];
     const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
     if(blk * 32 >= p.num_valid[0])
         return;
@@ -576,7 +582,7 @@ template <int MT, int KB>
 __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int grp, int expert)
 {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
-    const int n0 = grp * 512 + wave * 128;
+    const int n0 = (grp * p.waves + wave) * 128;
     if(n0 >= p.N)
         return;
     i32x8 x[MT][KB];
@@ -653,7 +659,7 @@ __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int g
 }
 
 template <int KB>
-__global__ __launch_bounds__(256) void moe_down_kernel(MoeGemmParams p)
+__global__ __launch_bounds__(512) void moe_down_kernel(MoeGemmParams p)
 {
     const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
     if(blk * 32 >= p.num_valid[0])
@@ -1016,9 +1022,9 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
         const dim3 grid((unsigned)((size_t)a.max_blocks * p.n_groups));
         switch(nt)
         {
-        case 4: hipLaunchKernelGGL(moe_gate_up_kernel<4>, grid, dim3(256), 0, stream, p); break;
-        case 2: hipLaunchKernelGGL(moe_gate_up_kernel<2>, grid, dim3(256), 0, stream, p); break;
-        default: hipLaunchKernelGGL(moe_gate_up_kernel<1>, grid, dim3(256), 0, stream, p); break;
+        case 4: hipLaunchKernelGGL(moe_gate_up_kernel<4>, grid, dim3(64 * kGateUpWaves), 0, stream, p); break;
+        case 2: hipLaunchKernelGGL(moe_gate_up_kernel<2>, grid, dim3(64 * kGateUpWaves), 0, stream, p); break;
+        default: hipLaunchKernelGGL(moe_gate_up_kernel<1>, grid, dim3(64 * kGateUpWaves), 0, stream, p); break;
         }
     }
 
@@ -1050,14 +1056,15 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     d.out_f32       = y32 ? 1 : 0;
     if(d.kblocks <= 4)
     {
-        d.n_groups      = (a.dim + 511) / 512;
+        d.waves         = (a.down_waves == 2 || a.down_waves == 4 || a.down_waves == 8) ? a.down_waves : 4;
+        d.n_groups      = (a.dim + 128 * d.waves - 1) / (128 * d.waves);
         const dim3 grid((unsigned)((size_t)a.max_blocks * d.n_groups));
         switch(d.kblocks)
         {
-        case 1: hipLaunchKernelGGL(moe_down_kernel<1>, grid, dim3(256), 0, stream, d); break;
-        case 2: hipLaunchKernelGGL(moe_down_kernel<2>, grid, dim3(256), 0, stream, d); break;
-        case 3: hipLaunchKernelGGL(moe_down_kernel<3>, grid, dim3(256), 0, stream, d); break;
-        default: hipLaunchKernelGGL(moe_down_kernel<4>, grid, dim3(256), 0, stream, d); break;
+        case 1: hipLaunchKernelGGL(moe_down_kernel<1>, grid, dim3(64 * d.waves), 0, stream, d); break;
+        case 2: hipLaunchKernelGGL(moe_down_kernel<2>, grid, dim3(64 * d.waves), 0, stream, d); break;
+        case 3: hipLaunchKernelGGL(moe_down_kernel<3>, grid, dim3(64 * d.waves), 0, stream, d); break;
+        default: hipLaunchKernelGGL(moe_down_kernel<4>, grid, dim3(64 * d.waves), 0, stream, d); break;
         }
     }
     else
