@@ -16,7 +16,7 @@
 // A workgroup owns one block of 32 sorted rows (one expert).  First GEMM: 32 gate + 32 up
 // columns, its 8 waves split K and add their partial tiles through LDS, the activation is applied
 // and the product written as bf16; the 1x128 quantiser of the dense path then turns it into fp8.
-// Second GEMM: 4 waves x 64 columns, K = inter_dim; rows are written per sorted slot (one writer
+// Second GEMM: waves x 128 columns, K = inter_dim; rows are written per sorted slot (one writer
 // per element, fp32 while that fits 1 GiB, else bf16), and a last kernel adds each token's slots
 // in slot order, weighted, into `out`: deterministic, unlike atomic accumulation.
 #include "gemm_common.h"
@@ -26,7 +26,8 @@ namespace fp8bs {
 
 namespace {
 
-constexpr int kSortChunk = 4096; // (token, slot) pairs per workgroup of the large sort
+constexpr int kSortChunk = 4096;      // most (token, slot) pairs the one-workgroup sort takes
+constexpr int kSortChunkMulti = 1024; // pairs per workgroup of the three-launch sort
 
 __device__ __forceinline__ float wave_max(float v)
 {
@@ -125,8 +126,8 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const T* __restrict__
 
 // ---------------------------------------------------------------------------------------------
 // Sorting.  Three launches: per-chunk histograms; one workgroup that turns them into per-chunk
-// write positions, block -> expert ids and the totals; a stable scatter in which thread e walks
-// the chunk (held in LDS) for expert e, so that pairs keep their (token, slot) order.
+// write positions, block -> expert ids and the totals; a stable scatter, one wave per chunk, so
+// that pairs keep their (token, slot) order.  Up to kSortChunk pairs one workgroup does it all.
 struct SortParams
 {
     const int32_t* topk_ids;     // [M][topk], row stride id_stride
@@ -162,8 +163,8 @@ __global__ __launch_bounds__(1024) void moe_sort_count_kernel(SortParams p)
         hist[e] = 0;
     __syncthreads();
     const int64_t n = (int64_t)sort_rows(p) * p.topk;
-    const int64_t lo = (int64_t)blockIdx.x * kSortChunk;
-    for(int i = threadIdx.x; i < kSortChunk; i += blockDim.x)
+    const int64_t lo = (int64_t)blockIdx.x * kSortChunkMulti;
+    for(int i = threadIdx.x; i < kSortChunkMulti; i += blockDim.x)
     {
         const int64_t f = lo + i;
         if(f >= n)
@@ -177,71 +178,85 @@ __global__ __launch_bounds__(1024) void moe_sort_count_kernel(SortParams p)
         p.counts[(size_t)blockIdx.x * p.experts + e] = hist[e];
 }
 
+// Exclusive scan over the experts (thread = expert, 1024 threads) of the padded run lengths and of
+// the "is local" flags: where each expert's run starts (-1 if masked out), its local id, and the
+// padded total.
+struct ExpertSpan
+{
+    int32_t begin, local, total;
+};
+__device__ __forceinline__ ExpertSpan expert_spans(bool live, int32_t padded_len)
+{
+    __shared__ int64_t wave_total[16];
+    int64_t       packed = ((int64_t)(live ? 1 : 0) << 40) | (int64_t)(live ? padded_len : 0);
+    const int64_t mine   = packed;
+#pragma unroll
+    for(int o = 1; o < 64; o <<= 1)
+    {
+        const int64_t up = __shfl_up(packed, o);
+        if((int)(threadIdx.x & 63) >= o)
+            packed += up;
+    }
+    if((threadIdx.x & 63) == 63)
+        wave_total[threadIdx.x >> 6] = packed;
+    __syncthreads();
+    int64_t base = 0, all = 0;
+    for(int w = 0; w < 16; ++w)
+    {
+        if(w < (int)(threadIdx.x >> 6))
+            base += wave_total[w];
+        all += wave_total[w];
+    }
+    const int64_t excl = base + packed - mine;
+    ExpertSpan    r;
+    r.begin = live ? (int32_t)(excl & 0xffffffffffll) : -1;
+    r.local = (int32_t)(excl >> 40);
+    r.total = (int32_t)(all & 0xffffffffffll);
+    return r;
+}
+
 __global__ __launch_bounds__(1024) void moe_sort_scan_kernel(SortParams p)
 {
-    extern __shared__ int32_t sh[]; // [experts] padded totals -> exclusive starts, [experts] local ids
-    int32_t* padded = sh;
-    int32_t* local  = sh + p.experts;
-    for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
-    {
-        int32_t run = 0;
+    const int e   = threadIdx.x;
+    int32_t   run = 0;
+    if(e < p.experts)
         for(int c = 0; c < p.chunks; ++c)
         {
             const int32_t n                       = p.counts[(size_t)c * p.experts + e];
             p.counts[(size_t)c * p.experts + e] = run; // position inside the expert's run
             run += n;
         }
-        const bool masked = p.expert_mask && p.expert_mask[e] == 0;
-        padded[e]         = masked ? -1 : (run + p.unit - 1) / p.unit * p.unit;
-        // the unpadded count rides in expert_begin until the starts are known
-        p.expert_begin[e] = run;
-    }
-    __syncthreads();
-    if(threadIdx.x == 0)
+    const bool       live = e < p.experts && !(p.expert_mask && p.expert_mask[e] == 0);
+    const int32_t    len  = (run + p.unit - 1) / p.unit * p.unit;
+    const ExpertSpan span = expert_spans(live, len);
+    if(e == 0)
     {
-        int32_t at = 0, lid = 0;
-        for(int e = 0; e < p.experts; ++e)
+        p.num_valid_ids[0] = span.total;
+        p.num_valid_ids[1] = sort_rows(p);
+    }
+    const int32_t pad_id = (p.topk << 24) | p.M;
+    if(e < p.experts)
+    {
+        p.expert_begin[e] = span.begin;
+        if(live)
         {
-            const int32_t len = padded[e];
-            padded[e]         = len < 0 ? -1 : at;
-            local[e]          = lid;
-            if(len >= 0)
+            for(int b = 0; b < len / p.unit; ++b)
+                p.sorted_expert_ids[span.begin / p.unit + b] = span.local;
+            for(int i = run; i < len; ++i)
             {
-                at += len;
-                ++lid;
+                p.sorted_ids[span.begin + i]     = pad_id;
+                p.sorted_weights[span.begin + i] = 0.f;
             }
         }
-        p.num_valid_ids[0] = at;
-        p.num_valid_ids[1] = sort_rows(p);
-        sh[2 * p.experts]  = at;
     }
-    __syncthreads();
-    const int32_t total = sh[2 * p.experts];
-    const int32_t pad_id = (p.topk << 24) | p.M;
-    for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
-    {
-        const int32_t begin = padded[e], count = p.expert_begin[e];
-        p.expert_begin[e]   = begin;
-        if(begin < 0)
-            continue;
-        const int32_t len = (count + p.unit - 1) / p.unit * p.unit;
-        for(int b = 0; b < len / p.unit; ++b)
-            p.sorted_expert_ids[begin / p.unit + b] = local[e];
-        for(int i = count; i < len; ++i)
-        {
-            p.sorted_ids[begin + i]     = pad_id;
-            p.sorted_weights[begin + i] = 0.f;
-        }
-    }
-    for(int b = total / p.unit + threadIdx.x; b < p.max_blocks; b += blockDim.x)
+    for(int b = span.total / p.unit + threadIdx.x; b < p.max_blocks; b += blockDim.x)
         p.sorted_expert_ids[b] = -1;
-    for(int i = total + threadIdx.x; i < p.max_padded; i += blockDim.x)
+    for(int i = span.total + threadIdx.x; i < p.max_padded; i += blockDim.x)
     {
         p.sorted_ids[i]     = pad_id;
         p.sorted_weights[i] = 0.f;
     }
 }
-
 
 // Stable scatter of one chunk of (token, slot) pairs held in LDS, by one wave: 64 pairs at a time,
 // a pair's rank among the earlier pairs of its expert comes from ballots over the bits of the
@@ -277,28 +292,27 @@ __device__ __forceinline__ void scatter_chunk(const SortParams& p, const int32_t
     }
 }
 
-__global__ __launch_bounds__(1024) void moe_sort_scatter_kernel(SortParams p)
+__global__ __launch_bounds__(64) void moe_sort_scatter_kernel(SortParams p)
 {
-    __shared__ int32_t ids[kSortChunk];
-    __shared__ float   wts[kSortChunk];
+    __shared__ int32_t ids[kSortChunkMulti];
+    __shared__ float   wts[kSortChunkMulti];
+    __shared__ int32_t begin[1024], running[1024];
     const int64_t      n  = (int64_t)sort_rows(p) * p.topk;
-    const int64_t      lo = (int64_t)blockIdx.x * kSortChunk;
-    const int          cnt = (int)((n - lo) < kSortChunk ? (n - lo > 0 ? n - lo : 0) : kSortChunk);
+    const int64_t      lo = (int64_t)blockIdx.x * kSortChunkMulti;
+    const int          cnt = (int)((n - lo) < kSortChunkMulti ? (n - lo > 0 ? n - lo : 0) : kSortChunkMulti);
     for(int i = threadIdx.x; i < cnt; i += blockDim.x)
     {
         const int64_t f = lo + i;
         ids[i]          = p.topk_ids[(f / p.topk) * p.id_stride + (f % p.topk)];
         wts[i]          = p.topk_weights[(f / p.topk) * p.w_stride + (f % p.topk)];
     }
-    __shared__ int32_t begin[1024], running[1024];
     for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
     {
         begin[e]   = p.expert_begin[e];
         running[e] = p.counts[(size_t)blockIdx.x * p.experts + e];
     }
     __syncthreads();
-    if(threadIdx.x < 64)
-        scatter_chunk(p, ids, wts, begin, running, cnt, lo);
+    scatter_chunk(p, ids, wts, begin, running, cnt, lo);
 }
 
 // All of it in one workgroup, for up to kSortChunk pairs (the decode regime): histogram in LDS,
@@ -324,40 +338,19 @@ __global__ __launch_bounds__(1024) void moe_sort_single_kernel(SortParams p)
             atomicAdd(&count[e], 1);
     }
     __syncthreads();
+    const bool       live_e = (int)threadIdx.x < p.experts && !(p.expert_mask && p.expert_mask[threadIdx.x] == 0);
+    const int32_t    len_e  = (int)threadIdx.x < p.experts ? (count[threadIdx.x] + p.unit - 1) / p.unit * p.unit : 0;
+    const ExpertSpan span   = expert_spans(live_e, len_e);
+    if((int)threadIdx.x < p.experts)
     {
-        // exclusive scan over the experts of (padded length, 1 if local), one expert per thread
-        const int  e      = threadIdx.x;
-        const bool live   = e < p.experts && !(p.expert_mask && p.expert_mask[e] == 0);
-        const int  len    = live ? (count[e] + p.unit - 1) / p.unit * p.unit : 0;
-        int64_t    packed = ((int64_t)(live ? 1 : 0) << 40) | (int64_t)len;
-        const int64_t mine = packed;
-#pragma unroll
-        for(int o = 1; o < 64; o <<= 1)
-        {
-            const int64_t up = __shfl_up(packed, o);
-            if((threadIdx.x & 63) >= o)
-                packed += up;
-        }
-        __shared__ int64_t wave_total[16];
-        if((threadIdx.x & 63) == 63)
-            wave_total[threadIdx.x >> 6] = packed;
-        __syncthreads();
-        int64_t base = 0;
-        for(int w = 0; w < (int)(threadIdx.x >> 6); ++w)
-            base += wave_total[w];
-        const int64_t excl = base + packed - mine;
-        if(e < p.experts)
-        {
-            begin[e] = live ? (int32_t)(excl & 0xffffffffffll) : -1;
-            local[e] = (int32_t)(excl >> 40);
-        }
-        if(threadIdx.x == 1023)
-        {
-            const int32_t at   = (int32_t)((base + packed) & 0xffffffffffll);
-            s_total            = at;
-            p.num_valid_ids[0] = at;
-            p.num_valid_ids[1] = rows;
-        }
+        begin[threadIdx.x] = span.begin;
+        local[threadIdx.x] = span.local;
+    }
+    if(threadIdx.x == 0)
+    {
+        s_total            = span.total;
+        p.num_valid_ids[0] = span.total;
+        p.num_valid_ids[1] = rows;
     }
     __syncthreads();
     const int32_t total  = s_total;
@@ -892,7 +885,7 @@ hipError_t launch_moe_sorting(const MoeSortArgs& a, hipStream_t stream)
     p.id_stride         = a.id_stride;
     p.w_stride          = a.w_stride;
     const int64_t n     = (int64_t)a.M * a.topk;
-    p.chunks            = (int32_t)((n + kSortChunk - 1) / kSortChunk);
+    p.chunks            = (int32_t)((n + kSortChunkMulti - 1) / kSortChunkMulti);
     if(p.chunks < 1)
         p.chunks = 1;
     uint8_t*     scratch = nullptr;
@@ -916,8 +909,8 @@ hipError_t launch_moe_sorting(const MoeSortArgs& a, hipStream_t stream)
         return hipGetLastError();
     }
     hipLaunchKernelGGL(moe_sort_count_kernel, dim3(p.chunks), dim3(1024), (size_t)a.experts * 4, stream, p);
-    hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(1), dim3(1024), ((size_t)a.experts * 2 + 1) * 4, stream, p);
-    hipLaunchKernelGGL(moe_sort_scatter_kernel, dim3(p.chunks), dim3(1024), 0, stream, p);
+    hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(1), dim3(1024), 0, stream, p);
+    hipLaunchKernelGGL(moe_sort_scatter_kernel, dim3(p.chunks), dim3(64), 0, stream, p);
     return hipGetLastError();
 }
 
