@@ -912,8 +912,14 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
         a.down_waves = 0;
         if(kernel_name && strncmp(kernel_name, "nt=", 3) == 0)
             a.gate_tiles = atoi(kernel_name + 3);
+        a.down_wave_cols = 0;
         if(kernel_name && strncmp(kernel_name, "dw=", 3) == 0)
             a.down_waves = atoi(kernel_name + 3);
+        if(kernel_name && strncmp(kernel_name, "dc=", 3) == 0)
+        {
+            a.down_wave_cols = 64;
+            a.down_waves     = atoi(kernel_name + 3);
+        }
         a.device_id         = input->device_id;
         if(M == 0)
             return; // nothing to do, and no device needed to say so

@@ -411,7 +411,8 @@ struct MoeGemmParams
     int32_t        M, K, N, inter, kblocks, n_groups, max_blocks, experts, activation;
     int32_t        out_f32; // second GEMM only: rows kept in fp32
     int32_t        topk;
-    int32_t        waves;   // second GEMM only: waves per workgroup, 128 columns each
+    int32_t        waves;   // second GEMM only: waves per workgroup
+    int32_t        wave_cols; // second GEMM only: columns per wave (64 or 128)
     int32_t*       where;   // first GEMM only: [M][topk] sorted position of each (token, slot) pair
     int64_t        lda;
 };
@@ -575,7 +576,7 @@ template <int MT, int KB>
 __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int grp, int expert)
 {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
-    const int n0 = (grp * p.waves + wave) * 128;
+    const int n0 = (grp * p.waves + wave) * p.wave_cols;
     if(n0 >= p.N)
         return;
     i32x8 x[MT][KB];
@@ -596,7 +597,8 @@ __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int g
     const size_t   tile_stride = (size_t)16 * (size_t)p.K;
     const uint8_t* wt  = p.w + (size_t)expert * (size_t)p.N * (size_t)p.K + (size_t)(n0 >> 4) * tile_stride;
     const float*   wsr = p.wsc + (size_t)expert * (p.N / 128) * KB;
-    const int      pairs = (p.N - n0) / 32 < 4 ? (p.N - n0) / 32 : 4; // N is a multiple of 256
+    const int      want  = p.wave_cols / 32;
+    const int      pairs = (p.N - n0) / 32 < want ? (p.N - n0) / 32 : want; // N is a multiple of 256
 
     auto fetch = [&](int pair, i32x8 (&w)[2][KB]) {
 #pragma unroll
@@ -1050,7 +1052,8 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     if(d.kblocks <= 4)
     {
         d.waves         = (a.down_waves == 2 || a.down_waves == 4 || a.down_waves == 8) ? a.down_waves : 4;
-        d.n_groups      = (a.dim + 128 * d.waves - 1) / (128 * d.waves);
+        d.wave_cols     = a.down_wave_cols == 64 ? 64 : 128;
+        d.n_groups      = (a.dim + d.wave_cols * d.waves - 1) / (d.wave_cols * d.waves);
         const dim3 grid((unsigned)((size_t)a.max_blocks * d.n_groups));
         switch(d.kblocks)
         {
