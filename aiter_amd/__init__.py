@@ -21,6 +21,7 @@ from .shuffle import shuffle_weight
 from .fused_moe import (
     ActivationType,
     fmoe_fp8_blockscale_g1u1,
+    fused_moe,
     fused_moe_blockscale,
     fused_topk,
     moe_sorting,
@@ -64,4 +65,5 @@ __all__ = [
     "moe_sorting",
     "fmoe_fp8_blockscale_g1u1",
     "fused_moe_blockscale",
+    "fused_moe",
 ]

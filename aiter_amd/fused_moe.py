@@ -14,6 +14,7 @@ from enum import IntEnum
 import torch
 
 from . import _ffi, dtypes
+from .enums import QuantType
 
 BLOCK_SIZE_M = 32  # aiter/fused_moe.py: rows per sorted block
 
@@ -82,4 +83,56 @@ def fused_moe_blockscale(hidden_states_q, w1_shuffled, w2_shuffled, topk_weights
     fmoe_fp8_blockscale_g1u1(out, hidden_states_q, w1_shuffled, w2_shuffled, sorted_ids, sorted_weights,
                              sorted_expert_ids, num_valid_ids, topk, a1_scale_t, w1_scale, w2_scale, "",
                              scale_blk[0], scale_blk[1], None, int(activation))
+    return out
+
+
+def fused_moe(hidden_states, w1, w2, topk_weight, topk_ids, expert_mask=None, activation=ActivationType.Silu,
+              quant_type=QuantType.per_1x128, doweight_stage1=False, w1_scale=None, w2_scale=None, a1_scale=None,
+              a2_scale=None, block_size_M=None, num_local_tokens=None, moe_sorting_dispatch_policy=0, dtype=None,
+              **other):
+    """The block-scale flavour of aiter/fused_moe.py:458-577: ``quant_type`` per_1x128 (or per_128x128,
+    which the reference maps onto it, :1310), gate/up experts (g1u1), fp8 weights pre-shuffled with layout
+    (16,16) and their 128x128 scales.
+
+    hidden_states: bf16/fp16 [tokens, dim] (quantised 1x128 inside, as the reference's kernel does,
+    :1133-1136), or fp8 with ``a1_scale`` [tokens, dim/128] (transposed here, as the reference does with
+    partial_transpose, :1152-1158).  Returns the bf16/fp16 result [tokens, dim].  Every other option of the
+    reference's entry point raises NotImplementedError naming it."""
+    qt = QuantType(quant_type)
+    if qt not in (QuantType.per_1x128, QuantType.per_128x128):
+        raise NotImplementedError(f"fused_moe: only the block-scale flavour (per_1x128) is part of this library, got {qt!r}")
+    for name, value, neutral in (("doweight_stage1", doweight_stage1, False), ("a2_scale", a2_scale, None)):
+        if value is not neutral and value:
+            raise NotImplementedError(f"fused_moe: {name} is not supported by the block-scale kernel")
+    def neutral(v):
+        return v is None or (isinstance(v, (bool, int)) and v in (0, -1)) or (isinstance(v, str) and v == "separated")
+
+    unsupported = {k: v for k, v in other.items() if not neutral(v)}
+    if unsupported:
+        raise NotImplementedError(f"fused_moe: unsupported options {sorted(unsupported)}")
+    if block_size_M not in (None, -1, 0, BLOCK_SIZE_M):
+        raise NotImplementedError(f"fused_moe: block_size_M must be {BLOCK_SIZE_M}")
+    if w1_scale is None or w2_scale is None:
+        raise ValueError("fused_moe: w1_scale and w2_scale are required for per_1x128")
+    tokens, dim = hidden_states.shape
+    E = w1.shape[0]
+    topk = topk_ids.shape[1]
+    if w1.shape[1] != 2 * w2.shape[2]:
+        raise NotImplementedError("fused_moe: only gated experts (w1 = [E, 2*inter_dim, dim]) are supported")
+    if dtype is None:
+        dtype = hidden_states.dtype if hidden_states.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
+    num_experts = E if expert_mask is None else expert_mask.numel()
+    sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, out = moe_sorting(
+        topk_ids, topk_weight, num_experts, dim, dtype, BLOCK_SIZE_M, expert_mask, num_local_tokens,
+        moe_sorting_dispatch_policy)
+    if hidden_states.dtype in (torch.bfloat16, torch.float16):
+        a1, scale_t = hidden_states, None
+    else:
+        if a1_scale is None:
+            raise ValueError("a1_scale must be provided for quantized input for fused_moe")
+        a1 = hidden_states
+        scale_t = a1_scale.reshape(tokens, dim // 128).t().contiguous()
+    fmoe_fp8_blockscale_g1u1(out, a1, w1, w2, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, topk,
+                             scale_t, w1_scale.reshape(E, -1), w2_scale.reshape(E, -1), "", 128, 128, None,
+                             int(ActivationType(activation)), BLOCK_SIZE_M)
     return out

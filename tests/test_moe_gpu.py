@@ -275,6 +275,28 @@ def test_fmoe_matches_float64_evaluation():
     assert_close(run_moe(p), reference(p, compute=torch.float64), "fp64")
 
 
+def test_fused_moe_entry_point():
+    # aiter/fused_moe.py:458 with quant_type=per_1x128: 16-bit tokens, or fp8 tokens with row-major scales
+    p = make_moe(24, 512, 128, 8, 2, seed=10)
+    w1 = aiter_amd.shuffle_weight(p["w1q"].view(torch.uint8)).view(dtypes.fp8)
+    w2 = aiter_amd.shuffle_weight(p["w2q"].view(torch.uint8)).view(dtypes.fp8)
+    tw, ti = p["tw"].to(DEV), p["ti"].to(DEV)
+    kw = dict(quant_type=aiter_amd.QuantType.per_1x128, w1_scale=p["w1s"], w2_scale=p["w2s"])
+    a = aiter_amd.fused_moe(p["x"], w1, w2, tw, ti, **kw)
+    b = aiter_amd.fused_moe(p["aq"].to(DEV), w1, w2, tw, ti, a1_scale=p["asc"].to(DEV), **kw)
+    torch.cuda.synchronize()
+    assert a.dtype == torch.bfloat16 and a.shape == (24, 512)
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    assert_close(a, reference(p), "fused_moe")
+    with pytest.raises(NotImplementedError, match="block-scale"):
+        aiter_amd.fused_moe(p["x"], w1, w2, tw, ti, quant_type=aiter_amd.QuantType.per_Token, w1_scale=p["w1s"],
+                            w2_scale=p["w2s"])
+    with pytest.raises(NotImplementedError, match="doweight_stage1"):
+        aiter_amd.fused_moe(p["x"], w1, w2, tw, ti, doweight_stage1=True, **kw)
+    with pytest.raises(NotImplementedError, match="bias1"):
+        aiter_amd.fused_moe(p["x"], w1, w2, tw, ti, bias1=torch.zeros(1), **kw)
+
+
 def test_fmoe_rejects_what_it_cannot_do():
     p = make_moe(4, 512, 128, 4, 2, seed=1)
     w1 = aiter_amd.shuffle_weight(p["w1q"].view(torch.uint8)).view(dtypes.fp8)
