@@ -227,6 +227,24 @@ def test_fmoe_many_tokens_sampled_rows():
     assert ((o - plain).norm() / plain.norm()).item() < 3e-2
 
 
+@pytest.mark.parametrize("hint", ["nt=1", "nt=2", "nt=4", "dw=2", "dw=8", "dc=4"])
+def test_fmoe_tuning_hints_do_not_change_the_result(hint):
+    # 300 tokens on 4 experts: runs of many blocks per expert, partly filled last blocks
+    p = make_moe(300, 512, 256, 4, 2, seed=21)
+    w1 = aiter_amd.shuffle_weight(p["w1q"].view(torch.uint8)).view(dtypes.fp8)
+    w2 = aiter_amd.shuffle_weight(p["w2q"].view(torch.uint8)).view(dtypes.fp8)
+    outs = []
+    for name in ("", hint):
+        s_ids, s_w, s_e, nv, out = aiter_amd.moe_sorting(p["ti"].to(DEV), p["tw"].to(DEV), 4, 512, torch.bfloat16)
+        aiter_amd.fmoe_fp8_blockscale_g1u1(out, p["aq"].to(DEV), w1, w2, s_ids, s_w, s_e, nv, 2,
+                                           p["asc"].t().contiguous().to(DEV), p["w1s"], p["w2s"], name)
+        torch.cuda.synchronize()
+        outs.append(out)
+    assert_close(outs[1], reference(p), hint)
+    # the first GEMM sums its K blocks in the same order whatever the tiling: bitwise the same result
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+
+
 def test_fmoe_is_deterministic_and_accumulates_into_out():
     p = make_moe(48, 1024, 256, 16, 4, seed=2)
     a = run_moe(p)
