@@ -245,6 +245,27 @@ def test_mid_kernel_pinned_k_ranges(name, m, n, k, dtype):
     assert torch.equal(out.view(torch.int16), again.view(torch.int16))
 
 
+def test_automatic_choice_on_random_shapes():
+    # the kernel family, tile and number of K ranges all come from a cost model: whatever it picks must be right
+    g = torch.Generator().manual_seed(2024)
+    shapes = []
+    while len(shapes) < 40:
+        m = int(torch.randint(1, 700, (1,), generator=g))
+        n = int(torch.randint(1, 2600, (1,), generator=g))
+        k = 128 * int(torch.randint(1, 40, (1,), generator=g))
+        if len(shapes) % 3 == 0:
+            n = (n + 15) // 16 * 16      # the common case: N a multiple of 16
+        if m * n * k > 6e8:              # keeps the fp64 oracle quick
+            continue
+        shapes.append((m, n, k))
+    for (m, n, k) in shapes:
+        xq, wq, xs, ws = make_problem(m, n, k, seed=m * 7 + n, outliers=0.01)
+        out = run_gpu(xq, wq, xs, ws)
+        assert_close_to_f64(out, xq, wq, xs, ws, f"auto {m}x{n}x{k}")
+        again = run_gpu(xq, wq, xs, ws)
+        assert torch.equal(out.view(torch.int16), again.view(torch.int16)), f"auto {m}x{n}x{k} not repeatable"
+
+
 def test_mid_kernel_rejects_malformed_range_count():
     for name in ("mid_128x128:s=0", "mid_128x128:s=x", "mid_128x128:q=2", "mid_32x32"):
         with pytest.raises(RuntimeError, match="unknown kernelName"):
