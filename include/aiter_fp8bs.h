@@ -7,8 +7,12 @@
  * :1595-1612): every tensor is a BORROWED descriptor (`aiter_tensor_t*`, the caller owns the
  * memory and keeps it alive until the stream has run the work); `Optional[Tensor]` is NULL;
  * `int` is int64_t, `bool` is int, `float` is float, `str` is const char*; the caller's HIP
- * stream is the last argument.  Functions only enqueue work on that stream: they never
- * synchronise and never allocate device memory, so they can be captured into a HIP graph.
+ * stream is the last argument.  Functions only enqueue work on that stream and can be captured
+ * into a HIP graph.  The GEMM entry points (when K is split across workgroups) and the
+ * mixture-of-experts entry points keep scratch buffers that the library allocates on the first
+ * call that needs a larger one (hipMalloc; a buffer being replaced is freed after a stream
+ * synchronisation): run such a call once before capturing, and do not overlap calls that use
+ * the scratch on one device.  Nothing else allocates or synchronises.
  * Return value: 0 on success, -1 on failure with the message available from
  * aiter_get_last_error() (thread local).  No C++ exception crosses this boundary.
  *
