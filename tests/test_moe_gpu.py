@@ -211,7 +211,7 @@ def test_fmoe_other_shapes(tokens, dim, inter, experts, topk):
 
 def test_fmoe_many_tokens_sampled_rows():
     # 20 000 tokens: many blocks per expert, the three-launch sort, and second-GEMM rows kept in bf16
-    # (160 504 slots x 2048 columns x 4 bytes would exceed the 1 GiB the fp32 form is allowed)
+    # (fp32 rows are for decode-size batches)
     tokens, dim, inter, experts, topk = 20000, 2048, 128, 16, 8
     p = make_moe(tokens, dim, inter, experts, topk, seed=12)
     out = run_moe(p)
