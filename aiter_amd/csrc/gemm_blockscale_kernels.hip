@@ -173,15 +173,20 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
     if(name == nullptr)
     {
         // Up to 64 activation rows the weight-streaming kernel wins everywhere.  Above that,
-        // the 256x256 tiling or the mid_* tilings, whichever is modelled faster: a 256x256
-        // iteration over one K block takes about 1.8 us against 0.8 us for a quarter of the
-        // area, so it wins once its tiles cover enough of the chip (measured on the DeepSeek
-        // shapes: from about 128 tiles).
-        const int64_t prefill_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
-        const float   prefill_us    = 12.f + (float)((prefill_tiles + 255) / 256) * (float)p.kblocks * 1.8f;
+        // the 256x256 tiling or the mid_* tilings, whichever is modelled faster.  Measured on the
+        // DeepSeek shapes, a 256x256 iteration over one K block takes 1.7 us while the tiles of a
+        // round cover up to 56 % of the compute units and up to 2.1 us when they cover all of them,
+        // against 0.8 us for a quarter of the area: it wins once its tiles cover about half of the
+        // chip.  Near a tie it is preferred: it gains more when the weights are still in the
+        // last-level cache.
+        const int64_t prefill_tiles  = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
+        const int64_t prefill_rounds = (prefill_tiles + 255) / 256;
+        const float   prefill_share  = (float)prefill_tiles / (float)(prefill_rounds * 256);
+        const float   prefill_iter   = 1.7f + (prefill_share > 0.56f ? (prefill_share - 0.56f) * 0.9f : 0.f);
+        const float   prefill_us     = 13.5f + (float)prefill_rounds * (float)p.kblocks * prefill_iter;
         if(p.M <= 64 && gemm_decode_supports(p))
             name = "decode_stream";
-        else if(gemm_mid_supports(p) && (!gemm_prefill_supports(p) || gemm_mid_estimate_us(p) < prefill_us))
+        else if(gemm_mid_supports(p) && (!gemm_prefill_supports(p) || gemm_mid_estimate_us(p) * 1.03f < prefill_us))
             name = "mid_auto";
         else if(gemm_prefill_supports(p))
             name = "prefill_256x256";

@@ -467,7 +467,7 @@ static MidPlan plan_cost(const GemmKernelParams& g, int tile, int splits)
     const int   occupancy = tile == 64 ? 2 : 1;
     const float fixed     = tile == 64 ? 4.5f : tile == 64128 ? 5.7f : 6.9f;
     const float iter0     = tile == 64 ? 0.56f : tile == 64128 ? 0.70f : 0.74f;
-    const float iter1     = tile == 64 ? 0.07f : tile == 64128 ? 0.05f : 0.06f;
+    const float iter1     = tile == 64 ? 0.07f : tile == 64128 ? 0.08f : 0.12f;
     const int   tiles     = ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
     const int   wgs = tiles * splits, slots = 256 * occupancy;
     const int   rounds    = (wgs + slots - 1) / slots;
