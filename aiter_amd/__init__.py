@@ -13,6 +13,7 @@ from .enums import QuantType
 from .gemm_op_a8w8 import (
     gemm_a8w8_blockscale,
     gemm_a8w8_blockscale_bpreshuffle,
+    gemm_a8w8_blockscale_bpreshuffle_asm,
     gemm_a8w8_blockscale_bpreshuffle_ck,
     gemm_a8w8_blockscale_ck,
     gemm_kernel_names,
@@ -25,6 +26,8 @@ from .fused_moe import (
     fused_moe_blockscale,
     fused_topk,
     moe_sorting,
+    moe_sorting_fwd,
+    topk_softmax,
 )
 from .quant import (
     dynamic_per_token_scaled_quant,
@@ -49,6 +52,7 @@ __all__ = [
     "weight_per_128x128_quant",
     "gemm_a8w8_blockscale_bpreshuffle",
     "gemm_a8w8_blockscale_bpreshuffle_ck",
+    "gemm_a8w8_blockscale_bpreshuffle_asm",
     "per_group_quant_hip",
     "dynamic_per_token_scaled_quant",
     "gemm_a8w8_blockscale",
@@ -63,6 +67,8 @@ __all__ = [
     "ActivationType",
     "fused_topk",
     "moe_sorting",
+    "moe_sorting_fwd",
+    "topk_softmax",
     "fmoe_fp8_blockscale_g1u1",
     "fused_moe_blockscale",
     "fused_moe",

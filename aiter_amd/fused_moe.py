@@ -15,6 +15,7 @@ import torch
 
 from . import _ffi, dtypes
 from .enums import QuantType
+from .torch_ops import fake_none, torch_op
 
 BLOCK_SIZE_M = 32  # aiter/fused_moe.py: rows per sorted block
 
@@ -23,6 +24,36 @@ class ActivationType(IntEnum):
     # csrc/include/aiter_enum.h:5-14 (the two the block-scale kernel accepts)
     Silu = 0
     Gelu = 1
+
+
+@torch_op(
+    "topk_softmax(Tensor(a!) topk_weights, Tensor(b!) topk_indices, Tensor(c!)? token_expert_indices, "
+    'Tensor gating_output, bool need_renorm, int num_shared_experts=0, str shared_expert_scoring_func="") -> ()',
+    fake_none,
+)
+def topk_softmax(topk_weights, topk_indices, token_expert_indices, gating_output, need_renorm,
+                 num_shared_experts=0, shared_expert_scoring_func=""):
+    """Native binding (aiter/ops/moe_op.py:29-66): softmax over the experts, top-k (ties to the lower
+    index), optional renormalisation; ``token_expert_indices`` (may be None) receives
+    ``slot * tokens + token``."""
+    if num_shared_experts:
+        raise NotImplementedError("topk_softmax: shared-expert scoring is not part of this library")
+    _ffi.call("topk_softmax", topk_weights, topk_indices, token_expert_indices, gating_output, bool(need_renorm))
+
+
+@torch_op(
+    "moe_sorting_fwd(Tensor topk_ids, Tensor topk_weights, Tensor(a!) sorted_token_ids, Tensor(b!) sorted_weights, "
+    "Tensor(c!) sorted_expert_ids, Tensor(d!) num_valid_ids, Tensor(e!) moe_buf, int num_experts, int unit_size, "
+    "Tensor? local_expert_mask=None, Tensor? num_local_tokens=None, int dispatch_policy=0) -> ()",
+    fake_none,
+)
+def moe_sorting_fwd(topk_ids, topk_weights, sorted_token_ids, sorted_weights, sorted_expert_ids, num_valid_ids,
+                    moe_buf, num_experts, unit_size, local_expert_mask=None, num_local_tokens=None,
+                    dispatch_policy=0):
+    """Native binding (aiter/ops/moe_sorting.py:11-25): fills the sorted arrays and zeroes ``moe_buf``."""
+    _ffi.call("moe_sorting_fwd", topk_ids, topk_weights, sorted_token_ids, sorted_weights, sorted_expert_ids,
+              num_valid_ids, moe_buf, int(num_experts), int(unit_size), local_expert_mask, num_local_tokens,
+              int(dispatch_policy))
 
 
 def fused_topk(hidden_states, gating_output, topk, renormalize, topk_ids=None, topk_weights=None):
@@ -36,7 +67,7 @@ def fused_topk(hidden_states, gating_output, topk, renormalize, topk_ids=None, t
         topk_ids = torch.empty(M, topk, dtype=dtypes.i32, device=dev)
     topk_weights, topk_ids = topk_weights[:M], topk_ids[:M]
     if M:
-        _ffi.call("topk_softmax", topk_weights, topk_ids, None, gating_output.contiguous(), bool(renormalize))
+        topk_softmax(topk_weights, topk_ids, None, gating_output.contiguous(), bool(renormalize))
     return topk_weights, topk_ids
 
 
@@ -53,12 +84,18 @@ def moe_sorting(topk_ids, topk_weights, num_experts, model_dim, moebuf_dtype, bl
     sorted_expert_ids = torch.empty(max_num_m_blocks, dtype=dtypes.i32, device=dev)
     num_valid_ids = torch.empty(2, dtype=dtypes.i32, device=dev)
     moe_buf = torch.empty((M, model_dim), dtype=moebuf_dtype, device=dev)
-    _ffi.call("moe_sorting_fwd", topk_ids, topk_weights, sorted_ids, sorted_weights, sorted_expert_ids,
-              num_valid_ids, moe_buf, int(num_experts), int(block_size), expert_mask, num_local_tokens,
-              int(dispatch_policy))
+    moe_sorting_fwd(topk_ids, topk_weights, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf,
+                    int(num_experts), int(block_size), expert_mask, num_local_tokens, int(dispatch_policy))
     return sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf
 
 
+@torch_op(
+    "fmoe_fp8_blockscale_g1u1(Tensor(a!) out, Tensor input, Tensor gate, Tensor down, Tensor sorted_token_ids, "
+    "Tensor sorted_weights, Tensor sorted_expert_ids, Tensor num_valid_ids, int topk, Tensor? input_scale, "
+    'Tensor fc1_scale, Tensor fc2_scale, str? kernelName="", int fc_scale_blkn=128, int fc_scale_blkk=128, '
+    "Tensor? fc2_smooth_scale=None, int? activation=0, int block_size_M=32) -> ()",
+    fake_none,
+)
 def fmoe_fp8_blockscale_g1u1(out, input, gate, down, sorted_token_ids, sorted_weights, sorted_expert_ids,
                              num_valid_ids, topk, input_scale, fc1_scale, fc2_scale, kernelName="",
                              fc_scale_blkn=128, fc_scale_blkk=128, fc2_smooth_scale=None,
@@ -66,7 +103,7 @@ def fmoe_fp8_blockscale_g1u1(out, input, gate, down, sorted_token_ids, sorted_we
     """out[token] += sum_k weight_k * down_e(act(gate_e x) * up_e x) on sorted tokens (in place)."""
     _ffi.call("fmoe_fp8_blockscale_g1u1", out, input, gate, down, sorted_token_ids, sorted_weights,
               sorted_expert_ids, num_valid_ids, int(topk), input_scale, fc1_scale, fc2_scale, kernelName or "",
-              int(fc_scale_blkn), int(fc_scale_blkk), fc2_smooth_scale, int(activation), int(block_size_M))
+              int(fc_scale_blkn), int(fc_scale_blkk), fc2_smooth_scale, int(activation or 0), int(block_size_M))
     return None
 
 

@@ -14,6 +14,17 @@ import torch
 from torch import Tensor
 
 from . import _ffi, dtypes
+from .torch_ops import fake_none, torch_op
+
+
+@torch_op(
+    "gemm_a8w8_blockscale_ck(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor(a!) Out, int splitK=0, "
+    'str kernelName="") -> ()',
+    fake_none,
+)
+def _blockscale_into(XQ: Tensor, WQ: Tensor, x_scale: Tensor, w_scale: Tensor, Out: Tensor, splitK: int = 0,
+                     kernelName: str = "") -> None:
+    _ffi.call("gemm_a8w8_blockscale", XQ, WQ, x_scale, w_scale, Out, int(splitK), kernelName or "")
 
 
 def gemm_a8w8_blockscale_ck(
@@ -26,11 +37,21 @@ def gemm_a8w8_blockscale_ck(
     kernelName: str = "",
 ) -> Tensor:
     """aiter/ops/gemm_op_a8w8.py:285-298: writes ``Out`` and returns it.  ``splitK`` is the log2
-    of the number of K partitions, ``kernelName`` one of :func:`gemm_kernel_names` or ""."""
-    _ffi.call("gemm_a8w8_blockscale", XQ, WQ, x_scale, w_scale, Out, int(splitK), kernelName or "")
+    of the number of K partitions (-1: the library chooses), ``kernelName`` one of
+    :func:`gemm_kernel_names` or ""."""
+    _blockscale_into(XQ, WQ, x_scale, w_scale, Out, splitK, kernelName)
     return Out
 
 
+def _gemm_fake(XQ, WQ, x_scale, w_scale, dtype=dtypes.bf16, *args, **kwargs):
+    return torch.empty(XQ.shape[0], WQ.shape[0], dtype=dtype, device=XQ.device)
+
+
+@torch_op(
+    "gemm_a8w8_blockscale(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, ScalarType dtype=bfloat16, "
+    "bool isBpreshuffled=False) -> Tensor",
+    _gemm_fake,
+)
 def gemm_a8w8_blockscale(
     XQ: Tensor,
     WQ: Tensor,
@@ -42,17 +63,31 @@ def gemm_a8w8_blockscale(
     """aiter/ops/gemm_op_a8w8.py:804-872.
 
     XQ [M,K] fp8, WQ [N,K] fp8, x_scale [M,K/128] fp32, w_scale [ceil(N/128),K/128] fp32;
-    returns a fresh [M,N] tensor of ``dtype`` (bf16 or fp16).
+    returns a fresh [M,N] tensor of ``dtype`` (bf16 or fp16).  With ``isBpreshuffled`` the
+    operands are those of :func:`gemm_a8w8_blockscale_bpreshuffle` (weights shuffled (16,16),
+    ``x_scale`` stored column-major), which the reference hands to its gfx950 assembly kernel for
+    M >= 16, K >= 512, bf16 (:821-825); no such limits here.
     """
     assert dtype in [dtypes.bf16, dtypes.fp16], f"Output {dtype=} is currently not supported in gemm_a8w8"
-    if isBpreshuffled:
-        raise NotImplementedError("the pre-shuffled weight layout is not part of this library")
     m = XQ.shape[0]
     n = WQ.shape[0]
     Y = torch.empty(m, n, dtype=dtype, device=XQ.device)
-    # -1: the library chooses kernel and K split from the shape
-    _ffi.call("gemm_a8w8_blockscale", XQ, WQ, x_scale, w_scale, Y, -1, "")
+    if isBpreshuffled:
+        _ffi.call("gemm_a8w8_blockscale_bpreshuffle", XQ, WQ, x_scale, w_scale, Y, "")
+    else:
+        # -1: the library chooses kernel and K split from the shape
+        _ffi.call("gemm_a8w8_blockscale", XQ, WQ, x_scale, w_scale, Y, -1, "")
     return Y
+
+
+@torch_op(
+    "gemm_a8w8_blockscale_bpreshuffle_ck(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor(a!) Out, "
+    'str kernelName="") -> ()',
+    fake_none,
+)
+def _bpreshuffle_into(XQ: Tensor, WQ: Tensor, x_scale: Tensor, w_scale: Tensor, Out: Tensor,
+                      kernelName: str = "") -> None:
+    _ffi.call("gemm_a8w8_blockscale_bpreshuffle", XQ, WQ, x_scale, w_scale, Out, kernelName or "")
 
 
 def gemm_a8w8_blockscale_bpreshuffle_ck(
@@ -65,8 +100,59 @@ def gemm_a8w8_blockscale_bpreshuffle_ck(
 ) -> Tensor:
     """aiter/ops/gemm_op_a8w8.py:318-330: ``WQ`` holds ``shuffle_weight(w, layout=(16, 16))`` and
     ``x_scale`` is column-major; writes ``Out`` and returns it."""
-    _ffi.call("gemm_a8w8_blockscale_bpreshuffle", XQ, WQ, x_scale, w_scale, Out, kernelName or "")
+    _bpreshuffle_into(XQ, WQ, x_scale, w_scale, Out, kernelName)
     return Out
+
+
+def gemm_a8w8_blockscale_bpreshuffle_asm(
+    A: Tensor,
+    B: Tensor,
+    out: Tensor,
+    A_scale: Tensor,
+    B_scale: Tensor,
+    bias: Optional[Tensor] = None,
+    splitK: Optional[int] = None,
+    kernelName: Optional[str] = None,
+    bpreshuffle: Optional[bool] = True,
+    zero_bias_buf: Optional[Tensor] = None,
+) -> Tensor:
+    """aiter/ops/gemm_op_a8w8.py:404-430: the reference's hand-scheduled kernel for the same
+    operands as :func:`gemm_a8w8_blockscale_bpreshuffle_ck` (argument order differs: ``out``
+    third).  ``splitK`` and the reference's kernel names are tuning hints of that kernel and are
+    not interpreted; a bias is not supported."""
+    if bias is not None:
+        raise NotImplementedError("gemm_a8w8_blockscale_bpreshuffle_asm: bias is not part of this library")
+    if not bpreshuffle:
+        raise NotImplementedError("gemm_a8w8_blockscale_bpreshuffle_asm: only pre-shuffled weights (bpreshuffle=True)")
+    _bpreshuffle_into(A, B, A_scale, B_scale, out, "")
+    return out
+
+
+def _bpreshuffle_fake(XQ, WQ, x_scale, w_scale, dtype=dtypes.bf16, out=None):
+    return torch.empty(XQ.shape[0], WQ.shape[0], dtype=dtype, device=XQ.device)
+
+
+def _bpreshuffle_eager(XQ, WQ, x_scale, w_scale, dtype=dtypes.bf16, out=None):
+    assert dtype in [dtypes.bf16, dtypes.fp16], f"Output {dtype=} is currently not supported in gemm_a8w8"
+    m = XQ.shape[0]
+    n = WQ.shape[0]
+    if out is not None:
+        assert out.shape == (m, n) and out.dtype == dtype and out.device == XQ.device, (
+            f"gemm_a8w8_blockscale_bpreshuffle: out buffer {tuple(out.shape)}/{out.dtype} != expected "
+            f"({m},{n})/{dtype}"
+        )
+        Y = out
+    else:
+        Y = torch.empty(m, n, dtype=dtype, device=XQ.device)
+    _ffi.call("gemm_a8w8_blockscale_bpreshuffle", XQ, WQ, x_scale, w_scale, Y, "")
+    return Y
+
+
+_bpreshuffle_op = torch_op(
+    "gemm_a8w8_blockscale_bpreshuffle(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, "
+    "ScalarType dtype=bfloat16, Tensor(a!)? out=None) -> Tensor",
+    _bpreshuffle_fake,
+)(_bpreshuffle_eager)
 
 
 def gemm_a8w8_blockscale_bpreshuffle(
@@ -82,21 +168,15 @@ def gemm_a8w8_blockscale_bpreshuffle(
     XQ [M,K] fp8; WQ [N,K] fp8 pre-shuffled with :func:`aiter_amd.shuffle_weight` (layout
     (16,16)); x_scale the [M,K/128] scales stored column-major (what the quant kernels write
     with ``transpose_scale=True``), either as a contiguous buffer or as a strided [M,K/128]
-    view; w_scale [ceil(N/128),K/128] fp32.  ``out``, when given, receives the result.
+    view; w_scale [ceil(N/128),K/128] fp32.  ``out``, when given, receives the result and is
+    returned.
     """
-    assert dtype in [dtypes.bf16, dtypes.fp16], f"Output {dtype=} is currently not supported in gemm_a8w8"
-    m = XQ.shape[0]
-    n = WQ.shape[0]
-    if out is not None:
-        assert out.shape == (m, n) and out.dtype == dtype and out.device == XQ.device, (
-            f"gemm_a8w8_blockscale_bpreshuffle: out buffer {tuple(out.shape)}/{out.dtype} != expected "
-            f"({m},{n})/{dtype}"
-        )
-        Y = out
-    else:
-        Y = torch.empty(m, n, dtype=dtype, device=XQ.device)
-    _ffi.call("gemm_a8w8_blockscale_bpreshuffle", XQ, WQ, x_scale, w_scale, Y, "")
-    return Y
+    if out is not None and torch.compiler.is_compiling():
+        # traced as "write into out": an op must not return one of its arguments
+        assert dtype in [dtypes.bf16, dtypes.fp16], f"Output {dtype=} is currently not supported in gemm_a8w8"
+        _bpreshuffle_into(XQ, WQ, x_scale, w_scale, out, "")
+        return out
+    return _bpreshuffle_op(XQ, WQ, x_scale, w_scale, dtype, out)
 
 
 def gemm_kernel_names():

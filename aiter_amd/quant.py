@@ -13,8 +13,14 @@ from torch import Tensor
 
 from . import _ffi, dtypes
 from .enums import QuantType
+from .torch_ops import fake_none, torch_op
 
 
+@torch_op(
+    "dynamic_per_token_scaled_quant(Tensor(a!) out, Tensor input, Tensor(b!) scales, Tensor? scale_ub=None, "
+    "bool shuffle_scale=False, Tensor? num_rows=None, int num_rows_factor=1) -> ()",
+    fake_none,
+)
 def dynamic_per_token_scaled_quant(
     out: Tensor,
     input: Tensor,
@@ -37,6 +43,19 @@ def dynamic_per_token_scaled_quant(
     )
 
 
+def _per_group_quant_fake(x, scale=None, quant_dtype=dtypes.fp8, group_size=128, transpose_scale=False,
+                          num_rows=None, num_rows_factor=1, scale_type=dtypes.fp32):
+    shape = x.shape
+    return (torch.empty(shape, dtype=quant_dtype, device=x.device),
+            torch.empty((*shape[:-1], shape[-1] // group_size), dtype=scale_type, device=x.device))
+
+
+@torch_op(
+    "per_group_quant_hip(Tensor x, Tensor? scale=None, ScalarType quant_dtype=float8_e4m3fn, int group_size=128, "
+    "bool transpose_scale=False, Tensor? num_rows=None, int num_rows_factor=1, ScalarType scale_type=float32) "
+    "-> (Tensor, Tensor)",
+    _per_group_quant_fake,
+)
 def per_group_quant_hip(
     x: Tensor,
     scale: Optional[Tensor] = None,

@@ -8,13 +8,20 @@ from __future__ import annotations
 from torch import Tensor
 
 from . import _ffi
+from .torch_ops import fake_none, torch_op
 
 
+@torch_op("rmsnorm(Tensor(a!) out, Tensor input, Tensor weight, float epsilon, bool gemma_norm=False) -> ()", fake_none)
 def rmsnorm(out: Tensor, input: Tensor, weight: Tensor, epsilon: float, gemma_norm: bool = False) -> None:
     """aiter/ops/rmsnorm.py:625-632."""
     _ffi.call("rmsnorm", out, input, weight, float(epsilon), bool(gemma_norm))
 
 
+@torch_op(
+    "rmsnorm_quant(Tensor(a!) out, Tensor input, Tensor(b!) scale, Tensor weight, float epsilon, int group_size=0, "
+    "bool shuffle_scale=False, bool gemma_norm=False) -> ()",
+    fake_none,
+)
 def rmsnorm_quant(
     out: Tensor,
     input: Tensor,
@@ -32,6 +39,11 @@ def rmsnorm_quant(
     )
 
 
+@torch_op(
+    "add_rmsnorm(Tensor(a!) out, Tensor input, Tensor residual_in, Tensor(b!) residual_out, Tensor weight, "
+    "float epsilon, bool gemma_norm=False) -> ()",
+    fake_none,
+)
 def add_rmsnorm(
     out: Tensor,
     input: Tensor,
@@ -45,6 +57,11 @@ def add_rmsnorm(
     _ffi.call("add_rmsnorm", out, input, residual_in, residual_out, weight, float(epsilon), bool(gemma_norm))
 
 
+@torch_op(
+    "add_rmsnorm_quant(Tensor(a!) out, Tensor input, Tensor residual_in, Tensor(b!) residual_out, Tensor(c!) scale, "
+    "Tensor weight, float epsilon, int group_size=0, bool shuffle_scale=False, bool gemma_norm=False) -> ()",
+    fake_none,
+)
 def add_rmsnorm_quant(
     out: Tensor,
     input: Tensor,
