@@ -907,7 +907,8 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
         a.max_padded        = (int32_t)(use_blocks * 32);
         a.activation        = (int32_t)activation;
         // the reference's names pick among its tuned kernels; here "nt=1|2|4" pins the first GEMM's
-        // columns per workgroup and anything else means choose
+        // columns per workgroup, "dw=" / "dc=" / "down=rows" pick the second GEMM that writes rows
+        // (and its shape), "down=cols" the one that sums per token in LDS, anything else means choose
         a.gate_tiles = 0;
         a.down_waves = 0;
         if(kernel_name && strncmp(kernel_name, "nt=", 3) == 0)
@@ -920,6 +921,12 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
             a.down_wave_cols = 64;
             a.down_waves     = atoi(kernel_name + 3);
         }
+        a.down_mode = 0;
+        if(kernel_name && (strncmp(kernel_name, "dw=", 3) == 0 || strncmp(kernel_name, "dc=", 3) == 0 ||
+                           strcmp(kernel_name, "down=rows") == 0))
+            a.down_mode = 1; // these hints are about the kernel that writes rows
+        if(kernel_name && strcmp(kernel_name, "down=cols") == 0)
+            a.down_mode = 2;
         a.device_id         = input->device_id;
         if(M == 0)
             return; // nothing to do, and no device needed to say so

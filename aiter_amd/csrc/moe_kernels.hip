@@ -16,9 +16,11 @@
 // A workgroup owns one block of 32 sorted rows (one expert).  First GEMM: 32 gate + 32 up
 // columns, its 8 waves split K and add their partial tiles through LDS, the activation is applied
 // and the product written as bf16; the 1x128 quantiser of the dense path then turns it into fp8.
-// Second GEMM: waves x 128 columns, K = inter_dim; rows are written per sorted slot (one writer
-// per element, fp32 for decode-size batches, else bf16), and a last kernel adds each token's slots
-// in slot order, weighted, into `out`: deterministic, unlike atomic accumulation.
+// Second GEMM, up to 128 tokens: a workgroup owns 16 output columns of every expert and adds each
+// token's weighted rows in LDS, in sorted order, then onto `out` (no intermediate rows at all).
+// Beyond: waves x 128 columns, K = inter_dim; rows are written per sorted slot (one writer per
+// element, fp32 while they take at most 32 MiB, else bf16), and a last kernel adds each token's
+// slots in slot order, weighted, into `out`.  Both are deterministic, unlike atomic accumulation.
 #include "gemm_common.h"
 #include "moe_launch.h"
 
@@ -414,6 +416,7 @@ struct MoeGemmParams
     int32_t        waves;   // second GEMM only: waves per workgroup
     int32_t        wave_cols; // second GEMM only: columns per wave (64 or 128)
     int32_t*       where;   // first GEMM only: [M][topk] sorted position of each (token, slot) pair
+    uint32_t*      block_mask; // first GEMM only: [blocks] bit r set = row r of the block is a real pair
     int64_t        lda;
 };
 
@@ -554,12 +557,20 @@ __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmP
     const int expert = p.sorted_expert_ids[blk];
     if(expert < 0 || expert >= p.experts)
         return;
-    if(grp == 0 && threadIdx.x < 32) // record where each (token, slot) pair sits, for the final sum
+    if(grp == 0 && threadIdx.x < 64) // record which rows are real pairs, and where each pair sits, for the final sum
     {
-        const int at = blk * 32 + threadIdx.x;
-        const int id = p.sorted_ids[at], token = id & 0xffffff, slot = (id >> 24) & 0xff;
-        if(token < p.M && slot < p.topk)
-            p.where[(size_t)token * p.topk + slot] = at;
+        bool real = false;
+        if(threadIdx.x < 32)
+        {
+            const int at = blk * 32 + threadIdx.x;
+            const int id = p.sorted_ids[at], token = id & 0xffffff, slot = (id >> 24) & 0xff;
+            real         = token < p.M && slot < p.topk;
+            if(real && p.where)
+                p.where[(size_t)token * p.topk + slot] = at;
+        }
+        const uint64_t rows = __ballot(real);
+        if(threadIdx.x == 0 && p.block_mask)
+            p.block_mask[blk] = (uint32_t)rows;
     }
     // rows of a block are real pairs first, padding after: the second 16 rows matter only if row 16 is real
     const bool second_half = (p.sorted_ids[blk * 32 + 16] & 0xffffff) < p.M;
@@ -744,6 +755,252 @@ __global__ __launch_bounds__(256) void moe_down_long_k_kernel(MoeGemmParams p)
         }
 }
 
+
+// Second GEMM fused with the per-token sum, for decode-size batches.  Workgroup = one 16-column
+// weight tile of every expert; wave kb multiplies K block kb.  A wave walks the (block, 16-row
+// half) units that hold real pairs, in sorted order, with the next kColsDepth units' operands
+// already requested (a unit is 2 KiB of weights per wave: the depth is what keeps a wave's share
+// of HBM in flight), and adds each weighted product row into its own [tokens][16] fp32 table in
+// LDS: one wave per table and a fixed walk, so the sum is deterministic.  The tables are added in
+// K-block order onto `out`.  No rows are written to memory and no position table is needed.
+struct DownColsParams
+{
+    const uint8_t*  xq;  // [slots][K] fp8 by sorted slot
+    const float*    xs;  // [slots][K/128]
+    const uint8_t*  w;   // [experts][N][K] fp8, pre-shuffled (16,16) per expert
+    const float*    wsc; // [experts][N/128][K/128]
+    const int32_t*  sorted_ids;
+    const float*    sorted_weights;
+    const int32_t*  sorted_expert_ids;
+    const int32_t*  num_valid;
+    const uint32_t* block_mask; // [blocks], written by the first GEMM
+    uint16_t*       out;        // [M][N], row stride out_stride
+    int64_t         out_stride;
+    int32_t         M, K, N, kblocks, max_blocks, experts;
+};
+
+constexpr int kColsDepth     = 8;
+constexpr int kColsMaxBlocks = 1024; // blocks the unit scan takes (16 per lane)
+
+struct ColsStage
+{
+    i32x4    wlo, whi, xlo, xhi;
+    float    xs, sw, ws;
+    int32_t  tok;
+    uint32_t mask;
+};
+
+// The walk's loads are issued from asm and waited for by count: left to the compiler, every
+// outstanding load is waited for at the head of the loop (one memory latency per kColsDepth units
+// instead of a steady stream).  Not templates: asm operands in a kernel template have cost the
+// kernel its host-side stub before.
+__device__ __forceinline__ void cols_load16(i32x4& d, const void* p)
+{
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void cols_load16_at16(i32x4& d, const void* p)
+{
+    asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=v"(d) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void cols_load16_at256(i32x4& d, const void* p)
+{
+    asm volatile("global_load_dwordx4 %0, %1, off offset:256" : "=v"(d) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void cols_load4(float& d, const void* p)
+{
+    asm volatile("global_load_dword %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void cols_load4(int32_t& d, const void* p)
+{
+    asm volatile("global_load_dword %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+}
+constexpr int kColsLoadsPerStage = 8; // cols_issue's loads, counted by cols_wait_oldest
+// the stage requested kColsDepth - 1 stages ago has arrived once at most (kColsDepth - 1) *
+// kColsLoadsPerStage = 56 younger loads are outstanding (loads return in order); the stage's
+// registers are operands so that nothing that reads them is moved above the wait
+__device__ __forceinline__ void cols_wait_oldest(ColsStage& s)
+{
+    asm volatile("s_waitcnt vmcnt(56)"
+                 : "+v"(s.wlo), "+v"(s.whi), "+v"(s.xlo), "+v"(s.xhi), "+v"(s.xs), "+v"(s.sw), "+v"(s.ws), "+v"(s.tok)
+                 :
+                 : "memory");
+}
+__device__ __forceinline__ void cols_drain() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+static_assert((kColsDepth - 1) * kColsLoadsPerStage == 56, "cols_wait_oldest counts 56 younger loads");
+
+template <In16 DT>
+__global__ __launch_bounds__(256) void moe_down_cols_kernel(DownColsParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) uint32_t cols_lds[];
+    __shared__ int n_units_s;
+    uint32_t*      unit_a = cols_lds;                    // block << 1 | half
+    uint32_t*      unit_b = cols_lds + 2 * p.max_blocks; // expert << 16 | the half's row mask
+    float*         acc    = (float*)(cols_lds + 4 * p.max_blocks); // [kblocks][M + 16][16], rows M.. are spares
+    const int      t = threadIdx.x, lane = t & 63, kb = t >> 6, l16 = lane & 15, kg = lane >> 4;
+
+    if(kb == 0) // list the units in sorted order
+    {
+        const int nv    = p.num_valid[0];
+        int       valid = (nv + 31) / 32;
+        valid           = valid < p.max_blocks ? valid : p.max_blocks;
+        int      e[kColsMaxBlocks / 64];
+        uint32_t m[kColsMaxBlocks / 64];
+#pragma unroll
+        for(int c = 0; c < kColsMaxBlocks / 64; ++c)
+        {
+            const int b = c * 64 + lane;
+            e[c]        = b < valid ? p.sorted_expert_ids[b] : -1;
+            m[c]        = b < valid ? p.block_mask[b] : 0u;
+        }
+        int            base = 0;
+        const uint64_t below = ((uint64_t)1 << lane) - 1;
+#pragma unroll
+        for(int c = 0; c < kColsMaxBlocks / 64; ++c)
+        {
+            const bool     ok = e[c] >= 0 && e[c] < p.experts;
+            const bool     h0 = ok && (m[c] & 0xffffu) != 0, h1 = ok && (m[c] >> 16) != 0;
+            const uint64_t b0 = __ballot(h0), b1 = __ballot(h1);
+            int            at = base + __popcll(b0 & below) + __popcll(b1 & below);
+            const uint32_t b  = (uint32_t)(c * 64 + lane);
+            if(h0)
+            {
+                unit_a[at] = b << 1;
+                unit_b[at] = (uint32_t)e[c] << 16 | (m[c] & 0xffffu);
+                ++at;
+            }
+            if(h1)
+            {
+                unit_a[at] = b << 1 | 1u;
+                unit_b[at] = (uint32_t)e[c] << 16 | (m[c] >> 16);
+            }
+            base += __popcll(b0) + __popcll(b1);
+        }
+        if(lane == 0)
+            n_units_s = base;
+    }
+    for(int i = t; i < p.kblocks * (p.M + 16) * 16; i += blockDim.x)
+        acc[i] = 0.f;
+    __syncthreads();
+    const int units = n_units_s;
+
+    const int      n0     = blockIdx.x * 16;
+    const size_t   wexp   = (size_t)p.N * (size_t)p.K;
+    const uint8_t* wlane  = p.w + (size_t)blockIdx.x * 16 * (size_t)p.K + (size_t)kb * 2048 + kg * 512 + l16 * 16;
+    const float*   wslane = p.wsc + (size_t)(n0 / 128) * p.kblocks + kb;
+    const size_t   wsexp  = (size_t)(p.N / 128) * p.kblocks;
+    float*         mine   = acc + (size_t)kb * (p.M + 16) * 16 + kg * 4;
+
+    // The walk is free of branches (the compiler then keeps the requested depth of loads in flight):
+    // past the last unit the last unit is requested again and its product goes to spare rows.
+    auto issue = [&](ColsStage& s, int u) {
+        u = u < units ? u : units - 1;
+        const uint32_t a = __builtin_amdgcn_readfirstlane(unit_a[u]);
+        const uint32_t b = __builtin_amdgcn_readfirstlane(unit_b[u]);
+        const int      expert = (int)(b >> 16);
+        s.mask                = b & 0xffffu;
+        const uint8_t* wp     = wlane + (size_t)expert * wexp;
+        cols_load16(s.wlo, wp);
+        cols_load16_at256(s.whi, wp);
+        cols_load4(s.ws, wslane + (size_t)expert * wsexp);
+        // rows that are padding read the unit's first real row instead: same cache lines, no traffic
+        const int    row  = (s.mask >> l16) & 1u ? l16 : __builtin_ctz(s.mask);
+        const size_t slot = (size_t)(a >> 1) * 32 + (a & 1u) * 16 + row;
+        const uint8_t* xp = p.xq + slot * (size_t)p.K + (size_t)kb * 128 + kg * 32;
+        cols_load16(s.xlo, xp);
+        cols_load16_at16(s.xhi, xp);
+        cols_load4(s.xs, p.xs + slot * p.kblocks + kb);
+        cols_load4(s.sw, p.sorted_weights + slot);
+        cols_load4(s.tok, p.sorted_ids + slot);
+    };
+    auto consume = [&](ColsStage& s, bool live) {
+        cols_wait_oldest(s);
+        const i32x8 w = i32x8{s.wlo[0], s.wlo[1], s.wlo[2], s.wlo[3], s.whi[0], s.whi[1], s.whi[2], s.whi[3]};
+        const i32x8 x = i32x8{s.xlo[0], s.xlo[1], s.xlo[2], s.xlo[3], s.xhi[0], s.xhi[1], s.xhi[2], s.xhi[3]};
+        const f32x4 prod = mfma_16x16x128_fp8(w, x, f32x4{0.f, 0.f, 0.f, 0.f});
+        // Padding rows go to a spare row per lane.  The table update is a plain read-add-write (LDS
+        // float atomics cost 0.3 us per instruction here): right as long as the 16 rows of a unit are
+        // 16 different tokens.  A routing that names an expert twice for a token puts the two pairs
+        // next to each other in the sorted order; such a unit is added one row at a time.
+        const bool  real = live && ((s.mask >> l16) & 1u);
+        const int   key  = real ? (s.tok & 0xffffff) : -1 - l16;
+        const int   prev = __builtin_amdgcn_update_dpp(-100, key, 0x111 /* row_shr:1 */, 0xf, 0xf, false);
+        const int   row  = real ? key : p.M + l16;
+        const float sc   = s.xs * s.ws;
+        float*      dst  = mine + (size_t)row * 16;
+        f32x4       add;
+#pragma unroll
+        for(int c = 0; c < 4; ++c)
+            add[c] = prod[c] * sc * s.sw;
+        if(__builtin_expect(__ballot(real && prev == key) == 0, 1))
+        {
+            f32x4 cur = *(f32x4*)dst;
+            cur += add;
+            *(f32x4*)dst = cur;
+        }
+        else
+        {
+            for(int r = 0; r < 16; ++r)
+            {
+                // rows of one token share `dst`: each row's read has to follow the previous row's
+                // write, which a compiler that reasons per lane is free to undo without this
+                asm volatile("" ::: "memory");
+                if(l16 == r)
+                {
+                    f32x4 cur = *(volatile f32x4*)dst;
+                    cur += add;
+                    *(volatile f32x4*)dst = cur;
+                }
+            }
+        }
+    };
+
+    if(units > 0)
+    {
+        ColsStage st[kColsDepth];
+#pragma unroll
+        for(int d = 0; d < kColsDepth; ++d)
+            issue(st[d], d);
+        for(int u0 = 0; u0 < units; u0 += kColsDepth)
+        {
+#pragma unroll
+            for(int d = 0; d < kColsDepth; ++d)
+            {
+                consume(st[d], u0 + d < units);
+                issue(st[d], u0 + d + kColsDepth);
+            }
+        }
+        cols_drain(); // requests past the last unit are still on their way to registers
+    }
+    __syncthreads();
+
+    // out[token][n0 .. n0+16) += the tables, K blocks in order
+    for(int i = t; i < p.M * 4; i += blockDim.x)
+    {
+        const int tok = i >> 2, q = i & 3;
+        f32x4     sum = f32x4{0.f, 0.f, 0.f, 0.f};
+        for(int k = 0; k < p.kblocks; ++k)
+            sum += *(const f32x4*)(acc + ((size_t)k * (p.M + 16) + tok) * 16 + q * 4);
+        uint16_t*   dst  = p.out + (size_t)tok * p.out_stride + n0 + q * 4;
+        const u32x2 prev = *(const u32x2*)dst;
+        float       o[4];
+        if constexpr(DT == In16::bf16)
+        {
+            o[0] = __uint_as_float(prev[0] << 16);
+            o[1] = __uint_as_float(prev[0] & 0xffff0000u);
+            o[2] = __uint_as_float(prev[1] << 16);
+            o[3] = __uint_as_float(prev[1] & 0xffff0000u);
+        }
+        else
+        {
+            o[0] = (float)__builtin_bit_cast(_Float16, (unsigned short)(prev[0] & 0xffffu));
+            o[1] = (float)__builtin_bit_cast(_Float16, (unsigned short)(prev[0] >> 16));
+            o[2] = (float)__builtin_bit_cast(_Float16, (unsigned short)(prev[1] & 0xffffu));
+            o[3] = (float)__builtin_bit_cast(_Float16, (unsigned short)(prev[1] >> 16));
+        }
+        *(u32x2*)dst = u32x2{pack2<DT>(o[0] + sum[0], o[1] + sum[1]), pack2<DT>(o[2] + sum[2], o[3] + sum[3])};
+    }
+}
+
 // out[token] += sum over the token's slots, in slot order, of weight * y[sorted position]
 template <In16 DT, bool Y32>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const void* __restrict__ y, const float* __restrict__ sorted_weights,
@@ -843,6 +1100,21 @@ size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 // them between the weight reads costs 5 % of the layer's time in fp32.
 bool rows_in_f32(const MoeArgs& a) { return (size_t)a.M * a.topk * a.dim * 4 <= ((size_t)32 << 20); }
 
+// Decode-size batches take the second GEMM that owns output columns and sums per token in LDS
+// (moe_down_cols_kernel): its tables, [inter/128][tokens + 16][16] fp32, and its unit list have to fit
+// 64 KiB of LDS.  Beyond, rows go through memory and moe_combine_kernel adds them.  down_mode 1 / 2
+// force the one / the other (2 only where it fits).
+bool down_by_columns(const MoeArgs& a)
+{
+    const int  kblocks = a.inter / 128;
+    const bool fits    = kblocks <= 4 && (size_t)kblocks * (a.M + 16) * 64 <= ((size_t)48 << 10) &&
+                      a.max_blocks <= kColsMaxBlocks && a.dim % 16 == 0;
+    if(a.down_mode == 1 || !fits)
+        return false;
+    // measured on the DeepSeek-V3 layer: 12 % faster at 1 token, 1-2 % up to 128, slower from 256
+    return a.down_mode == 2 || a.M <= 128;
+}
+
 } // namespace
 
 hipError_t launch_topk_softmax(const TopkSoftmaxArgs& a, hipStream_t stream)
@@ -927,6 +1199,7 @@ size_t moe_workspace_bytes(const MoeArgs& a)
     b += align_up(slots * (a.inter / 128) * 4);  // its scales
     b += align_up(slots * a.dim * (rows_in_f32(a) ? 4 : 2)); // second GEMM's rows
     b += align_up((size_t)a.M * a.topk * 4);     // sorted position of each (token, slot)
+    b += align_up((size_t)a.max_blocks * 4);     // real rows of each block
     if(a.x16)
     {
         b += align_up((size_t)a.M * a.dim);             // quantised tokens
@@ -955,6 +1228,10 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     ws += align_up(slots * a.dim * (y32 ? 4 : 2));
     int32_t* where = (int32_t*)ws; // sorted position of each (token, slot) pair, -1 = not routed here
     ws += align_up((size_t)a.M * a.topk * 4);
+    uint32_t* block_mask = (uint32_t*)ws;
+    ws += align_up((size_t)a.max_blocks * 4);
+    const bool cols = down_by_columns(a);
+    if(!cols)
     {
         const size_t n = (size_t)a.M * a.topk;
         unsigned     g = (unsigned)((n + 255) / 256);
@@ -1003,7 +1280,8 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     p.kblocks           = a.dim / 128;
 
     p.topk              = a.topk;
-    p.where             = where;
+    p.where             = cols ? nullptr : where;
+    p.block_mask        = block_mask;
     p.max_blocks        = a.max_blocks;
     p.experts           = a.experts;
     p.activation        = a.activation;
@@ -1039,6 +1317,35 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     e                  = launch_group_quant(qa, stream);
     if(e != hipSuccess)
         return e;
+
+    if(cols)
+    {
+        DownColsParams c{};
+        c.xq                = hq;
+        c.xs                = hs;
+        c.w                 = a.w2;
+        c.wsc               = a.w2_scale;
+        c.sorted_ids        = a.sorted_ids;
+        c.sorted_weights    = a.sorted_weights;
+        c.sorted_expert_ids = a.sorted_expert_ids;
+        c.num_valid         = a.num_valid;
+        c.block_mask        = block_mask;
+        c.out               = (uint16_t*)a.out;
+        c.out_stride        = a.out_stride;
+        c.M                 = a.M;
+        c.K                 = a.inter;
+        c.N                 = a.dim;
+        c.kblocks           = a.inter / 128;
+        c.max_blocks        = a.max_blocks;
+        c.experts           = a.experts;
+        const size_t lds    = (size_t)a.max_blocks * 16 + (size_t)c.kblocks * (a.M + 16) * 64;
+        const dim3   grid((unsigned)(a.dim / 16)), block((unsigned)(64 * c.kblocks));
+        if(a.out_dtype == In16::bf16)
+            hipLaunchKernelGGL(moe_down_cols_kernel<In16::bf16>, grid, block, lds, stream, c);
+        else
+            hipLaunchKernelGGL(moe_down_cols_kernel<In16::fp16>, grid, block, lds, stream, c);
+        return hipGetLastError();
+    }
 
     MoeGemmParams d = p;
     d.xq            = hq;

@@ -229,9 +229,11 @@ int moe_sorting_fwd(aiter_tensor_t* topk_ids, aiter_tensor_t* topk_weights, aite
  *   the four sorted arrays as moe_sorting_fwd writes them with unit_size 32
  *   activation 0 = silu, 1 = gelu; fc_scale_blkn = fc_scale_blkk = 128; block_size_M = 32;
  *   fc2_smooth_scale must be NULL; kernel_name names the reference's tuned kernels and is only a
- *   tuning hint here ("nt=1|2|4", "dw=2|4|8", "dc=2|4|8"; anything else: choose).
+ *   tuning hint here ("nt=1|2|4", "dw=2|4|8", "dc=2|4|8", "down=rows", "down=cols"; anything
+ *   else: choose).
  * The product of the first GEMM is quantised 1x128 to fp8 for the second.  Each token's k
- * contributions are added in slot order: results do not depend on timing.  Scratch memory is
+ * contributions are added in a fixed order (sorted order up to 128 tokens, slot order beyond):
+ * results do not depend on timing.  Scratch memory is
  * allocated by the library on first use and grown on demand.
  */
 int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_tensor_t* gate, aiter_tensor_t* down,

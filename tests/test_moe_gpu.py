@@ -160,16 +160,24 @@ def make_moe(tokens, dim, inter, experts, topk, seed, w_std=0.1):
     return dict(x=x, aq=aq, asc=asc, w1q=w1q, w1s=w1s, w2q=w2q, w2s=w2s, tw=tw, ti=ti)
 
 
-def run_moe(p, dtype=torch.bfloat16, activation=aiter_amd.ActivationType.Silu, expert_mask=None, bf16_input=False):
+def run_moe(p, dtype=torch.bfloat16, activation=aiter_amd.ActivationType.Silu, expert_mask=None, bf16_input=False,
+            kernel_name=""):
     w1 = aiter_amd.shuffle_weight(p["w1q"].view(torch.uint8)).view(dtypes.fp8)
     w2 = aiter_amd.shuffle_weight(p["w2q"].view(torch.uint8)).view(dtypes.fp8)
     if bf16_input:
         a, a_scale = p["x"], None
     else:
         a, a_scale = p["aq"].to(DEV), p["asc"].t().contiguous().to(DEV)
-    out = aiter_amd.fused_moe_blockscale(a, w1, w2, p["tw"].to(DEV), p["ti"].to(DEV), p["w1s"], p["w2s"], a_scale,
-                                         dtype=dtype, activation=activation,
-                                         expert_mask=expert_mask.to(DEV) if expert_mask is not None else None)
+    mask = expert_mask.to(DEV) if expert_mask is not None else None
+    if not kernel_name:
+        out = aiter_amd.fused_moe_blockscale(a, w1, w2, p["tw"].to(DEV), p["ti"].to(DEV), p["w1s"], p["w2s"], a_scale,
+                                             dtype=dtype, activation=activation, expert_mask=mask)
+    else:  # the same call sequence with a kernel hint
+        ti, tw = p["ti"].to(DEV), p["tw"].to(DEV)
+        E = w1.shape[0] if mask is None else mask.numel()
+        s_ids, s_w, s_e, nv, out = aiter_amd.moe_sorting(ti, tw, E, a.shape[1], dtype, expert_mask=mask)
+        aiter_amd.fmoe_fp8_blockscale_g1u1(out, a, w1, w2, s_ids, s_w, s_e, nv, ti.shape[1], a_scale, p["w1s"],
+                                           p["w2s"], kernel_name, 128, 128, None, int(activation))
     torch.cuda.synchronize()
     return out
 
@@ -206,7 +214,23 @@ def test_fmoe_reference_shapes(tokens):
                                                            (300, 256, 128, 4, 1), (33, 2048, 512, 16, 6)])
 def test_fmoe_other_shapes(tokens, dim, inter, experts, topk):
     p = make_moe(tokens, dim, inter, experts, topk, seed=dim + inter)
-    assert_close(run_moe(p), reference(p), f"{tokens}x{dim}x{inter} E={experts} k={topk}")
+    refs = reference(p)
+    assert_close(run_moe(p), refs, f"{tokens}x{dim}x{inter} E={experts} k={topk}")
+    # both second GEMMs: the one that sums per token in LDS (chosen up to 128 tokens) and the one
+    # that writes rows and adds them in a further kernel
+    assert_close(run_moe(p, kernel_name="down=rows"), refs, f"{tokens}x{dim}x{inter} E={experts} k={topk}, rows")
+    assert_close(run_moe(p, kernel_name="down=cols"), refs, f"{tokens}x{dim}x{inter} E={experts} k={topk}, cols")
+
+
+def test_fmoe_both_second_gemms_on_the_reference_shape():
+    p = make_moe(48, 7168, 256, 32, 8, seed=3)
+    refs = reference(p)
+    by_columns, by_rows = run_moe(p), run_moe(p, kernel_name="down=rows")
+    assert torch.equal(by_columns.view(torch.int16), run_moe(p, kernel_name="down=cols").view(torch.int16))
+    assert_close(by_columns, refs, "per-token sum in LDS")
+    assert_close(by_rows, refs, "rows through memory")
+    # same products, summed in a different order
+    assert ((by_columns.float() - by_rows.float()).norm() / by_rows.float().norm()).item() < 4e-3
 
 
 def test_fmoe_many_tokens_sampled_rows():
@@ -227,6 +251,19 @@ def test_fmoe_many_tokens_sampled_rows():
     assert ((o - plain).norm() / plain.norm()).item() < 3e-2
 
 
+def test_fmoe_routing_that_repeats_an_expert_for_a_token():
+    # the reference accumulates with atomics, so a token may name an expert more than once; here the
+    # two pairs sit next to each other in a block and must both be added
+    p = make_moe(40, 512, 256, 8, 4, seed=13)
+    ti = p["ti"].clone()
+    ti[::3, 1] = ti[::3, 0]
+    ti[5, :] = ti[5, 0]  # the same expert four times
+    p = dict(p, ti=ti)
+    refs = reference(p)
+    assert_close(run_moe(p), refs, "repeated expert, per-token sum in LDS")
+    assert_close(run_moe(p, kernel_name="down=rows"), refs, "repeated expert, rows through memory")
+
+
 @pytest.mark.parametrize("hint", ["nt=1", "nt=2", "nt=4", "dw=2", "dw=8", "dc=4"])
 def test_fmoe_tuning_hints_do_not_change_the_result(hint):
     # 300 tokens on 4 experts: runs of many blocks per expert, partly filled last blocks
@@ -234,7 +271,8 @@ def test_fmoe_tuning_hints_do_not_change_the_result(hint):
     w1 = aiter_amd.shuffle_weight(p["w1q"].view(torch.uint8)).view(dtypes.fp8)
     w2 = aiter_amd.shuffle_weight(p["w2q"].view(torch.uint8)).view(dtypes.fp8)
     outs = []
-    for name in ("", hint):
+    # "dw=" / "dc=" shape the second GEMM that writes rows: compare with that kernel's default shape
+    for name in ("down=rows" if hint[0] == "d" else "", hint):
         s_ids, s_w, s_e, nv, out = aiter_amd.moe_sorting(p["ti"].to(DEV), p["tw"].to(DEV), 4, 512, torch.bfloat16)
         aiter_amd.fmoe_fp8_blockscale_g1u1(out, p["aq"].to(DEV), w1, w2, s_ids, s_w, s_e, nv, 2,
                                            p["asc"].t().contiguous().to(DEV), p["w1s"], p["w2s"], name)
