@@ -825,7 +825,15 @@ __device__ __forceinline__ void cols_wait_oldest(ColsStage& s)
                  :
                  : "memory");
 }
-__device__ __forceinline__ void cols_drain() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// waits for every outstanding load; the stage's registers are operands so that they count as
+// occupied until then (a request past the last unit is still on its way into them after the walk)
+__device__ __forceinline__ void cols_drain(ColsStage& s)
+{
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(s.wlo), "+v"(s.whi), "+v"(s.xlo), "+v"(s.xhi), "+v"(s.xs), "+v"(s.sw), "+v"(s.ws), "+v"(s.tok)
+                 :
+                 : "memory");
+}
 static_assert((kColsDepth - 1) * kColsLoadsPerStage == 56, "cols_wait_oldest counts 56 younger loads");
 
 template <In16 DT>
@@ -969,7 +977,9 @@ __global__ __launch_bounds__(256) void moe_down_cols_kernel(DownColsParams p)
                 issue(st[d], u0 + d + kColsDepth);
             }
         }
-        cols_drain(); // requests past the last unit are still on their way to registers
+#pragma unroll
+        for(int d = 0; d < kColsDepth; ++d)
+            cols_drain(st[d]);
     }
     __syncthreads();
 
