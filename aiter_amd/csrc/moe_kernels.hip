@@ -317,36 +317,106 @@ __global__ __launch_bounds__(64) void moe_sort_scatter_kernel(SortParams p)
     scatter_chunk(p, ids, wts, begin, running, cnt, lo);
 }
 
-// All of it in one workgroup, for up to kSortChunk pairs (the decode regime): histogram in LDS,
-// a serial scan over the experts, then thread e walks the pairs for expert e.
+// All of it in one workgroup, for up to kSortChunk pairs (the decode regime).  The pairs are cut
+// into kSortWaves contiguous runs, one per wave: histograms per run (LDS), a scan over the experts
+// and, per expert, over the runs, then every wave scatters its own run, starting each expert at
+// the fill level the earlier runs leave -- the (token, slot) order of the pairs is kept.
+constexpr int kSortWaves = 8;
+constexpr int kSortRunSteps = kSortChunk / kSortWaves / 64; // 64-pair steps of the longest run
+
+// scatter_chunk for one run of the one-workgroup sort: the weights come from memory, all of the
+// run's requested before the first step (they would otherwise cost a round trip per step)
+__device__ __forceinline__ void scatter_run(const SortParams& p, const int32_t* ids, const int32_t* begin,
+                                            int32_t* running, int cnt, int first)
+{
+    const int lane = threadIdx.x & 63;
+    float     w[kSortRunSteps];
+#pragma unroll
+    for(int st = 0; st < kSortRunSteps; ++st)
+    {
+        const int f = first + st * 64 + lane;
+        w[st]       = st * 64 + lane < cnt ? p.topk_weights[(size_t)(f / p.topk) * p.w_stride + (f % p.topk)] : 0.f;
+    }
+#pragma unroll
+    for(int st = 0; st < kSortRunSteps; ++st)
+    {
+        if(st * 64 >= cnt)
+            break;
+        const int  i  = st * 64 + lane;
+        const int  e  = i < cnt ? ids[i] : -1;
+        const bool in = e >= 0 && e < p.experts && begin[e] >= 0;
+        uint64_t   same = __ballot(in);
+#pragma unroll
+        for(int b = 0; b < 10; ++b)
+        {
+            const uint64_t bal = __ballot((e >> b) & 1);
+            same &= ((e >> b) & 1) ? bal : ~bal;
+        }
+        if(in)
+        {
+            const int     rank = __popcll(same & ((1ull << lane) - 1ull));
+            const int     n    = __popcll(same);
+            const int32_t fill = running[e];
+            const int32_t at   = begin[e] + fill + rank;
+            const int     f    = first + i;
+            p.sorted_ids[at]     = ((int32_t)(f % p.topk) << 24) | (int32_t)(f / p.topk);
+            p.sorted_weights[at] = w[st];
+            if(rank == n - 1)
+                running[e] = fill + n;
+        }
+    }
+}
+
 __global__ __launch_bounds__(1024) void moe_sort_single_kernel(SortParams p)
 {
     __shared__ int32_t ids[kSortChunk];
-    __shared__ float   wts[kSortChunk];
+    __shared__ int32_t fill[kSortWaves][1024]; // per run: the expert's count, then its fill level
     __shared__ int32_t count[1024], begin[1024], local[1024];
     __shared__ int32_t s_total;
     const int rows = sort_rows(p);
     const int cnt  = rows * p.topk; // <= kSortChunk, checked at launch
-    for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
-        count[e] = 0;
+    const int run_len = ((cnt + kSortWaves - 1) / kSortWaves + 63) / 64 * 64;
+    for(int i = threadIdx.x; i < kSortWaves * 1024; i += blockDim.x)
+        (&fill[0][0])[i] = 0;
     __syncthreads();
     for(int i = threadIdx.x; i < cnt; i += blockDim.x)
     {
         const int     r = i / p.topk, k = i - r * p.topk;
         const int32_t e = p.topk_ids[(size_t)r * p.id_stride + k];
         ids[i]          = e;
-        wts[i]          = p.topk_weights[(size_t)r * p.w_stride + k];
         if(e >= 0 && e < p.experts)
-            atomicAdd(&count[e], 1);
+            atomicAdd(&fill[i / run_len][e], 1);
     }
     __syncthreads();
+    if((int)threadIdx.x < p.experts)
+    {
+        int32_t run = 0;
+#pragma unroll
+        for(int w = 0; w < kSortWaves; ++w)
+        {
+            const int32_t n       = fill[w][threadIdx.x];
+            fill[w][threadIdx.x] = run;
+            run += n;
+        }
+        count[threadIdx.x] = run;
+    }
     const bool       live_e = (int)threadIdx.x < p.experts && !(p.expert_mask && p.expert_mask[threadIdx.x] == 0);
     const int32_t    len_e  = (int)threadIdx.x < p.experts ? (count[threadIdx.x] + p.unit - 1) / p.unit * p.unit : 0;
     const ExpertSpan span   = expert_spans(live_e, len_e);
+    const int32_t pad_id    = (p.topk << 24) | p.M;
     if((int)threadIdx.x < p.experts)
     {
         begin[threadIdx.x] = span.begin;
-        local[threadIdx.x] = span.local;
+        if(span.begin >= 0)
+        {
+            for(int b = 0; b < len_e / p.unit; ++b)
+                p.sorted_expert_ids[span.begin / p.unit + b] = span.local;
+            for(int32_t at = span.begin + count[threadIdx.x]; at < span.begin + len_e; ++at)
+            {
+                p.sorted_ids[at]     = pad_id;
+                p.sorted_weights[at] = 0.f;
+            }
+        }
     }
     if(threadIdx.x == 0)
     {
@@ -355,28 +425,15 @@ __global__ __launch_bounds__(1024) void moe_sort_single_kernel(SortParams p)
         p.num_valid_ids[1] = rows;
     }
     __syncthreads();
-    const int32_t total  = s_total;
-    const int32_t pad_id = (p.topk << 24) | p.M;
-    for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
+    const int32_t total = s_total;
+    const int     wave  = threadIdx.x >> 6;
+    if(wave < kSortWaves)
     {
-        const int32_t b0 = begin[e];
-        if(b0 < 0)
-            continue;
-        const int32_t len = (count[e] + p.unit - 1) / p.unit * p.unit;
-        for(int b = 0; b < len / p.unit; ++b)
-            p.sorted_expert_ids[b0 / p.unit + b] = local[e];
-        for(int32_t at = b0 + count[e]; at < b0 + len; ++at)
-        {
-            p.sorted_ids[at]     = pad_id;
-            p.sorted_weights[at] = 0.f;
-        }
+        const int lo = wave * run_len;
+        const int n  = cnt - lo < run_len ? cnt - lo : run_len;
+        if(n > 0)
+            scatter_run(p, ids + lo, begin, fill[wave], n, lo);
     }
-    __syncthreads();
-    for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
-        local[e] = 0; // from here on: the expert's fill level
-    __syncthreads();
-    if(threadIdx.x < 64)
-        scatter_chunk(p, ids, wts, begin, local, cnt, 0);
     for(int b = total / p.unit + threadIdx.x; b < p.max_blocks; b += blockDim.x)
         p.sorted_expert_ids[b] = -1;
     for(int i = total + threadIdx.x; i < p.max_padded; i += blockDim.x)
