@@ -871,7 +871,7 @@ __device__ __forceinline__ void cols_load4(int32_t& d, const void* p)
 {
     asm volatile("global_load_dword %0, %1, off" : "=v"(d) : "v"(p) : "memory");
 }
-constexpr int kColsLoadsPerStage = 8; // cols_issue's loads, counted by cols_wait_oldest
+constexpr int kColsLoadsPerStage = 8; // loads the walk requests per unit, counted by cols_wait_oldest
 // the stage requested kColsDepth - 1 stages ago has arrived once at most (kColsDepth - 1) *
 // kColsLoadsPerStage = 56 younger loads are outstanding (loads return in order); the stage's
 // registers are operands so that nothing that reads them is moved above the wait
@@ -1168,13 +1168,13 @@ size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 bool rows_in_f32(const MoeArgs& a) { return (size_t)a.M * a.topk * a.dim * 4 <= ((size_t)32 << 20); }
 
 // Decode-size batches take the second GEMM that owns output columns and sums per token in LDS
-// (moe_down_cols_kernel): its tables, [inter/128][tokens + 16][16] fp32, and its unit list have to fit
-// 64 KiB of LDS.  Beyond, rows go through memory and moe_combine_kernel adds them.  down_mode 1 / 2
+// (moe_down_cols_kernel): its tables, [inter/128][tokens + 16][16] fp32 (at most 44 KiB), and its unit list
+// (16 bytes per block, at most 16 KiB) have to fit 64 KiB of LDS.  Beyond, rows go through memory and moe_combine_kernel adds them.  down_mode 1 / 2
 // force the one / the other (2 only where it fits).
 bool down_by_columns(const MoeArgs& a)
 {
     const int  kblocks = a.inter / 128;
-    const bool fits    = kblocks <= 4 && (size_t)kblocks * (a.M + 16) * 64 <= ((size_t)48 << 10) &&
+    const bool fits    = kblocks <= 4 && (size_t)kblocks * (a.M + 16) * 64 <= ((size_t)44 << 10) &&
                       a.max_blocks <= kColsMaxBlocks && a.dim % 16 == 0;
     if(a.down_mode == 1 || !fits)
         return false;
