@@ -1,0 +1,125 @@
+"""The reference's own test mains for this path, at their default shapes, with their data recipes
+and their pass criteria (and tighter ones where this library is exact):
+
+    op_tests/test_gemm_a8w8_blockscale.py:88-160,262-300   GEMM, M = 1 ... 10240 on (24576, 1536), both layouts
+    op_tests/test_quant.py:21-47,87-96                      1x128 quant, M = 1 ... 163840 on N = 4096, 8192
+    op_tests/test_rmsnorm2dFusedAddQuant.py:188-290,326-340 fused (add +) RMSNorm + 1x128 quant
+
+As there, the expected values are computed with torch on the GPU at run time."""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import aiter_amd
+from aiter_amd import dtypes
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+def check_allclose(a, b, rtol=1e-2, atol=1e-2, catastrophic=False):
+    """aiter/test_common.py:479-564: the fraction of elements outside the tolerance (0.0 if none);
+    with `catastrophic`, a non-finite value or a difference above half the reference's largest
+    magnitude raises, as there."""
+    close = torch.isclose(a, b, rtol=rtol, atol=atol)
+    if bool(close.all()):
+        return 0.0
+    if catastrophic:
+        assert bool(torch.isfinite(a).all()) and bool(torch.isfinite(b).all()), "non-finite values"
+        assert (a - b).abs().max().item() <= 0.5 * b.abs().max().item(), "catastrophic difference"
+    return (~close).sum().item() / a.numel()
+
+
+def torch_quant_1x128(x, group=128):
+    """get_torch_quant(per_1x128): pertoken_quant on [-1, 128] views (aiter/ops/quant.py:64-94, :331-346)."""
+    v = x.float().view(-1, group)
+    amax = v.abs().amax(dim=-1, keepdim=True)
+    scale = amax / 448.0
+    scale[scale == 0] = 1
+    return (v / scale).to(dtypes.fp8).view(x.shape), scale.view(*x.shape[:-1], x.shape[-1] // group)
+
+
+GEMM_M = [1, 2, 4, 8, 16, 32, 64, 96, 128, 160, 192, 224, 256, 288, 320, 352, 384, 416, 448, 480, 512, 1024, 2048,
+          4096, 6144, 8192, 10240]
+
+
+@pytest.mark.parametrize("m", GEMM_M)
+def test_gemm_grid(m):
+    n, k = 24576, 1536
+    g = torch.Generator(device=DEV).manual_seed(m)
+    x = (torch.rand((m, k), generator=g, device=DEV) / 10).to(dtypes.fp8)
+    weight = (torch.rand((n, k), generator=g, device=DEV) / 10).to(dtypes.fp8)
+    x_scale = torch.rand([m, k // 128], generator=g, device=DEV)
+    w_scale = torch.rand([n // 128, k // 128], generator=g, device=DEV)
+    # run_torch (:28-54)
+    xd = x.float() * x_scale.repeat_interleave(128, dim=1)
+    wd = weight.float() * w_scale.repeat_interleave(128, dim=0).repeat_interleave(128, dim=1)
+    want = F.linear(xd, wd).to(torch.bfloat16)
+    del xd, wd
+    got = aiter_amd.gemm_a8w8_blockscale(x, weight, x_scale, w_scale, torch.bfloat16)
+    assert check_allclose(want.float(), got.float(), catastrophic=True) <= 1e-4
+    # ck_preshuffle=True (:112-129): shuffled weight, transposed x_scale as a buffer and as a strided view
+    wsh = aiter_amd.shuffle_weight(weight, layout=(16, 16))
+    x_scale_t = x_scale.transpose(0, 1).contiguous().view(*x_scale.shape)
+    got_t = aiter_amd.gemm_a8w8_blockscale_bpreshuffle(x, wsh, x_scale_t, w_scale, torch.bfloat16)
+    assert check_allclose(want.float(), got_t.float(), catastrophic=True) <= 1e-4
+    x_scale_strided = x_scale.transpose(0, 1).contiguous().transpose(0, 1)
+    got_s = aiter_amd.gemm_a8w8_blockscale_bpreshuffle(x, wsh, x_scale_strided, w_scale, torch.bfloat16)
+    assert torch.equal(got_t, got_s)
+    # the reference's third route to the same operands (:138)
+    out = torch.empty_like(got_t)
+    aiter_amd.gemm_a8w8_blockscale_bpreshuffle_asm(x, wsh, out, x_scale_t, w_scale)
+    assert torch.equal(got_t, out)
+
+
+@pytest.mark.parametrize("h_dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n", [4096, 8192])
+@pytest.mark.parametrize("m", [1, 2, 16, 32, 64, 128, 192, 256, 512, 1024, 16384, 163840])
+def test_quant_grid(m, n, h_dtype):
+    g = torch.Generator(device=DEV).manual_seed(m + n)
+    x = torch.randn((m, n), generator=g, device=DEV).to(h_dtype)
+    ref, ref_scale = torch_quant_1x128(x)
+    out, scale = aiter_amd.get_hip_quant(aiter_amd.QuantType.per_1x128)(x, quant_dtype=dtypes.fp8)
+    # the reference's criteria: rtol = atol = 1e-3 on scales and codes, up to 5 % of the elements off
+    # (torch on the GPU divides through reciprocals: a scale is one step off here and there, and a
+    # quotient that sits on a rounding boundary lands on the other code -- a few per thousand)
+    assert check_allclose(ref_scale, scale, rtol=1e-3, atol=1e-3) == 0.0
+    assert check_allclose(ref.float(), out.float(), rtol=1e-3, atol=1e-3) < 0.01
+    # against the same definition evaluated with IEEE divisions (torch on the CPU): the same bits
+    rows = torch.arange(m) if m <= 1024 else torch.cat([torch.arange(64), torch.arange(m - 64, m)])
+    exact, exact_scale = torch_quant_1x128(x[rows.to(DEV)].cpu())
+    assert torch.equal(exact.view(torch.uint8), out[rows.to(DEV)].cpu().view(torch.uint8))
+    assert torch.equal(exact_scale.view(torch.int32), scale[rows.to(DEV)].cpu().view(torch.int32))
+
+
+@pytest.mark.parametrize("add_residual", [False, True])
+@pytest.mark.parametrize("n", [1024, 2048, 3584, 4096, 8192])
+@pytest.mark.parametrize("m", [8, 256, 256 * 8, 256 * 10, 32768])
+def test_rmsnorm_quant_grid(m, n, add_residual):
+    g = torch.Generator(device=DEV).manual_seed(m + n)
+    x = torch.randn((m, n), generator=g, device=DEV).bfloat16()
+    weight = torch.randn(n, generator=g, device=DEV).bfloat16()
+    res = torch.randn((m, n), generator=g, device=DEV).bfloat16() if add_residual else None
+    # run_torch (:23-55): optional add in the input dtype, F.rms_norm, 1x128 quant of the bf16 result
+    summed = x + res if add_residual else x
+    normed = F.rms_norm(summed, (n,), weight=weight, eps=1e-5)
+    a, yscale_a = torch_quant_1x128(normed)
+    c = torch.empty((m, n), dtype=dtypes.fp8, device=DEV)
+    yscale_c = torch.empty((m, n // 128), dtype=torch.float32, device=DEV)
+    if add_residual:
+        res_c = torch.empty_like(x)
+        aiter_amd.rmsnorm2d_fwd_with_add_dynamicquant(c, x, res, res_c, yscale_c, weight, 1e-5, 0, group_size=128)
+        assert torch.equal(summed, res_c)
+    else:
+        aiter_amd.rmsnorm2d_fwd_with_dynamicquant(c, x, yscale_c, weight, 1e-5, 0, group_size=128)
+    # the reference's criteria (:276-287): codes at atol 1e-2 with up to 5 % of the elements off, scales
+    # at the default 1e-2.  torch's own reduction order moves a bf16 value by one step now and then,
+    # and its fp8 code with it: well under 1 % of the elements.
+    assert check_allclose(a.float(), c.float(), rtol=0, atol=1e-2) < 0.01
+    assert check_allclose(yscale_a, yscale_c) == 0.0
+    # and the fused kernel is the unfused pair, bit for bit
+    n16 = torch.empty_like(x)
+    aiter_amd.rmsnorm(n16, summed, weight, 1e-5)
+    q, s = aiter_amd.per_group_quant_hip(n16)
+    assert torch.equal(q.view(torch.uint8), c.view(torch.uint8)) and torch.equal(s, yscale_c)
