@@ -694,9 +694,13 @@ int moe_sorting_fwd(aiter_tensor_t* topk_ids, aiter_tensor_t* topk_weights, aite
         same_device(fn, {topk_ids, topk_weights, sorted_token_ids, sorted_weights, sorted_expert_ids, num_valid_ids,
                          moe_buf, local_expert_mask, num_local_tokens});
         (void)dispatch_policy; // a tuning hint of the reference's kernels
-        if(topk_ids->ndim != 2 || topk_weights->ndim != 2 || topk_ids->shape[0] != topk_weights->shape[0] ||
-           topk_ids->shape[1] != topk_weights->shape[1])
-            fail(fn, "topk_ids and topk_weights must both be [tokens, topk]");
+        // with num_local_tokens the ids may carry more rows than are in use, and than the weights have
+        // (op_tests/test_moe_sorting.py:180-187)
+        if(topk_ids->ndim != 2 || topk_weights->ndim != 2 || topk_ids->shape[1] != topk_weights->shape[1] ||
+           (num_local_tokens ? topk_weights->shape[0] > topk_ids->shape[0]
+                             : topk_weights->shape[0] != topk_ids->shape[0]))
+            fail(fn, "topk_ids and topk_weights must both be [tokens, topk] (topk_weights may have fewer rows when "
+                     "num_local_tokens is given)");
         const int64_t M = topk_ids->shape[0], topk = topk_ids->shape[1];
         if(topk_ids->dtype_ != AITER_DTYPE_i32 || topk_weights->dtype_ != AITER_DTYPE_fp32)
             fail(fn, "topk_ids must be int32 and topk_weights fp32");
@@ -750,13 +754,14 @@ int moe_sorting_fwd(aiter_tensor_t* topk_ids, aiter_tensor_t* topk_weights, aite
         a.moe_buf           = buf_bytes ? moe_buf->ptr : nullptr;
         a.moe_buf_bytes     = buf_bytes;
         a.M                 = (int32_t)M;
+        a.w_rows            = (int32_t)topk_weights->shape[0];
         a.topk              = (int32_t)topk;
         a.experts           = (int32_t)num_experts;
         a.unit              = (int32_t)unit_size;
         a.max_padded        = (int32_t)max_padded;
         a.max_blocks        = (int32_t)max_blocks;
         a.id_stride         = M > 1 ? topk_ids->strides[0] : topk;
-        a.w_stride          = M > 1 ? topk_weights->strides[0] : topk;
+        a.w_stride          = topk_weights->shape[0] > 1 ? topk_weights->strides[0] : topk;
         a.device_id         = topk_ids->device_id;
         if(max_padded >= (1LL << 31))
             fail(fn, "problem too large");

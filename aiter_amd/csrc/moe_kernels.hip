@@ -143,6 +143,7 @@ struct SortParams
     int32_t*       counts; // workspace [chunks][experts]: counts, then positions
     int32_t*       expert_begin; // workspace [experts + 1]: start of each expert's padded run
     int32_t        M, topk, experts, unit, chunks;
+    int32_t        w_rows; // rows of topk_weights (may be fewer than M when num_local_tokens says so)
     int32_t        max_padded, max_blocks;
     int64_t        id_stride, w_stride;
 };
@@ -155,7 +156,7 @@ __device__ __forceinline__ int32_t sort_rows(const SortParams& p)
         const int32_t r = *p.num_local_tokens;
         rows            = r < 0 ? 0 : (r < rows ? r : rows);
     }
-    return rows;
+    return rows < p.w_rows ? rows : p.w_rows;
 }
 
 __global__ __launch_bounds__(1024) void moe_sort_count_kernel(SortParams p)
@@ -1220,6 +1221,7 @@ hipError_t launch_moe_sorting(const MoeSortArgs& a, hipStream_t stream)
     p.sorted_expert_ids = a.sorted_expert_ids;
     p.num_valid_ids     = a.num_valid_ids;
     p.M                 = a.M;
+    p.w_rows            = a.w_rows;
     p.topk              = a.topk;
     p.experts           = a.experts;
     p.unit              = a.unit;

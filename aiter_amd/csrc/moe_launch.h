@@ -31,6 +31,7 @@ struct MoeSortArgs
     void*          moe_buf;           // zeroed (may be null)
     size_t         moe_buf_bytes;     // multiple of 16
     int32_t        M, topk, experts, unit, max_padded, max_blocks;
+    int32_t        w_rows;            // rows of topk_weights, <= M
     int64_t        id_stride, w_stride;
     int            device_id;
 };

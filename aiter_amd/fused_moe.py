@@ -72,9 +72,16 @@ def fused_topk(hidden_states, gating_output, topk, renormalize, topk_ids=None, t
 
 
 def moe_sorting(topk_ids, topk_weights, num_experts, model_dim, moebuf_dtype, block_size=BLOCK_SIZE_M,
-                expert_mask=None, num_local_tokens=None, dispatch_policy=0):
+                expert_mask=None, num_local_tokens=None, dispatch_policy=0, return_local_topk_ids=False,
+                accumulate=True, flat=False, output_aux=False):
     """Returns (sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf), sized as the
-    reference sizes them; moe_buf [M, model_dim] comes back zeroed."""
+    reference sizes them (aiter/fused_moe.py:208-224); moe_buf [M, model_dim] comes back zeroed.  With
+    ``accumulate=False`` and no expert mask moe_buf is the reference's (0, 0) placeholder.  The
+    reference's other extras (local top-k ids, flat routing, auxiliary outputs) belong to kernels
+    outside this path."""
+    for name, value in (("return_local_topk_ids", return_local_topk_ids), ("flat", flat), ("output_aux", output_aux)):
+        if value:
+            raise NotImplementedError(f"moe_sorting: {name} is not part of this library")
     dev = topk_ids.device
     M, topk = topk_ids.shape
     max_num_tokens_padded = int(topk_ids.numel() + num_experts * block_size - topk)
@@ -83,7 +90,10 @@ def moe_sorting(topk_ids, topk_weights, num_experts, model_dim, moebuf_dtype, bl
     sorted_weights = torch.empty(max_num_tokens_padded, dtype=dtypes.fp32, device=dev)
     sorted_expert_ids = torch.empty(max_num_m_blocks, dtype=dtypes.i32, device=dev)
     num_valid_ids = torch.empty(2, dtype=dtypes.i32, device=dev)
-    moe_buf = torch.empty((M, model_dim), dtype=moebuf_dtype, device=dev)
+    if expert_mask is not None or accumulate:
+        moe_buf = torch.empty((M, model_dim), dtype=moebuf_dtype, device=dev)
+    else:
+        moe_buf = torch.empty((0, 0), dtype=moebuf_dtype, device=dev)
     moe_sorting_fwd(topk_ids, topk_weights, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf,
                     int(num_experts), int(block_size), expert_mask, num_local_tokens, int(dispatch_policy))
     return sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, moe_buf
