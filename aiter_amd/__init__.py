@@ -15,7 +15,9 @@ from .gemm_op_a8w8 import (
     gemm_a8w8_blockscale_bpreshuffle,
     gemm_a8w8_blockscale_bpreshuffle_asm,
     gemm_a8w8_blockscale_bpreshuffle_ck,
+    gemm_a8w8_blockscale_bpreshuffle_cktile,
     gemm_a8w8_blockscale_ck,
+    gemm_a8w8_blockscale_cktile,
     gemm_kernel_names,
 )
 from .shuffle import shuffle_weight
@@ -57,6 +59,8 @@ __all__ = [
     "dynamic_per_token_scaled_quant",
     "gemm_a8w8_blockscale",
     "gemm_a8w8_blockscale_ck",
+    "gemm_a8w8_blockscale_cktile",
+    "gemm_a8w8_blockscale_bpreshuffle_cktile",
     "gemm_kernel_names",
     "rmsnorm",
     "rmsnorm_quant",

@@ -39,7 +39,7 @@ def gemm_a8w8_blockscale_ck(
     """aiter/ops/gemm_op_a8w8.py:285-298: writes ``Out`` and returns it.  ``splitK`` is the log2
     of the number of K partitions (-1: the library chooses), ``kernelName`` one of
     :func:`gemm_kernel_names` or ""."""
-    _blockscale_into(XQ, WQ, x_scale, w_scale, Out, splitK, kernelName)
+    _blockscale_into(XQ, WQ, x_scale, w_scale, Out, splitK, _own_kernel_name(kernelName))
     return Out
 
 
@@ -100,8 +100,50 @@ def gemm_a8w8_blockscale_bpreshuffle_ck(
 ) -> Tensor:
     """aiter/ops/gemm_op_a8w8.py:318-330: ``WQ`` holds ``shuffle_weight(w, layout=(16, 16))`` and
     ``x_scale`` is column-major; writes ``Out`` and returns it."""
-    _bpreshuffle_into(XQ, WQ, x_scale, w_scale, Out, kernelName)
+    _bpreshuffle_into(XQ, WQ, x_scale, w_scale, Out, _own_kernel_name(kernelName))
     return Out
+
+
+def _own_kernel_name(kernelName: Optional[str]) -> str:
+    """The reference's tuned tables name kernels of its own zoo ("a8w8_blockscale_..."): tuning
+    hints that mean nothing here and are dropped (the library then chooses).  Anything else goes to
+    the library, which knows its own names and rejects the rest."""
+    name = kernelName or ""
+    return "" if name.startswith("a8w8_blockscale_") else name
+
+
+def gemm_a8w8_blockscale_cktile(
+    XQ: Tensor,
+    WQ: Tensor,
+    x_scale: Tensor,
+    w_scale: Tensor,
+    Out: Tensor,
+    isBpreshuffled: bool = False,
+    splitK: int = 0,
+    kernelName: str = "",
+) -> Tensor:
+    """aiter/ops/gemm_op_a8w8.py:301-315, the reference's second kernel family behind the same
+    operands (csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale_cktile.cu:62-93): row-major weights
+    and x_scale, or, with ``isBpreshuffled``, shuffled weights and column-major x_scale
+    (include/gemm_a8w8_blockscale_cktile_common.cuh:334-358).  One library serves both families."""
+    if isBpreshuffled:
+        _bpreshuffle_into(XQ, WQ, x_scale, w_scale, Out, _own_kernel_name(kernelName))
+    else:
+        _blockscale_into(XQ, WQ, x_scale, w_scale, Out, splitK, _own_kernel_name(kernelName))
+    return Out
+
+
+def gemm_a8w8_blockscale_bpreshuffle_cktile(
+    XQ: Tensor,
+    WQ: Tensor,
+    x_scale: Tensor,
+    w_scale: Tensor,
+    Out: Tensor,
+    isBpreshuffled: bool = True,
+    kernelName: str = "",
+) -> Tensor:
+    """aiter/ops/gemm_op_a8w8.py:333-346 (gemm_a8w8_blockscale_cktile.cu:96-107)."""
+    return gemm_a8w8_blockscale_cktile(XQ, WQ, x_scale, w_scale, Out, isBpreshuffled, 0, kernelName)
 
 
 def gemm_a8w8_blockscale_bpreshuffle_asm(
