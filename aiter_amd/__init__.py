@@ -40,7 +40,10 @@ from .quant import (
 from .rmsnorm import (
     add_rmsnorm,
     add_rmsnorm_quant,
+    rms_norm,
     rmsnorm,
+    rmsnorm2d_fwd,
+    rmsnorm2d_fwd_with_add,
     rmsnorm2d_fwd_with_add_dynamicquant,
     rmsnorm2d_fwd_with_dynamicquant,
     rmsnorm_quant,
@@ -64,6 +67,9 @@ __all__ = [
     "gemm_kernel_names",
     "rmsnorm",
     "rmsnorm_quant",
+    "rms_norm",
+    "rmsnorm2d_fwd",
+    "rmsnorm2d_fwd_with_add",
     "add_rmsnorm",
     "add_rmsnorm_quant",
     "rmsnorm2d_fwd_with_dynamicquant",

@@ -5,6 +5,7 @@
 
 from __future__ import annotations
 
+import torch
 from torch import Tensor
 
 from . import _ffi
@@ -79,6 +80,50 @@ def add_rmsnorm_quant(
         "add_rmsnorm_quant", out, input, residual_in, residual_out, scale, weight, float(epsilon),
         int(group_size), bool(shuffle_scale), bool(gemma_norm),
     )
+
+
+def _require_common(input: Tensor, use_model_sensitive_rmsnorm: int, what: str) -> None:
+    # aiter/ops/rmsnorm.py:386-397: the case the reference routes to module_rmsnorm_quant; the rest
+    # (fp32, hidden > 8192, the model-sensitive variant) goes to kernels outside this path
+    if use_model_sensitive_rmsnorm != 0 or input.element_size() != 2 or input.shape[-1] > 8192:
+        raise NotImplementedError(
+            f"{what}: only bf16/fp16 rows of up to 8192 elements with use_model_sensitive_rmsnorm=0 are part of "
+            "this library"
+        )
+
+
+def _rms_norm_fake(input, weight, epsilon, use_model_sensitive_rmsnorm=0):
+    return torch.empty_like(input)
+
+
+@torch_op("rms_norm(Tensor input, Tensor weight, float epsilon, int use_model_sensitive_rmsnorm=0) -> Tensor",
+          _rms_norm_fake)
+def rms_norm(input: Tensor, weight: Tensor, epsilon: float, use_model_sensitive_rmsnorm: int = 0) -> Tensor:
+    """aiter/ops/rmsnorm.py:415-423: returns a fresh tensor."""
+    _require_common(input, use_model_sensitive_rmsnorm, "rms_norm")
+    out = torch.empty_like(input)
+    _ffi.call("rmsnorm", out, input, weight, float(epsilon), False)
+    return out
+
+
+def rmsnorm2d_fwd(input: Tensor, weight: Tensor, epsilon: float, use_model_sensitive_rmsnorm: int = 0) -> Tensor:
+    """aiter/ops/rmsnorm.py:426-433."""
+    return rms_norm(input, weight, epsilon, use_model_sensitive_rmsnorm)
+
+
+def rmsnorm2d_fwd_with_add(
+    out: Tensor,
+    input: Tensor,
+    residual_in: Tensor,
+    residual_out: Tensor,
+    weight: Tensor,
+    epsilon: float,
+    gemma_norm: bool = False,
+    use_model_sensitive_rmsnorm: int = 0,
+) -> None:
+    """aiter/ops/rmsnorm.py:436-465: residual_out = input + residual_in, out = rmsnorm(residual_out)."""
+    _require_common(input, use_model_sensitive_rmsnorm, "rmsnorm2d_fwd_with_add")
+    add_rmsnorm(out, input, residual_in, residual_out, weight, epsilon, gemma_norm)
 
 
 def _require_grouped(yscale: Tensor, group_size: int, what: str) -> None:

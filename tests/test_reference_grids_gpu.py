@@ -148,9 +148,15 @@ def test_rmsnorm_quant_grid(m, n, add_residual):
     # and its fp8 code with it: well under 1 % of the elements.
     assert check_allclose(a.float(), c.float(), rtol=0, atol=1e-2) < 0.01
     assert check_allclose(yscale_a, yscale_c) == 0.0
-    # and the fused kernel is the unfused pair, bit for bit
-    n16 = torch.empty_like(x)
-    aiter_amd.rmsnorm(n16, summed, weight, 1e-5)
+    # and the fused kernel is the unfused pair, bit for bit (run_ck's plain calls, :66-84)
+    n16 = aiter_amd.rmsnorm2d_fwd(summed, weight, 1e-5)
+    if add_residual:
+        o2, r2 = torch.empty_like(x), torch.empty_like(x)
+        aiter_amd.rmsnorm2d_fwd_with_add(o2, x, res, r2, weight, 1e-5)
+        assert torch.equal(o2, n16) and torch.equal(r2, summed)
+    # against torch's own norm: the same bf16 value, or the neighbouring one where the sums round apart
+    step = (n16.view(torch.int16).int() - normed.view(torch.int16).int()).abs()
+    assert int(step.max()) <= 1 and (step != 0).float().mean().item() < 0.02
     q, s = aiter_amd.per_group_quant_hip(n16)
     assert torch.equal(q.view(torch.uint8), c.view(torch.uint8)) and torch.equal(s, yscale_c)
 

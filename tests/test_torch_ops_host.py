@@ -14,7 +14,7 @@ from aiter_amd import dtypes, torch_ops
 EXPECTED = {
     "dynamic_per_token_scaled_quant", "per_group_quant_hip", "gemm_a8w8_blockscale", "gemm_a8w8_blockscale_ck",
     "gemm_a8w8_blockscale_bpreshuffle", "gemm_a8w8_blockscale_bpreshuffle_ck", "rmsnorm", "rmsnorm_quant",
-    "add_rmsnorm", "add_rmsnorm_quant", "topk_softmax", "moe_sorting_fwd", "fmoe_fp8_blockscale_g1u1",
+    "add_rmsnorm", "add_rmsnorm_quant", "rms_norm", "topk_softmax", "moe_sorting_fwd", "fmoe_fp8_blockscale_g1u1",
 }
 
 
