@@ -15,7 +15,7 @@ import threading
 
 import torch
 
-from .dtypes import aiter_tensor_t, torch_to_aiter
+from .dtypes import aiter_tensor_t, shared_descriptor
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libaiter_fp8bs.so")
@@ -82,9 +82,15 @@ def load_library():
     return _lib
 
 
+# the raw handle of the current stream without building a torch.cuda.Stream object (2 us less per call)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _current_stream(device_index):
-    if device_index is None or device_index < 0 or not torch.cuda.is_available():
+    if device_index is None or device_index < 0:
         return None
+    if _raw_stream is not None:
+        return _raw_stream(device_index)
     return torch.cuda.current_stream(device_index).cuda_stream
 
 
@@ -98,7 +104,7 @@ def call(name: str, *args):
         if isinstance(a, torch.Tensor):
             if device is None and a.is_cuda:
                 device = a.device.index
-            at = torch_to_aiter(a)
+            at = shared_descriptor(a)
             keep.append(at)
             c_args.append(ctypes.byref(at))
         elif isinstance(a, str):
