@@ -29,7 +29,7 @@ namespace fp8bs {
 namespace {
 
 constexpr int kSortChunk = 4096;      // most (token, slot) pairs the one-workgroup sort takes
-constexpr int kSortChunkMulti = 1024; // pairs per workgroup of the three-launch sort
+constexpr int kSortChunkMulti = 1024; // most pairs per workgroup (chunk) of the three-launch sort
 
 __device__ __forceinline__ float wave_max(float v)
 {
@@ -143,7 +143,10 @@ struct SortParams
     int32_t*       counts; // workspace [chunks][experts]: counts, then positions
     int32_t*       expert_begin; // workspace [experts + 1]: start of each expert's padded run
     int32_t        M, topk, experts, unit, chunks;
+    int32_t        chunk_pairs; // pairs per chunk of the three-launch sort, <= kSortChunkMulti
     int32_t        w_rows; // rows of topk_weights (may be fewer than M when num_local_tokens says so)
+    u32x4*         zero_dst;  // buffer to clear (may be null), by the workgroups behind the sorting ones
+    size_t         zero_vecs; // its size in 16-byte units
     int32_t        max_padded, max_blocks;
     int64_t        id_stride, w_stride;
 };
@@ -159,15 +162,29 @@ __device__ __forceinline__ int32_t sort_rows(const SortParams& p)
     return rows < p.w_rows ? rows : p.w_rows;
 }
 
+// The output buffer of the expert layer has to come back zeroed.  Rather than a launch of its own,
+// the workgroups of the first sorting launch beyond the `first` that sort clear it.
+__device__ __forceinline__ void zero_slice(const SortParams& p, int first)
+{
+    const size_t workers = (size_t)(gridDim.x - first) * blockDim.x;
+    for(size_t i = (size_t)(blockIdx.x - first) * blockDim.x + threadIdx.x; i < p.zero_vecs; i += workers)
+        p.zero_dst[i] = u32x4{0u, 0u, 0u, 0u};
+}
+
 __global__ __launch_bounds__(1024) void moe_sort_count_kernel(SortParams p)
 {
+    if((int)blockIdx.x >= p.chunks)
+    {
+        zero_slice(p, p.chunks);
+        return;
+    }
     extern __shared__ int32_t hist[];
     for(int e = threadIdx.x; e < p.experts; e += blockDim.x)
         hist[e] = 0;
     __syncthreads();
     const int64_t n = (int64_t)sort_rows(p) * p.topk;
-    const int64_t lo = (int64_t)blockIdx.x * kSortChunkMulti;
-    for(int i = threadIdx.x; i < kSortChunkMulti; i += blockDim.x)
+    const int64_t lo = (int64_t)blockIdx.x * p.chunk_pairs;
+    for(int i = threadIdx.x; i < p.chunk_pairs; i += blockDim.x)
     {
         const int64_t f = lo + i;
         if(f >= n)
@@ -223,11 +240,19 @@ __global__ __launch_bounds__(1024) void moe_sort_scan_kernel(SortParams p)
     const int e   = threadIdx.x;
     int32_t   run = 0;
     if(e < p.experts)
-        for(int c = 0; c < p.chunks; ++c)
+        for(int c0 = 0; c0 < p.chunks; c0 += 8) // eight counts requested together: one round trip, not eight
         {
-            const int32_t n                       = p.counts[(size_t)c * p.experts + e];
-            p.counts[(size_t)c * p.experts + e] = run; // position inside the expert's run
-            run += n;
+            int32_t n[8];
+#pragma unroll
+            for(int i = 0; i < 8; ++i)
+                n[i] = c0 + i < p.chunks ? p.counts[(size_t)(c0 + i) * p.experts + e] : 0;
+#pragma unroll
+            for(int i = 0; i < 8; ++i)
+                if(c0 + i < p.chunks)
+                {
+                    p.counts[(size_t)(c0 + i) * p.experts + e] = run; // position inside the expert's run
+                    run += n[i];
+                }
         }
     const bool       live = e < p.experts && !(p.expert_mask && p.expert_mask[e] == 0);
     const int32_t    len  = (run + p.unit - 1) / p.unit * p.unit;
@@ -301,8 +326,8 @@ __global__ __launch_bounds__(64) void moe_sort_scatter_kernel(SortParams p)
     __shared__ float   wts[kSortChunkMulti];
     __shared__ int32_t begin[1024], running[1024];
     const int64_t      n  = (int64_t)sort_rows(p) * p.topk;
-    const int64_t      lo = (int64_t)blockIdx.x * kSortChunkMulti;
-    const int          cnt = (int)((n - lo) < kSortChunkMulti ? (n - lo > 0 ? n - lo : 0) : kSortChunkMulti);
+    const int64_t      lo = (int64_t)blockIdx.x * p.chunk_pairs;
+    const int          cnt = (int)((n - lo) < p.chunk_pairs ? (n - lo > 0 ? n - lo : 0) : p.chunk_pairs);
     for(int i = threadIdx.x; i < cnt; i += blockDim.x)
     {
         const int64_t f = lo + i;
@@ -370,6 +395,11 @@ __device__ __forceinline__ void scatter_run(const SortParams& p, const int32_t* 
 
 __global__ __launch_bounds__(1024) void moe_sort_single_kernel(SortParams p)
 {
+    if(blockIdx.x > 0)
+    {
+        zero_slice(p, 1);
+        return;
+    }
     __shared__ int32_t ids[kSortChunk];
     __shared__ int32_t fill[kSortWaves][1024]; // per run: the expert's count, then its fill level
     __shared__ int32_t count[1024], begin[1024], local[1024];
@@ -442,12 +472,6 @@ __global__ __launch_bounds__(1024) void moe_sort_single_kernel(SortParams p)
         p.sorted_ids[i]     = pad_id;
         p.sorted_weights[i] = 0.f;
     }
-}
-
-__global__ __launch_bounds__(256) void fill_zero_kernel(u32x4* __restrict__ dst, size_t vecs)
-{
-    for(size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < vecs; i += (size_t)gridDim.x * 256)
-        dst[i] = u32x4{0u, 0u, 0u, 0u};
 }
 
 __global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* __restrict__ dst, size_t n, int32_t v)
@@ -1230,7 +1254,10 @@ hipError_t launch_moe_sorting(const MoeSortArgs& a, hipStream_t stream)
     p.id_stride         = a.id_stride;
     p.w_stride          = a.w_stride;
     const int64_t n     = (int64_t)a.M * a.topk;
-    p.chunks            = (int32_t)((n + kSortChunkMulti - 1) / kSortChunkMulti);
+    // a chunk is scattered by one wave, 64 pairs per step: short chunks while the scan (one pass over
+    // the chunks per expert) stays short, long ones for very many pairs
+    p.chunk_pairs       = n <= 65536 ? 256 : kSortChunkMulti;
+    p.chunks            = (int32_t)((n + p.chunk_pairs - 1) / p.chunk_pairs);
     if(p.chunks < 1)
         p.chunks = 1;
     uint8_t*     scratch = nullptr;
@@ -1241,19 +1268,21 @@ hipError_t launch_moe_sorting(const MoeSortArgs& a, hipStream_t stream)
     p.counts       = (int32_t*)scratch;
     p.expert_begin = (int32_t*)(scratch + counts_bytes);
 
+    // workgroups of 1024 threads that clear the output buffer, about 64 KiB each, riding in the first launch
+    unsigned zero_groups = 0;
     if(a.moe_buf && a.moe_buf_bytes)
     {
-        const size_t vecs = a.moe_buf_bytes / 16;
-        unsigned     g    = (unsigned)((vecs + 255) / 256);
-        g                 = g > 4096 ? 4096 : (g < 1 ? 1 : g);
-        hipLaunchKernelGGL(fill_zero_kernel, dim3(g), dim3(256), 0, stream, (u32x4*)a.moe_buf, vecs);
+        p.zero_dst  = (u32x4*)a.moe_buf;
+        p.zero_vecs = a.moe_buf_bytes / 16;
+        const size_t g = (p.zero_vecs + 4095) / 4096;
+        zero_groups    = (unsigned)(g > 1024 ? 1024 : g);
     }
     if(n <= kSortChunk)
     {
-        hipLaunchKernelGGL(moe_sort_single_kernel, dim3(1), dim3(1024), 0, stream, p);
+        hipLaunchKernelGGL(moe_sort_single_kernel, dim3(1 + zero_groups), dim3(1024), 0, stream, p);
         return hipGetLastError();
     }
-    hipLaunchKernelGGL(moe_sort_count_kernel, dim3(p.chunks), dim3(1024), (size_t)a.experts * 4, stream, p);
+    hipLaunchKernelGGL(moe_sort_count_kernel, dim3(p.chunks + zero_groups), dim3(1024), (size_t)a.experts * 4, stream, p);
     hipLaunchKernelGGL(moe_sort_scan_kernel, dim3(1), dim3(1024), 0, stream, p);
     hipLaunchKernelGGL(moe_sort_scatter_kernel, dim3(p.chunks), dim3(64), 0, stream, p);
     return hipGetLastError();
