@@ -474,11 +474,6 @@ __global__ __launch_bounds__(1024) void moe_sort_single_kernel(SortParams p)
     }
 }
 
-__global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* __restrict__ dst, size_t n, int32_t v)
-{
-    for(size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256)
-        dst[i] = v;
-}
 
 // ---------------------------------------------------------------------------------------------
 // The two grouped GEMMs.
@@ -1094,10 +1089,16 @@ __global__ __launch_bounds__(256) void moe_down_cols_kernel(DownColsParams p)
 }
 
 // out[token] += sum over the token's slots, in slot order, of weight * y[sorted position]
+// The position table is never cleared: an entry counts only if the sorted array holds this very
+// (token, slot) pair at that position, which a stale or uninitialised entry cannot fake (a pair
+// occurs once in the sorted array, so an entry that passes is the pair's position).
 template <In16 DT, bool Y32>
 __global__ __launch_bounds__(256) void moe_combine_kernel(const void* __restrict__ y, const float* __restrict__ sorted_weights,
-                                                          const int32_t* __restrict__ where, uint16_t* __restrict__ out,
-                                                          int32_t M, int32_t topk, int32_t dim, int64_t out_stride)
+                                                          const int32_t* __restrict__ where,
+                                                          const int32_t* __restrict__ sorted_ids,
+                                                          const int32_t* __restrict__ num_valid, int32_t max_padded,
+                                                          uint16_t* __restrict__ out, int32_t M, int32_t topk,
+                                                          int32_t dim, int64_t out_stride)
 {
     const int quads = dim / 4;
     const int token = blockIdx.x;
@@ -1107,8 +1108,9 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const void* __restrict
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     for(int k = 0; k < topk; ++k)
     {
-        const int32_t at = where[(size_t)token * topk + k];
-        if(at < 0)
+        const int32_t at    = where[(size_t)token * topk + k];
+        const int32_t valid = num_valid[0] < max_padded ? num_valid[0] : max_padded;
+        if(at < 0 || at >= valid || sorted_ids[at] != ((k << 24) | token))
             continue;
         const float w = sorted_weights[at];
         if constexpr(Y32)
@@ -1324,18 +1326,11 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     const bool y32 = rows_in_f32(a);
     uint16_t*  y   = (uint16_t*)ws;
     ws += align_up(slots * a.dim * (y32 ? 4 : 2));
-    int32_t* where = (int32_t*)ws; // sorted position of each (token, slot) pair, -1 = not routed here
+    int32_t* where = (int32_t*)ws; // sorted position of each (token, slot) pair; stale where the pair is not routed here
     ws += align_up((size_t)a.M * a.topk * 4);
     uint32_t* block_mask = (uint32_t*)ws;
     ws += align_up((size_t)a.max_blocks * 4);
     const bool cols = down_by_columns(a);
-    if(!cols)
-    {
-        const size_t n = (size_t)a.M * a.topk;
-        unsigned     g = (unsigned)((n + 255) / 256);
-        g              = g > 2048 ? 2048 : g;
-        hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, stream, where, n, -1);
-    }
 
     const uint8_t* xq = a.xq;
     const float*   xs = a.xs;
@@ -1481,8 +1476,8 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     auto combine = a.out_dtype == In16::bf16
                        ? (y32 ? moe_combine_kernel<In16::bf16, true> : moe_combine_kernel<In16::bf16, false>)
                        : (y32 ? moe_combine_kernel<In16::fp16, true> : moe_combine_kernel<In16::fp16, false>);
-    hipLaunchKernelGGL(combine, cgrid, dim3(256), 0, stream, (const void*)y, a.sorted_weights, where,
-                       (uint16_t*)a.out, a.M, a.topk, a.dim, a.out_stride);
+    hipLaunchKernelGGL(combine, cgrid, dim3(256), 0, stream, (const void*)y, a.sorted_weights, where, a.sorted_ids,
+                       a.num_valid, a.max_padded, (uint16_t*)a.out, a.M, a.topk, a.dim, a.out_stride);
     return hipGetLastError();
 }
 
