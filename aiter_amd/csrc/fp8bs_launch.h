@@ -25,6 +25,7 @@ struct QuantArgs
     const int32_t* num_rows;     // optional device scalar limiting the rows processed
     int32_t     num_rows_factor;
     In16        dtype;
+    int32_t     scale_row_stride = 0; // row-major scales with this many floats between rows (0: groups_per_row)
 };
 hipError_t launch_group_quant(const QuantArgs& a, hipStream_t stream);
 

@@ -477,10 +477,17 @@ __global__ __launch_bounds__(1024) void moe_sort_single_kernel(SortParams p)
 
 // ---------------------------------------------------------------------------------------------
 // The two grouped GEMMs.
+
+// What the second GEMM needs to know about a sorted row besides its activations, in one 32-byte
+// record (one cache line touched instead of three): floats 0..3 the row's 1x128 scales (written by
+// the quantiser), float 4 its routing weight, float 5 its token id as bits (written by the first
+// GEMM).  Used while inter_dim / 128 <= 4.
+constexpr int kRowInfo = 8;
+
 struct MoeGemmParams
 {
     const uint8_t* xq;   // first GEMM: [M][K] fp8 tokens (row stride lda); second: [slots][K] by sorted slot
-    const float*   xs;   // first: [K/128][M]; second: [slots][K/128]
+    const float*   xs;   // first: [K/128][M]; second: [slots][xs_stride], a slot's K/128 scales first
     const uint8_t* w;    // [experts][N][K] fp8, pre-shuffled (16,16) per expert
     const float*   wsc;  // [experts][N/128][K/128]
     const int32_t* sorted_ids;
@@ -494,6 +501,9 @@ struct MoeGemmParams
     int32_t        wave_cols; // second GEMM only: columns per wave (64 or 128)
     int32_t*       where;   // first GEMM only: [M][topk] sorted position of each (token, slot) pair
     uint32_t*      block_mask; // first GEMM only: [blocks] bit r set = row r of the block is a real pair
+    float*         row_info;   // first GEMM only: [slots][kRowInfo] records, see below (null: not wanted)
+    const float*   sorted_weights; // first GEMM only, for row_info
+    int32_t        xs_stride;  // second GEMM only: floats between the scale rows of two slots
     int64_t        lda;
 };
 
@@ -644,6 +654,11 @@ __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmP
             real         = token < p.M && slot < p.topk;
             if(real && p.where)
                 p.where[(size_t)token * p.topk + slot] = at;
+            if(p.row_info)
+            {
+                p.row_info[(size_t)at * kRowInfo + 4] = p.sorted_weights[at];
+                p.row_info[(size_t)at * kRowInfo + 5] = __int_as_float(real ? token : p.M);
+            }
         }
         const uint64_t rows = __ballot(real);
         if(threadIdx.x == 0 && p.block_mask)
@@ -679,7 +694,7 @@ __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int g
         for(int kb = 0; kb < KB; ++kb)
         {
             x[j][kb]  = load_x_fragment(p.xq + slot * p.lda + (size_t)kb * 128, kg);
-            xs[j][kb] = p.xs[slot * KB + kb];
+            xs[j][kb] = p.xs[slot * p.xs_stride + kb];
         }
     }
     const size_t   tile_stride = (size_t)16 * (size_t)p.K;
@@ -778,7 +793,7 @@ __global__ __launch_bounds__(256) void moe_down_long_k_kernel(MoeGemmParams p)
     {
         const size_t slot = (size_t)blk * 32 + j * 16 + l16;
         xrow[j]           = p.xq + slot * p.lda;
-        xsr[j]            = p.xs + slot * p.kblocks;
+        xsr[j]            = p.xs + slot * p.xs_stride;
         real[j]           = (p.sorted_ids[slot] & 0xffffff) < p.M;
     }
     const uint8_t* wt  = p.w + (size_t)expert * (size_t)p.N * (size_t)p.K + (size_t)(n0 >> 4) * 16 * (size_t)p.K;
@@ -843,11 +858,9 @@ __global__ __launch_bounds__(256) void moe_down_long_k_kernel(MoeGemmParams p)
 struct DownColsParams
 {
     const uint8_t*  xq;  // [slots][K] fp8 by sorted slot
-    const float*    xs;  // [slots][K/128]
+    const float*    row_info; // [slots][kRowInfo]: scales, routing weight, token id of each sorted row
     const uint8_t*  w;   // [experts][N][K] fp8, pre-shuffled (16,16) per expert
     const float*    wsc; // [experts][N/128][K/128]
-    const int32_t*  sorted_ids;
-    const float*    sorted_weights;
     const int32_t*  sorted_expert_ids;
     const int32_t*  num_valid;
     const uint32_t* block_mask; // [blocks], written by the first GEMM
@@ -862,8 +875,8 @@ constexpr int kColsMaxBlocks = 1024; // blocks the unit scan takes (16 per lane)
 struct ColsStage
 {
     i32x4    wlo, whi, xlo, xhi;
-    float    xs, sw, ws;
-    int32_t  tok;
+    float    xs, ws;
+    u32x2    sw_tok; // routing weight (as bits) and token id
     uint32_t mask;
 };
 
@@ -887,18 +900,18 @@ __device__ __forceinline__ void cols_load4(float& d, const void* p)
 {
     asm volatile("global_load_dword %0, %1, off" : "=v"(d) : "v"(p) : "memory");
 }
-__device__ __forceinline__ void cols_load4(int32_t& d, const void* p)
+__device__ __forceinline__ void cols_load8_at16(u32x2& d, const void* p)
 {
-    asm volatile("global_load_dword %0, %1, off" : "=v"(d) : "v"(p) : "memory");
+    asm volatile("global_load_dwordx2 %0, %1, off offset:16" : "=v"(d) : "v"(p) : "memory");
 }
-constexpr int kColsLoadsPerStage = 8; // loads the walk requests per unit, counted by cols_wait_oldest
+constexpr int kColsLoadsPerStage = 7; // loads the walk requests per unit, counted by cols_wait_oldest
 // the stage requested kColsDepth - 1 stages ago has arrived once at most (kColsDepth - 1) *
-// kColsLoadsPerStage = 56 younger loads are outstanding (loads return in order); the stage's
+// kColsLoadsPerStage = 49 younger loads are outstanding (loads return in order); the stage's
 // registers are operands so that nothing that reads them is moved above the wait
 __device__ __forceinline__ void cols_wait_oldest(ColsStage& s)
 {
-    asm volatile("s_waitcnt vmcnt(56)"
-                 : "+v"(s.wlo), "+v"(s.whi), "+v"(s.xlo), "+v"(s.xhi), "+v"(s.xs), "+v"(s.sw), "+v"(s.ws), "+v"(s.tok)
+    asm volatile("s_waitcnt vmcnt(49)"
+                 : "+v"(s.wlo), "+v"(s.whi), "+v"(s.xlo), "+v"(s.xhi), "+v"(s.xs), "+v"(s.ws), "+v"(s.sw_tok)
                  :
                  : "memory");
 }
@@ -907,11 +920,11 @@ __device__ __forceinline__ void cols_wait_oldest(ColsStage& s)
 __device__ __forceinline__ void cols_drain(ColsStage& s)
 {
     asm volatile("s_waitcnt vmcnt(0)"
-                 : "+v"(s.wlo), "+v"(s.whi), "+v"(s.xlo), "+v"(s.xhi), "+v"(s.xs), "+v"(s.sw), "+v"(s.ws), "+v"(s.tok)
+                 : "+v"(s.wlo), "+v"(s.whi), "+v"(s.xlo), "+v"(s.xhi), "+v"(s.xs), "+v"(s.ws), "+v"(s.sw_tok)
                  :
                  : "memory");
 }
-static_assert((kColsDepth - 1) * kColsLoadsPerStage == 56, "cols_wait_oldest counts 56 younger loads");
+static_assert((kColsDepth - 1) * kColsLoadsPerStage == 49, "cols_wait_oldest counts 49 younger loads");
 
 template <In16 DT>
 __global__ __launch_bounds__(256) void moe_down_cols_kernel(DownColsParams p)
@@ -993,9 +1006,9 @@ __global__ __launch_bounds__(256) void moe_down_cols_kernel(DownColsParams p)
         const uint8_t* xp = p.xq + slot * (size_t)p.K + (size_t)kb * 128 + kg * 32;
         cols_load16(s.xlo, xp);
         cols_load16_at16(s.xhi, xp);
-        cols_load4(s.xs, p.xs + slot * p.kblocks + kb);
-        cols_load4(s.sw, p.sorted_weights + slot);
-        cols_load4(s.tok, p.sorted_ids + slot);
+        const float* info = p.row_info + slot * kRowInfo;
+        cols_load4(s.xs, info + kb);
+        cols_load8_at16(s.sw_tok, info);
     };
     auto consume = [&](ColsStage& s, bool live) {
         cols_wait_oldest(s);
@@ -1007,7 +1020,7 @@ __global__ __launch_bounds__(256) void moe_down_cols_kernel(DownColsParams p)
         // 16 different tokens.  A routing that names an expert twice for a token puts the two pairs
         // next to each other in the sorted order; such a unit is added one row at a time.
         const bool  real = live && ((s.mask >> l16) & 1u);
-        const int   key  = real ? (s.tok & 0xffffff) : -1 - l16;
+        const int   key  = real ? (int)s.sw_tok[1] : -1 - l16;
         const int   prev = __builtin_amdgcn_update_dpp(-100, key, 0x111 /* row_shr:1 */, 0xf, 0xf, false);
         const int   row  = real ? key : p.M + l16;
         const float sc   = s.xs * s.ws;
@@ -1015,7 +1028,7 @@ __global__ __launch_bounds__(256) void moe_down_cols_kernel(DownColsParams p)
         f32x4       add;
 #pragma unroll
         for(int c = 0; c < 4; ++c)
-            add[c] = prod[c] * sc * s.sw;
+            add[c] = prod[c] * sc * __uint_as_float(s.sw_tok[0]);
         if(__builtin_expect(__ballot(real && prev == key) == 0, 1))
         {
             f32x4 cur = *(f32x4*)dst;
@@ -1290,13 +1303,17 @@ hipError_t launch_moe_sorting(const MoeSortArgs& a, hipStream_t stream)
     return hipGetLastError();
 }
 
+// floats per sorted row in the buffer the quantiser writes its scales to: a row record while the
+// second GEMM's K has at most four scale blocks, the bare scales beyond
+size_t scale_floats_per_slot(const MoeArgs& a) { return a.inter / 128 <= 4 ? (size_t)kRowInfo : (size_t)(a.inter / 128); }
+
 size_t moe_workspace_bytes(const MoeArgs& a)
 {
     const size_t slots = (size_t)a.max_padded;
     size_t       b     = 0;
     b += align_up(slots * a.inter * 2);          // activation product, bf16
     b += align_up(slots * a.inter);              // the same as fp8
-    b += align_up(slots * (a.inter / 128) * 4);  // its scales
+    b += align_up(slots * scale_floats_per_slot(a) * 4); // its scales, or the row records that hold them
     b += align_up(slots * a.dim * (rows_in_f32(a) ? 4 : 2)); // second GEMM's rows
     b += align_up((size_t)a.M * a.topk * 4);     // sorted position of each (token, slot)
     b += align_up((size_t)a.max_blocks * 4);     // real rows of each block
@@ -1322,7 +1339,7 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     uint8_t* hq = ws;
     ws += align_up(slots * a.inter);
     float* hs = (float*)ws;
-    ws += align_up(slots * (a.inter / 128) * 4);
+    ws += align_up(slots * scale_floats_per_slot(a) * 4);
     const bool y32 = rows_in_f32(a);
     uint16_t*  y   = (uint16_t*)ws;
     ws += align_up(slots * a.dim * (y32 ? 4 : 2));
@@ -1375,6 +1392,8 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     p.topk              = a.topk;
     p.where             = cols ? nullptr : where;
     p.block_mask        = block_mask;
+    p.row_info          = a.inter / 128 <= 4 ? hs : nullptr;
+    p.sorted_weights    = a.sorted_weights;
     p.max_blocks        = a.max_blocks;
     p.experts           = a.experts;
     p.activation        = a.activation;
@@ -1405,6 +1424,7 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     qa.group           = 128;
     qa.transpose_scale = false;
     qa.num_rows        = a.num_valid; // only the rows that exist
+    qa.scale_row_stride = a.inter / 128 <= 4 ? kRowInfo : 0;
     qa.num_rows_factor = 1;
     qa.dtype           = In16::bf16;
     e                  = launch_group_quant(qa, stream);
@@ -1415,11 +1435,9 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     {
         DownColsParams c{};
         c.xq                = hq;
-        c.xs                = hs;
+        c.row_info          = hs;
         c.w                 = a.w2;
         c.wsc               = a.w2_scale;
-        c.sorted_ids        = a.sorted_ids;
-        c.sorted_weights    = a.sorted_weights;
         c.sorted_expert_ids = a.sorted_expert_ids;
         c.num_valid         = a.num_valid;
         c.block_mask        = block_mask;
@@ -1450,6 +1468,7 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
     d.N             = a.dim;
     d.kblocks       = a.inter / 128;
     d.lda           = a.inter;
+    d.xs_stride     = (int32_t)scale_floats_per_slot(a);
     d.out_f32       = y32 ? 1 : 0;
     if(d.kblocks <= 4)
     {

@@ -249,6 +249,7 @@ struct QuantKernelParams
     const int32_t* num_rows;
     int32_t        num_rows_factor;
     int32_t        transpose_scale;
+    uint32_t       scale_row_stride; // 0: scales are contiguous
 };
 
 constexpr int kQuantBlock = 256;
@@ -304,6 +305,12 @@ __global__ __launch_bounds__(kQuantBlock) void group_quant_kernel(QuantKernelPar
                     uint32_t col = g - row * p.groups_per_row;
                     idx          = (size_t)col * rows + row;
                 }
+                else if(p.scale_row_stride)
+                {
+                    uint32_t row = g / p.groups_per_row;
+                    uint32_t col = g - row * p.groups_per_row;
+                    idx          = (size_t)row * p.scale_row_stride + col;
+                }
                 p.scale[idx] = s;
             }
         }
@@ -325,6 +332,7 @@ static hipError_t launch_group_quant_t(const QuantArgs& a, hipStream_t stream)
     p.num_rows        = a.num_rows;
     p.num_rows_factor = a.num_rows_factor;
     p.transpose_scale = a.transpose_scale ? 1 : 0;
+    p.scale_row_stride = (uint32_t)a.scale_row_stride;
     const uint64_t n_groups = (uint64_t)a.rows * (uint64_t)a.groups_per_row;
     if(n_groups == 0)
         return hipSuccess;
