@@ -19,6 +19,7 @@ from .gemm_op_a8w8 import (
     gemm_a8w8_blockscale_ck,
     gemm_a8w8_blockscale_cktile,
     gemm_kernel_names,
+    get_CKGEMM_config,
 )
 from .shuffle import shuffle_weight
 from .fused_moe import (
@@ -65,6 +66,7 @@ __all__ = [
     "gemm_a8w8_blockscale_cktile",
     "gemm_a8w8_blockscale_bpreshuffle_cktile",
     "gemm_kernel_names",
+    "get_CKGEMM_config",
     "rmsnorm",
     "rmsnorm_quant",
     "rms_norm",

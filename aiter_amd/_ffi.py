@@ -50,6 +50,7 @@ EXPORTED_SYMBOLS = sorted(
         "aiter_get_last_error",
         "aiter_clear_last_error",
         "aiter_fp8bs_gemm_kernel_names",
+        "aiter_fp8bs_gemm_choice",
     ]
 )
 
@@ -74,6 +75,9 @@ def load_library():
         lib.aiter_get_last_error.restype = ctypes.c_char_p
         lib.aiter_clear_last_error.restype = None
         lib.aiter_fp8bs_gemm_kernel_names.restype = ctypes.c_char_p
+        lib.aiter_fp8bs_gemm_choice.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
+                                                ctypes.c_char_p, ctypes.c_int64]
+        lib.aiter_fp8bs_gemm_choice.restype = ctypes.c_int
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(lib, name)
             fn.argtypes = argtypes + [ctypes.c_void_p]
@@ -126,3 +130,12 @@ def call(name: str, *args):
 
 def gemm_kernel_names():
     return load_library().aiter_fp8bs_gemm_kernel_names().decode().split(",")
+
+
+def gemm_choice(m: int, n: int, k: int, preshuffled: bool = False) -> str:
+    lib = load_library()
+    buf = ctypes.create_string_buffer(64)
+    if lib.aiter_fp8bs_gemm_choice(int(m), int(n), int(k), 1 if preshuffled else 0, buf, 64) != 0:
+        raw = lib.aiter_get_last_error()
+        raise RuntimeError(f"aiter_fp8bs_gemm_choice failed: {raw.decode(errors='replace') if raw else '?'}")
+    return buf.value.decode()

@@ -433,6 +433,19 @@ void aiter_clear_last_error(void) { g_last_error.clear(); }
 
 const char* aiter_fp8bs_gemm_kernel_names(void) { return fp8bs::gemm_kernel_names(); }
 
+int aiter_fp8bs_gemm_choice(int64_t M, int64_t N, int64_t K, int preshuffled, char* out, int64_t out_len)
+{
+    return guarded([&] {
+        const char* fn = "aiter_fp8bs_gemm_choice";
+        if(out == nullptr || out_len < 32)
+            fail(fn, "out must hold at least 32 characters");
+        if(M < 1 || N < 1 || K < 128 || K % 128 != 0 || M > 0x7fffffffLL / 2 || N > 0x7fffffffLL / 2 ||
+           K > 0x7fffffffLL / 2)
+            fail(fn, "M and N must be positive and K a positive multiple of 128, got ", M, " x ", N, " x ", K);
+        fp8bs::gemm_describe_choice(M, N, K, preshuffled != 0, out, (size_t)out_len);
+    });
+}
+
 int dynamic_per_token_scaled_quant(aiter_tensor_t* out, aiter_tensor_t* input,
                                    aiter_tensor_t* scales, aiter_tensor_t* scale_ub,
                                    int shuffle_scale, aiter_tensor_t* num_rows,

@@ -165,34 +165,34 @@ static const char* const kKernelNames =
 
 const char* gemm_kernel_names() { return kKernelNames; }
 
+// The kernel family taken when the caller names none.
+// Up to 64 activation rows the weight-streaming kernel wins everywhere.  Above that, the 256x256
+// tiling or the mid_* tilings, whichever is modelled faster.  Measured on the DeepSeek shapes, a
+// 256x256 iteration over one K block takes 1.7 us while the tiles of a round cover up to 56 % of
+// the compute units and up to 2.1 us when they cover all of them, against 0.8 us for a quarter of
+// the area: it wins once its tiles cover about half of the chip.  Near a tie it is preferred: it
+// gains more when the weights are still in the last-level cache.
+static const char* automatic_choice(const GemmKernelParams& p)
+{
+    const int64_t prefill_tiles  = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
+    const int64_t prefill_rounds = (prefill_tiles + 255) / 256;
+    const float   prefill_share  = (float)prefill_tiles / (float)(prefill_rounds * 256);
+    const float   prefill_iter   = 1.7f + (prefill_share > 0.56f ? (prefill_share - 0.56f) * 0.9f : 0.f);
+    const float   prefill_us     = 13.5f + (float)prefill_rounds * (float)p.kblocks * prefill_iter;
+    if(p.M <= 64 && gemm_decode_supports(p))
+        return "decode_stream";
+    if(gemm_mid_supports(p) && (!gemm_prefill_supports(p) || gemm_mid_estimate_us(p) * 1.03f < prefill_us))
+        return "mid_auto";
+    if(gemm_prefill_supports(p))
+        return "prefill_256x256";
+    return "tile_128x128";
+}
+
 template <In16 DT>
 static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStream_t stream,
                            const char** why)
 {
-    const char* name = (a.kernel_name && a.kernel_name[0]) ? a.kernel_name : nullptr;
-    if(name == nullptr)
-    {
-        // Up to 64 activation rows the weight-streaming kernel wins everywhere.  Above that,
-        // the 256x256 tiling or the mid_* tilings, whichever is modelled faster.  Measured on the
-        // DeepSeek shapes, a 256x256 iteration over one K block takes 1.7 us while the tiles of a
-        // round cover up to 56 % of the compute units and up to 2.1 us when they cover all of them,
-        // against 0.8 us for a quarter of the area: it wins once its tiles cover about half of the
-        // chip.  Near a tie it is preferred: it gains more when the weights are still in the
-        // last-level cache.
-        const int64_t prefill_tiles  = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
-        const int64_t prefill_rounds = (prefill_tiles + 255) / 256;
-        const float   prefill_share  = (float)prefill_tiles / (float)(prefill_rounds * 256);
-        const float   prefill_iter   = 1.7f + (prefill_share > 0.56f ? (prefill_share - 0.56f) * 0.9f : 0.f);
-        const float   prefill_us     = 13.5f + (float)prefill_rounds * (float)p.kblocks * prefill_iter;
-        if(p.M <= 64 && gemm_decode_supports(p))
-            name = "decode_stream";
-        else if(gemm_mid_supports(p) && (!gemm_prefill_supports(p) || gemm_mid_estimate_us(p) * 1.03f < prefill_us))
-            name = "mid_auto";
-        else if(gemm_prefill_supports(p))
-            name = "prefill_256x256";
-        else
-            name = "tile_128x128";
-    }
+    const char* name = (a.kernel_name && a.kernel_name[0]) ? a.kernel_name : automatic_choice(p);
     if(strcmp(name, "tile_16x256") == 0)
         return launch_tile<DT, 16, 256, 1, 4>(p, stream);
     if(strcmp(name, "tile_64x128") == 0)
@@ -276,6 +276,23 @@ hipError_t launch_gemm_blockscale(const GemmArgs& a, hipStream_t stream, const c
     p.w_shuffled = a.w_shuffled ? 1 : 0;
     return a.out_dtype == In16::bf16 ? dispatch<In16::bf16>(a, p, stream, why)
                                      : dispatch<In16::fp16>(a, p, stream, why);
+}
+
+void gemm_describe_choice(int64_t M, int64_t N, int64_t K, bool shuffled, char* buf, size_t n)
+{
+    GemmKernelParams p{};
+    p.M          = (int32_t)M;
+    p.N          = (int32_t)N;
+    p.K          = (int32_t)K;
+    p.lda        = K;
+    p.ldb        = K;
+    p.kblocks    = (int32_t)(K / 128);
+    p.w_shuffled = shuffled ? 1 : 0;
+    const char* name = automatic_choice(p);
+    if(strcmp(name, "mid_auto") == 0)
+        gemm_mid_describe(p, buf, n);
+    else
+        snprintf(buf, n, "%s", name);
 }
 
 } // namespace fp8bs

@@ -80,6 +80,7 @@ hipError_t launch_gemm_mid(const GemmKernelParams& p, In16 out_dtype, int split_
                            hipStream_t stream, int tile = 0, int splits = 0);
 bool       gemm_mid_supports(const GemmKernelParams& p);
 // modelled duration (us) of the best mid_* tiling, for the choice between kernel families
+void       gemm_mid_describe(const GemmKernelParams& g, char* buf, size_t n);
 float      gemm_mid_estimate_us(const GemmKernelParams& p);
 // Per-device workspace for K split across workgroups (fp32 partial tiles + tickets that are zero
 // between launches), shared by the kernels that split K; grown on demand, kept for the life of

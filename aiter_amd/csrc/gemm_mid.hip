@@ -18,6 +18,8 @@
 // 1 us per K block.
 #include "gemm_common.h"
 
+#include <cstdio>
+
 namespace fp8bs {
 
 namespace {
@@ -538,6 +540,14 @@ hipError_t launch_gemm_mid(const GemmKernelParams& g, In16 out_dtype, int split_
     case 64128: return launch_shape<64, 128>(p, -1, splits, device_id, stream);
     default: return launch_shape<64, 64>(p, -1, splits, device_id, stream);
     }
+}
+
+// "mid_128x128:s=2": the tiling and K range count the automatic choice takes for this problem
+void gemm_mid_describe(const GemmKernelParams& g, char* buf, size_t n)
+{
+    const MidPlan pl = best_plan(g, 0);
+    snprintf(buf, n, "%s:s=%d", pl.tile == 128 ? "mid_128x128" : pl.tile == 64128 ? "mid_64x128" : "mid_64x64",
+             pl.splits);
 }
 
 } // namespace fp8bs

@@ -221,6 +221,17 @@ def gemm_a8w8_blockscale_bpreshuffle(
     return _bpreshuffle_op(XQ, WQ, x_scale, w_scale, dtype, out)
 
 
+def get_CKGEMM_config(M: int, N: int, K: int, tuned_file: Optional[str] = None, isBpreshuffled: bool = False):
+    """aiter/ops/gemm_op_a8w8.py:448-490 looks (M, N, K) up in tuned CSV tables and returns the row as a
+    dict (``kernelName``, ``splitK``, ``libtype`` ...) or None.  Here the choice is a shape rule inside the
+    library and every shape has one; it is returned in the same form, with a ``kernelName`` that the
+    low-level entry points accept.  ``tuned_file`` is accepted and not read."""
+    name = _ffi.gemm_choice(M, N, K, isBpreshuffled)
+    splits = int(name.split(":s=")[1]) if ":s=" in name else 1
+    return {"M": M, "N": N, "K": K, "libtype": "hip", "kernelName": name, "splitK": max(splits - 1, 0).bit_length(),
+            "kRanges": splits}
+
+
 def gemm_kernel_names():
     """Names accepted as ``kernelName`` (the counterpart of the reference's kernel zoo,
     csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale_instance.py:73-117)."""

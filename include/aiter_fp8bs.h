@@ -179,6 +179,13 @@ int gemm_a8w8_blockscale_bpreshuffle(aiter_tensor_t* XQ, aiter_tensor_t* WQ, ait
  * csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale_instance.py:73-117). */
 const char* aiter_fp8bs_gemm_kernel_names(void);
 
+/* The kernel the library takes for contiguous operands of shape M x N x K when kernelName is empty,
+ * written to `out` (at least 32 characters) in the form kernelName accepts, e.g. "decode_stream",
+ * "prefill_256x256", "mid_128x128:s=2".  Host-only: no device is touched.  The counterpart of the
+ * reference's lookup in its tuned tables, get_CKGEMM_config (aiter/ops/gemm_op_a8w8.py:448-490):
+ * here the choice is a shape rule inside the library. */
+int aiter_fp8bs_gemm_choice(int64_t M, int64_t N, int64_t K, int preshuffled, char* out, int64_t out_len);
+
 /*
  * ---- block-scale mixture of experts (gated experts, fp8 e4m3fn, 1x128 / 128x128 scales) ----
  *

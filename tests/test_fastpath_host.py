@@ -26,3 +26,25 @@ def test_fast_division_is_ieee_exact(checker, mode):
     out = subprocess.run([checker, mode], capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stdout + out.stderr
     assert out.stdout.startswith("OK")
+
+
+def test_kernel_choice_query_on_the_headline_shapes():
+    """The shape rule that stands in for the reference's tuned-table lookup (get_CKGEMM_config,
+    aiter/ops/gemm_op_a8w8.py:448-490) can be asked without a GPU."""
+    import aiter_amd
+
+    names = set(aiter_amd.gemm_kernel_names())
+    for m in (1, 16, 64):
+        for n, k in ((7168, 2048), (24576, 1536), (2112, 7168)):
+            assert aiter_amd.get_CKGEMM_config(m, n, k)["kernelName"] == "decode_stream"
+    assert aiter_amd.get_CKGEMM_config(8192, 36864, 7168)["kernelName"] == "prefill_256x256"
+    assert aiter_amd.get_CKGEMM_config(2048, 4096, 7168)["kernelName"] == "prefill_256x256"
+    cfg = aiter_amd.get_CKGEMM_config(128, 4096, 7168)  # few tiles, long K: K is split
+    assert cfg["kernelName"].startswith("mid_") and cfg["kRanges"] > 1 and cfg["libtype"] == "hip"
+    for m, n, k in ((65, 512, 128), (300, 1000, 384), (4096, 2112, 7168), (100000, 128, 128)):
+        cfg = aiter_amd.get_CKGEMM_config(m, n, k, isBpreshuffled=(n % 16 == 0))
+        assert cfg["kernelName"].split(":")[0] in names
+    import pytest
+
+    with pytest.raises(RuntimeError, match="multiple of 128"):
+        aiter_amd.get_CKGEMM_config(4, 512, 100)

@@ -306,3 +306,14 @@ def test_fused_config_shape_sampled_rows():
     rows = torch.randperm(m, generator=torch.Generator().manual_seed(2))[:64]
     ref = tr.gemm_a8w8_blockscale_ref(xq[rows], wq, xs[rows], ws)
     assert tr.check_allclose_ratio(out.cpu()[rows], ref, RTOL, ATOL) == 0.0
+
+
+@pytest.mark.parametrize("m,n,k", [(8, 2112, 1024), (130, 4096, 7168), (1000, 2112, 2048), (2048, 4096, 1024)])
+def test_kernel_choice_query_names_what_runs(m, n, k):
+    # naming the kernel the query reports gives the bits the automatic choice gives
+    xq, wq, xs, ws = (t.to(DEV) for t in make_problem(m, n, k, seed=17))
+    cfg = aiter_amd.get_CKGEMM_config(m, n, k)
+    auto = aiter_amd.gemm_a8w8_blockscale(xq, wq, xs, ws)
+    named = torch.empty_like(auto)
+    aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, xs, ws, named, splitK=-1, kernelName=cfg["kernelName"])
+    assert torch.equal(auto, named), cfg
