@@ -479,8 +479,8 @@ static MidPlan plan_cost(const GemmKernelParams& g, int tile, int splits)
                  (float)(rounds - 1) * (fixed - 2.4f);
     if(splits > 1)
     {
-        const float reduce = 1.7f + (float)splits * (float)g.M * (float)g.N * 4.f / 6.0e6f;
-        cost += 1.5f + (reduce < 4.8f ? 4.8f : reduce);
+        // partial tiles written and read back at about 6 TB/s, plus the second launch
+        cost += 3.2f + (float)splits * (float)g.M * (float)g.N * 4.f / 6.0e6f;
     }
     return MidPlan{tile, splits, cost};
 }
