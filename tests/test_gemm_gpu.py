@@ -234,6 +234,21 @@ def test_mid_kernel(kernel, m, n, k, splitk):
         assert (out.view(torch.int16) != tile.view(torch.int16)).float().mean().item() < 0.02
 
 
+@pytest.mark.parametrize("kblocks", [1, 2, 3, 4, 5, 6, 7, 8, 9, 11, 12, 13, 18])
+def test_mid_64x64_lone_workgroups_every_k_length(kblocks):
+    # no more workgroups than compute units: the 64x64 tile runs its six-stage ring, filled two K
+    # blocks at a time; every K length up to and past two trips round the ring, odd and even
+    m, n, k = 100, 200, 128 * kblocks
+    xq, wq, xs, ws = make_problem(m, n, k, seed=900 + kblocks, outliers=0.01)
+    out = run_gpu(xq, wq, xs, ws, kernel="mid_64x64", splitK=0)
+    assert_close_to_f64(out, xq, wq, xs, ws, f"mid_64x64 {m}x{n}x{k}")
+    tile = run_gpu(xq, wq, xs, ws, kernel="tile_128x128")
+    assert torch.equal(out.view(torch.int16), tile.view(torch.int16))
+    if kblocks >= 8:
+        halves = run_gpu(xq, wq, xs, ws, kernel="mid_64x64:s=2", splitK=-1)
+        assert_close_to_f64(halves, xq, wq, xs, ws, f"mid_64x64:s=2 {m}x{n}x{k}")
+
+
 @pytest.mark.parametrize("name", ["mid_128x128:s=3", "mid_64x64:s=5", "mid_64x128:s=7", "mid_auto:s=2"])
 @pytest.mark.parametrize("m,n,k,dtype", [(200, 520, 2304, torch.bfloat16), (128, 2112, 7168, torch.float16)])
 def test_mid_kernel_pinned_k_ranges(name, m, n, k, dtype):
