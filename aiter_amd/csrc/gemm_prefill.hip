@@ -11,6 +11,7 @@
 // Workgroups are renumbered so that the 32 tiles resident on one XCD at a time form a compact
 // 8 (m) x 4 (n) patch: each XCD's L2 then serves every operand slab to several CUs.
 #include "gemm_common.h"
+#include <algorithm>
 
 namespace fp8bs {
 
@@ -20,6 +21,7 @@ constexpr int kBM = 256, kBN = 256, kThreads = 512;
 constexpr int kSlabBytes  = (kBM + kBN) * 128; // 64 KiB: 256 weight rows then 256 activation rows
 constexpr int kStageBytes = kSlabBytes + kBM * 4; // + this K block's x_scale for the 256 rows
 constexpr int kStages = 2;
+constexpr uint32_t kEpiPitch = 272; // bytes per row of a wave's 64 x 128 16-bit output block in LDS
 constexpr int kGroupN = 4; // n tiles swept together by consecutive workgroups
 
 // 16-byte chunk c of stage row r is stored at chunk c ^ ((r >> 1) & 7): the 16 rows one
@@ -45,13 +47,26 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    typedef const volatile i32x4 __attribute__((address_space(3)))* lds_vec_ptr;
+    typedef uint8_t __attribute__((address_space(3)))*              lds_byte_ptr;
+    const lds_byte_ptr smem3 = (lds_byte_ptr)smem;
+
+    // The workgroup walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... (one workgroup per compute
+    // unit when there are more tiles than compute units): a tile's output stores drain, and the
+    // next tile's first slabs arrive, behind one wait instead of a workgroup's end and start.
+    const int total = tiles_m * tiles_n;
+    for(int tile = blockIdx.x; tile < total; tile += gridDim.x)
+    {
+    // Everything derived from the lane index is derived again for every tile (the empty asm
+    // hides that it is the same value): kept live across the K loop it would not fit the registers.
+    int t = threadIdx.x;
+    asm volatile("" : "+v"(t));
+    const int lane = t & 63, wave = t >> 6;
     const int l16 = lane & 15, kg = lane >> 4;
     const int wn = wave & 1, wm = wave >> 1; // n half (128 rows), m quarter (64 rows)
 
     // ---- tile choice: XCD-aware renumbering, then n-groups swept m-fastest
-    const int total = tiles_m * tiles_n;
-    int       v     = blockIdx.x;
+    int       v     = tile;
     if((total & 7) == 0)
         v = (v & 7) * (total >> 3) + (v >> 3); // workgroups go round-robin over the 8 XCDs
     const int group  = v / (kGroupN * tiles_m);
@@ -60,10 +75,6 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     const int tm     = within / gn;
     const int tn     = group * kGroupN + (within - tm * gn);
     const int m0 = tm * kBM, n0 = tn * kBN;
-
-    typedef const volatile i32x4 __attribute__((address_space(3)))* lds_vec_ptr;
-    typedef uint8_t __attribute__((address_space(3)))*              lds_byte_ptr;
-    const lds_byte_ptr smem3 = (lds_byte_ptr)smem;
 
     // ---- global -> LDS plan: per stage 64 units of 8 rows (1 KiB); wave w moves units i*8+w.
     // Lane p of a unit fills LDS chunk p, i.e. stage row 8u + p/8, stored chunk p%8, which must
@@ -326,32 +337,52 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
 #undef FP8BS_MFMA
 #undef FP8BS_FMA4
 
-    // ---- epilogue: lane owns out[m][n .. n+3] for each of its 8 x 4 tiles
-#pragma unroll
-    for(int j = 0; j < 4; ++j)
+    // ---- epilogue.  A lane owns out[m][n .. n+3] for each of its 8 x 4 tiles: stored from there,
+    // one instruction would touch 16 rows with 32 bytes each.  The wave's 64 x 128 block goes
+    // through its own LDS region instead (the stage buffers are free after the loop's last
+    // barrier; rows padded to 272 bytes so the 16 rows of one write fall on different banks) and
+    // leaves as 16-byte stores, 16 lanes per 256-byte row piece, 4 rows per instruction.  LDS
+    // operations of one wave complete in order, so no barrier stands between write and read.
     {
-        const int m = m0 + wm * 64 + j * 16 + l16;
-        if(m >= p.M)
-            continue;
+        const uint32_t ebase = (uint32_t)wave * (64u * kEpiPitch);
+        typedef u32x2 __attribute__((address_space(3)))*       lds_u2_ptr;
+        typedef const u32x4 __attribute__((address_space(3)))* lds_u4_ptr;
 #pragma unroll
-        for(int i = 0; i < 8; ++i)
+        for(int j = 0; j < 4; ++j)
+#pragma unroll
+            for(int i = 0; i < 8; ++i)
+                *(lds_u2_ptr)(smem3 + ebase + (uint32_t)(j * 16 + l16) * kEpiPitch +
+                              (uint32_t)(i * 16 + kg * 4) * 2u) =
+                    u32x2{pack2<DT>(acc[i][j][0], acc[i][j][1]), pack2<DT>(acc[i][j][2], acc[i][j][3])};
+
+        const int  col    = (lane & 15) * 8;
+        const int  n      = n0 + wn * 128 + col;
+        const bool vec_ok = (p.N & 7) == 0 && ((uintptr_t)p.out & 15) == 0 && n + 8 <= p.N;
+#pragma unroll
+        for(int c = 0; c < 16; ++c)
         {
-            const int n   = n0 + wn * 128 + i * 16 + kg * 4;
+            const int   row = c * 4 + (lane >> 4);
+            const int   m   = m0 + wm * 64 + row;
+            const u32x4 vv  = *(lds_u4_ptr)(smem3 + ebase + (uint32_t)row * kEpiPitch + (uint32_t)col * 2u);
+            if(m >= p.M)
+                continue;
             uint16_t* dst = p.out + (size_t)m * p.N + n;
-            if(n + 3 < p.N)
+            if(vec_ok)
             {
-                *(u32x2*)dst = u32x2{pack2<DT>(acc[i][j][0], acc[i][j][1]),
-                                     pack2<DT>(acc[i][j][2], acc[i][j][3])};
+                *(u32x4*)dst = vv;
             }
             else
             {
 #pragma unroll
-                for(int r = 0; r < 4; ++r)
+                for(int r = 0; r < 8; ++r)
                     if(n + r < p.N)
-                        dst[r] = (uint16_t)(pack2<DT>(acc[i][j][r], 0.f) & 0xffffu);
+                        dst[r] = (uint16_t)((vv[r >> 1] >> ((r & 1) * 16)) & 0xffffu);
             }
         }
     }
+    // the next tile's first slabs must not land in LDS while another wave still reads its block
+    __syncthreads();
+    } // tiles of this workgroup
 }
 
 } // namespace
@@ -367,16 +398,40 @@ bool gemm_prefill_supports(const GemmKernelParams& p)
 hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, hipStream_t stream)
 {
     const int    tiles_m = (p.M + kBM - 1) / kBM, tiles_n = (p.N + kBN - 1) / kBN;
-    const size_t smem    = (size_t)kStages * kStageBytes;
+    // the two stages, or the eight waves' output blocks of the epilogue, whichever is larger
+    const size_t smem    = std::max((size_t)kStages * kStageBytes, (size_t)8 * 64 * kEpiPitch);
     const bool   bf      = out_dtype == In16::bf16;
     auto         kernel  = p.w_shuffled ? (bf ? gemm_prefill_kernel<In16::bf16, true> : gemm_prefill_kernel<In16::fp16, true>)
                                         : (bf ? gemm_prefill_kernel<In16::bf16, false> : gemm_prefill_kernel<In16::fp16, false>);
-    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)smem);
+    // Per device and instantiation, once: the opt-in to more than 64 KiB of LDS, and the number of
+    // compute units.  (Racing first calls repeat the same idempotent set-up.)
+    constexpr int kMaxDevices = 64;
+    static int    cus_of[kMaxDevices];
+    static bool   ready[kMaxDevices][4];
+    int           device = 0, cus = 0;
+    hipError_t    e = hipGetDevice(&device);
     if(e != hipSuccess)
         return e;
-    hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(kThreads), smem, stream, p, tiles_m,
-                       tiles_n);
+    const int inst = (p.w_shuffled ? 2 : 0) + (bf ? 0 : 1);
+    if(device < 0 || device >= kMaxDevices || !ready[device][inst])
+    {
+        if((e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem)) != hipSuccess ||
+           (e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device)) != hipSuccess)
+            return e;
+        if(device >= 0 && device < kMaxDevices)
+        {
+            cus_of[device]      = cus;
+            ready[device][inst] = true;
+        }
+    }
+    else
+        cus = cus_of[device];
+    // one workgroup fills a compute unit (LDS, registers); with more tiles than compute units the
+    // workgroups walk the tiles.  A multiple of 8 keeps a workgroup's tiles on one XCD's patch order.
+    const int total = tiles_m * tiles_n;
+    const int grid  = (total > cus && cus >= 8) ? (cus & ~7) : total;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), smem, stream, p, tiles_m, tiles_n);
     return hipGetLastError();
 }
 

@@ -332,3 +332,66 @@ def test_kernel_choice_query_names_what_runs(m, n, k):
     named = torch.empty_like(auto)
     aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, xs, ws, named, splitK=-1, kernelName=cfg["kernelName"])
     assert torch.equal(auto, named), cfg
+
+
+def _gpu_problem(m, n, k, seed, outliers=False):
+    """Operands made on the GPU (too big for the CPU helpers to be quick): x ~ N(0,1), optionally
+    1 % of channels x50, quantised 1x128; w ~ N(0,0.02) quantised per 128x128 block.  Both
+    quantisers are checked bit for bit against the oracle in their own tests."""
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    x = torch.randn(m, k, generator=g, device=DEV)
+    if outliers:
+        x[:, torch.randperm(k, generator=g, device=DEV)[: max(1, k // 100)]] *= 50.0
+    xq, xs = aiter_amd.get_hip_quant(aiter_amd.QuantType.per_1x128)(x.bfloat16(), quant_dtype=dtypes.fp8)
+    del x
+    w = (torch.randn(n, k, generator=g, device=DEV) * 0.02).bfloat16()
+    wq, ws = aiter_amd.weight_per_128x128_quant(w, quant_dtype=dtypes.fp8)
+    return xq, wq, xs, ws
+
+
+def _check_rows_against_f64(out, xq, wq, xs, ws, rows, what):
+    ref = tr.gemm_a8w8_blockscale_ref_f64(xq[rows].cpu(), wq.cpu(), xs[rows].cpu(), ws.cpu())
+    o = out[rows].cpu().double()
+    err = (o - ref).abs()
+    bad = (err > ATOL + RTOL * ref.abs()).sum().item()
+    assert bad == 0, f"{what}: {bad} of {o.numel()} outside rtol=atol=1e-2, max abs err {err.max().item():.4g}"
+
+
+@pytest.mark.parametrize("m,n,k", [(4352, 4096, 256), (4352, 4352, 128), (4100, 4360, 256)])
+def test_prefill_kernel_more_tiles_than_compute_units(m, n, k):
+    # 272 / 289 / 306 tiles of 256x256 on 256 compute units: workgroups take a second tile (a
+    # multiple of 8 tiles with the per-XCD renumbering, not a multiple, ragged edges)
+    xq, wq, xs, ws = _gpu_problem(m, n, k, seed=m + n + k)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, xs, ws, out, kernelName="prefill_256x256")
+    tile = torch.empty_like(out)
+    aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, xs, ws, tile, kernelName="tile_128x128")
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), tile.view(torch.int16))
+    rows = torch.tensor([0, 255, 256, 2047, 4095, 4096, m - 1], device=DEV)
+    _check_rows_against_f64(out, xq, wq, xs, ws, rows, f"prefill {m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("layout", ["plain", "preshuffled"])
+def test_config4_full_size(layout):
+    # BASELINE config 4: M=8192, N=36864, K=7168 through the library's own kernel choice.  Every
+    # output is compared bit for bit with the generic tile kernel (same products, same order of
+    # additions), and 16 rows x all N with the fp64 reference on the CPU.
+    m, n, k = 8192, 36864, 7168
+    xq, wq, xs, ws = _gpu_problem(m, n, k, seed=4, outliers=True)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    if layout == "preshuffled":
+        xs_t = xs.t().contiguous().t()  # column-major x_scale, as the quantiser's transpose_scale=True gives
+        wsh = aiter_amd.shuffle_weight(wq.view(torch.uint8)).view(wq.dtype)
+        aiter_amd.gemm_a8w8_blockscale_bpreshuffle_ck(xq, wsh, xs_t, ws, out)
+        del wsh
+    else:
+        aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, xs, ws, out, splitK=-1)
+    tile = torch.empty_like(out)
+    aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, xs, ws, tile, kernelName="tile_128x128")
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), tile.view(torch.int16))
+    del tile
+    rows = torch.tensor([0, 1, 255, 256, 1000, 2047, 2048, 3333, 4095, 4096, 5000, 6143, 6144, 7777, 8190, 8191],
+                        device=DEV)
+    _check_rows_against_f64(out, xq, wq, xs, ws, rows, f"config 4 {layout}")
