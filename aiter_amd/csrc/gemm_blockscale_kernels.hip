@@ -174,11 +174,7 @@ const char* gemm_kernel_names() { return kKernelNames; }
 // gains more when the weights are still in the last-level cache.
 static const char* automatic_choice(const GemmKernelParams& p)
 {
-    const int64_t prefill_tiles  = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
-    const int64_t prefill_rounds = (prefill_tiles + 255) / 256;
-    const float   prefill_share  = (float)prefill_tiles / (float)(prefill_rounds * 256);
-    const float   prefill_iter   = 1.7f + (prefill_share > 0.56f ? (prefill_share - 0.56f) * 0.9f : 0.f);
-    const float   prefill_us     = 13.5f + (float)prefill_rounds * (float)p.kblocks * prefill_iter;
+    const float prefill_us = gemm_prefill_plan(p, 256).us; // fitted on a 256-CU part, like the mid model
     if(p.M <= 64 && gemm_decode_supports(p))
         return "decode_stream";
     if(gemm_mid_supports(p) && (!gemm_prefill_supports(p) || gemm_mid_estimate_us(p) * 1.03f < prefill_us))
@@ -241,14 +237,23 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
         *why = "splitK > 0 is only available with the decode_stream and mid_* kernels";
         return hipErrorInvalidValue;
     }
-    if(strcmp(name, "prefill_256x256") == 0)
+    // "prefill_256x256" by name keeps every tile in one workgroup (bitwise the result of the
+    // tile_* kernels); "prefill_256x256:s=2" pins the number of K ranges per tile; chosen
+    // automatically, the launcher decides
+    if(strncmp(name, "prefill_256x256", 15) == 0 && (name[15] == 0 || name[15] == ':'))
     {
+        int splits = (a.kernel_name && a.kernel_name[0]) ? 1 : 0;
+        if(name[15] == ':' && (sscanf(name + 15, ":s=%d", &splits) != 1 || splits < 1 || splits > 16))
+        {
+            *why = "unknown kernelName (see aiter_fp8bs_gemm_kernel_names())";
+            return hipErrorInvalidValue;
+        }
         if(!gemm_prefill_supports(p))
         {
             *why = "prefill_256x256 needs N % 4 == 0 and operand matrices below 4 GiB";
             return hipErrorInvalidValue;
         }
-        return launch_gemm_prefill(p, DT, stream);
+        return launch_gemm_prefill(p, DT, stream, splits);
     }
     *why = "unknown kernelName (see aiter_fp8bs_gemm_kernel_names())";
     return hipErrorInvalidValue;

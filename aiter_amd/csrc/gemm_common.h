@@ -71,7 +71,16 @@ __device__ __forceinline__ uint32_t lds_off(uint32_t row, uint32_t chunk)
 
 
 // launchers living in their own translation units
-hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, hipStream_t stream);
+// K ranges per tile that the prefill kernel would choose on `cus` compute units, and the modelled
+// duration (us) with them
+struct PrefillPlan
+{
+    int   splits;
+    float us;
+};
+PrefillPlan gemm_prefill_plan(const GemmKernelParams& p, int cus);
+// want_splits: K ranges per tile; 0 lets the launcher choose, 1 keeps a tile in one workgroup
+hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, hipStream_t stream, int want_splits);
 bool       gemm_prefill_supports(const GemmKernelParams& p);
 hipError_t launch_gemm_decode(const GemmKernelParams& p, In16 out_dtype, int split_k_log2, int device_id,
                               hipStream_t stream, const char* tuning = nullptr);

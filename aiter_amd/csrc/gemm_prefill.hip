@@ -43,7 +43,10 @@ __device__ __forceinline__ i32x8 read_frag(const uint8_t* base, uint32_t row, ui
 // tile), and a lane's fragment halves sit at kg*512 + l16*16 and 256 bytes further.
 template <In16 DT, bool SHUF>
 __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams p, int tiles_m,
-                                                                int tiles_n)
+                                                                int tiles_n, int splits,
+                                                                int kb_per_split, float* partial,
+                                                                uint32_t partial_bytes,
+                                                                uint32_t* tickets)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
@@ -54,9 +57,14 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     // The workgroup walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... (one workgroup per compute
     // unit when there are more tiles than compute units): a tile's output stores drain, and the
     // next tile's first slabs arrive, behind one wait instead of a workgroup's end and start.
+    // With fewer tiles than compute units the K blocks of a tile are shared out over `splits`
+    // workgroups (item = split * tiles + tile); see the epilogue for how their sums meet.
     const int total = tiles_m * tiles_n;
-    for(int tile = blockIdx.x; tile < total; tile += gridDim.x)
+    __shared__ uint32_t s_ticket;
+    for(int item = blockIdx.x; item < total * splits; item += gridDim.x)
     {
+    const int split = item / total, tile = item - split * total;
+    const int kb_lo = split * kb_per_split, kb_hi = min(p.kblocks, kb_lo + kb_per_split);
     // Everything derived from the lane index is derived again for every tile (the empty asm
     // hides that it is the same value): kept live across the K loop it would not fit the registers.
     int t = threadIdx.x;
@@ -196,7 +204,7 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         const int k = kb0 + lane;
         return ws_row[k < p.kblocks ? k : p.kblocks - 1];
     };
-    float ws_vec = load_ws_window(0);
+    float ws_vec = load_ws_window(kb_lo & ~63);
     auto  ws_at  = [&](int kb) -> float {
         return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(ws_vec), kb & 63));
     };
@@ -205,10 +213,11 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         const uint32_t dst0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(smem3 + wave * 1024));
 #pragma unroll
         for(int i = 0; i < 8; ++i)
-            dma16(dst0 + i * 8192, goff[i], i < 4 ? p.wq : p.xq);
+            dma16(dst0 + i * 8192, goff[i],
+                  i < 4 ? p.wq + (size_t)kb_lo * (SHUF ? 2048 : 128) : p.xq + (size_t)kb_lo * 128);
         if(wave < 4)
             dma4(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(smem3 + kSlabBytes + wave * 256)),
-                 xs_goff, p.xs);
+                 xs_goff + (uint32_t)kb_lo * (uint32_t)p.xs_k * 4u, p.xs);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's LDS-direct loads have landed
     __syncthreads();
@@ -243,17 +252,17 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
 
     typedef const volatile float __attribute__((address_space(3)))* lds_f32_ptr;
 
-    for(int kb = 0; kb < p.kblocks; ++kb)
+    for(int kb = kb_lo; kb < kb_hi; ++kb)
     {
-        const int      cur      = kb & 1;
+        const int      cur      = (kb - kb_lo) & 1;
         const uint32_t stage    = (uint32_t)cur * kStageBytes;
-        const int      kn       = kb + 1 < p.kblocks ? kb + 1 : kb; // last pass re-fetches, unused
+        const int      kn       = kb + 1 < kb_hi ? kb + 1 : kb; // last pass re-fetches, unused
         const uint32_t dma_dst  = __builtin_amdgcn_readfirstlane(
             (uint32_t)(uintptr_t)(smem3 + (cur ^ 1) * kStageBytes + wave * 1024));
         const size_t   dma_koff   = (size_t)kn * 128;
         const size_t   dma_koff_w = SHUF ? (size_t)kn * 2048 : dma_koff;
 
-        if((kb & 63) == 0 && kb != 0)
+        if((kb & 63) == 0 && kb != kb_lo)
             ws_vec = load_ws_window(kb);
         const float wsc = ws_at(kb);
 
@@ -337,12 +346,70 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
 #undef FP8BS_MFMA
 #undef FP8BS_FMA4
 
+    // ---- K shared out over workgroups: every workgroup parks its fp32 accumulators in the
+    // workspace exactly as its lanes hold them (item slot x 32 MFMA tiles x 512 lanes x 16 bytes:
+    // every store and load is 1 KiB contiguous per wave), takes a ticket, and the one that draws
+    // the last ticket of the tile adds the slots in split order (so the result does not depend on
+    // who came last) and carries on into the ordinary epilogue.  The workgroups of a tile run on
+    // different XCDs, whose L2 caches are not coherent with each other: the parked tiles are
+    // written and read past them (sc1), and the stores are waited for before the ticket is taken.
+    bool writes_out = true;
+    if(splits > 1)
+    {
+        const __amdgpu_buffer_rsrc_t rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(partial, 0, (int)partial_bytes, 0x00020000);
+        constexpr int kCoherent = 16;
+        const uint32_t mine     = ((uint32_t)(tile * splits + split) * 32u * 512u + (uint32_t)t) * 16u;
+#pragma unroll
+        for(int i = 0; i < 8; ++i)
+#pragma unroll
+            for(int j = 0; j < 4; ++j)
+                __builtin_amdgcn_raw_buffer_store_b128(
+                    __builtin_bit_cast(u32x4, f32x4{acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]}),
+                    rsrc, mine + (uint32_t)(i * 4 + j) * (512u * 16u), 0, kCoherent);
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): the stores above have reached memory
+        __syncthreads();
+        if(t == 0)
+            s_ticket = __hip_atomic_fetch_add(tickets + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        writes_out = s_ticket == (uint32_t)splits - 1u;
+        if(writes_out)
+        {
+            if(t == 0) // leave the ticket ready for the next launch
+                __hip_atomic_store(tickets + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for(int i = 0; i < 8; ++i)
+#pragma unroll
+                for(int j = 0; j < 4; ++j)
+                {
+                    // 0 + p0 + p1 + ... whoever is last; its own term comes from its registers
+                    // (the same bits it parked), the others from the workspace
+                    const f32x4 own = f32x4{acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+                    f32x4       sum = f32x4{0.f, 0.f, 0.f, 0.f};
+                    for(int sp = 0; sp < splits; ++sp)
+                    {
+                        const uint32_t off =
+                            ((uint32_t)(tile * splits + sp) * 32u * 512u + (uint32_t)t) * 16u +
+                            (uint32_t)(i * 4 + j) * (512u * 16u);
+                        if(sp == split) // uniform
+                            sum += own;
+                        else
+                            sum += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, kCoherent));
+                    }
+#pragma unroll
+                    for(int r = 0; r < 4; ++r)
+                        acc[i][j][r] = sum[r];
+                }
+        }
+    }
+
     // ---- epilogue.  A lane owns out[m][n .. n+3] for each of its 8 x 4 tiles: stored from there,
     // one instruction would touch 16 rows with 32 bytes each.  The wave's 64 x 128 block goes
     // through its own LDS region instead (the stage buffers are free after the loop's last
     // barrier; rows padded to 272 bytes so the 16 rows of one write fall on different banks) and
     // leaves as 16-byte stores, 16 lanes per 256-byte row piece, 4 rows per instruction.  LDS
     // operations of one wave complete in order, so no barrier stands between write and read.
+    if(writes_out) // uniform
     {
         const uint32_t ebase = (uint32_t)wave * (64u * kEpiPitch);
         typedef u32x2 __attribute__((address_space(3)))*       lds_u2_ptr;
@@ -382,7 +449,7 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     }
     // the next tile's first slabs must not land in LDS while another wave still reads its block
     __syncthreads();
-    } // tiles of this workgroup
+    } // items of this workgroup
 }
 
 } // namespace
@@ -395,7 +462,40 @@ bool gemm_prefill_supports(const GemmKernelParams& p)
            (uint64_t)p.M * (uint64_t)p.kblocks < (1ull << 30) && (p.N % 4) == 0;
 }
 
-hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, hipStream_t stream)
+// Duration model (us) on `cus` compute units, fitted to event timings with weights from HBM:
+// a round of workgroups costs 8 us (first slabs, output tile) plus, per K block, 1.36 us while
+// the workgroups of a round cover up to 44 % of the compute units, rising to 1.79 us when they
+// cover all (8192 x 36864 x 7168: 18 rounds x (8 + 56 x 1.79) = 1948 us, measured 1950).  K
+// ranges over s workgroups per tile cost 4 us plus the parked tiles' traffic, (2 s - 1) x 256 KiB
+// per tile at about 5 TB/s (2048 x 4096 x 7168: 89.8 us as one range, 77-80 us as two).
+PrefillPlan gemm_prefill_plan(const GemmKernelParams& p, int cus)
+{
+    const int tiles = ((p.M + kBM - 1) / kBM) * ((p.N + kBN - 1) / kBN);
+    cus             = std::max(cus, 1);
+    auto cost = [&](int s) {
+        const int   items  = tiles * s;
+        const int   rounds = (items + cus - 1) / cus;
+        const float share  = (float)items / (float)(rounds * cus);
+        const float iter   = 1.36f + (share > 0.44f ? (share - 0.44f) * 0.77f : 0.f);
+        const int   kb     = (p.kblocks + s - 1) / s;
+        return (float)rounds * (8.f + (float)kb * iter) +
+               (s > 1 ? 4.f + (float)tiles * (float)(2 * s - 1) * 0.05f : 0.f);
+    };
+    PrefillPlan best{1, cost(1)};
+    for(int s = 2; s <= 3; ++s)
+    {
+        // (below 64 tiles the model is off: 1024 x 2112 x 7168, 36 tiles x 3, takes 67 us where it
+        // says 47, and the mid_* kernels need 51)
+        if(tiles < 64 || tiles * s > cus || p.kblocks / s < 8 || (p.N & 3) != 0)
+            break;
+        const float c = cost(s);
+        if(c < best.us * 0.97f)
+            best = PrefillPlan{s, c};
+    }
+    return best;
+}
+
+hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, hipStream_t stream, int want_splits)
 {
     const int    tiles_m = (p.M + kBM - 1) / kBM, tiles_n = (p.N + kBN - 1) / kBN;
     // the two stages, or the eight waves' output blocks of the epilogue, whichever is larger
@@ -430,8 +530,26 @@ hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, hipStr
     // one workgroup fills a compute unit (LDS, registers); with more tiles than compute units the
     // workgroups walk the tiles.  A multiple of 8 keeps a workgroup's tiles on one XCD's patch order.
     const int total = tiles_m * tiles_n;
-    const int grid  = (total > cus && cus >= 8) ? (cus & ~7) : total;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), smem, stream, p, tiles_m, tiles_n);
+    // want_splits: 0 = the plan's choice, otherwise as told
+    int splits = want_splits > 0 ? want_splits : gemm_prefill_plan(p, cus).splits;
+    if(total * splits > 4096) // 32-bit byte offsets into the parked tiles
+        splits = 1;
+    splits                 = std::max(1, std::min(splits, (int)p.kblocks));
+    const int kb_per_split = (p.kblocks + splits - 1) / splits;
+    splits                 = (p.kblocks + kb_per_split - 1) / kb_per_split;
+    float*    partial = nullptr;
+    uint32_t* tickets = nullptr;
+    size_t    bytes   = 0;
+    if(splits > 1)
+    {
+        bytes = (size_t)total * splits * 32 * 512 * 16;
+        if((e = gemm_split_workspace(device, bytes, (size_t)total, stream, &partial, &tickets)) != hipSuccess)
+            return e;
+    }
+    const int items = total * splits;
+    const int grid  = (items > cus && cus >= 8) ? (cus & ~7) : items;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), smem, stream, p, tiles_m, tiles_n, splits,
+                       kb_per_split, partial, (uint32_t)bytes, tickets);
     return hipGetLastError();
 }
 

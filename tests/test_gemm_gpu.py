@@ -395,3 +395,31 @@ def test_config4_full_size(layout):
     rows = torch.tensor([0, 1, 255, 256, 1000, 2047, 2048, 3333, 4095, 4096, 5000, 6143, 6144, 7777, 8190, 8191],
                         device=DEV)
     _check_rows_against_f64(out, xq, wq, xs, ws, rows, f"config 4 {layout}")
+
+
+@pytest.mark.parametrize("m,n,k,name", [
+    (512, 768, 2048, "prefill_256x256:s=2"),   # 6 tiles x 2 ranges of 8 K blocks
+    (300, 1000, 1408, "prefill_256x256:s=3"),  # ragged tiles, 11 K blocks as 4 + 4 + 3
+    (256, 256, 4096, "prefill_256x256:s=4"),   # one tile, four workgroups
+    (2048, 4096, 7168, ""),                    # BASELINE config 5's GEMM: the library's own choice (2 ranges)
+])
+def test_prefill_kernel_k_ranges_across_workgroups(m, n, k, name):
+    xq, wq, xs, ws = _gpu_problem(m, n, k, seed=m + n + k, outliers=True)
+    outs = []
+    for _ in range(3):  # the tickets must be back at zero after every launch
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+        if name:
+            aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, xs, ws, out, kernelName=name)
+        else:
+            aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, xs, ws, out, splitK=-1)
+        outs.append(out)
+    tile = torch.empty_like(outs[0])
+    aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, xs, ws, tile, kernelName="tile_128x128")
+    torch.cuda.synchronize()
+    # the ranges are added in range order whichever workgroup finishes last: same bits every time
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
+    # against one workgroup per tile only the grouping of the fp32 additions differs
+    assert (outs[0].view(torch.int16) != tile.view(torch.int16)).float().mean().item() < 0.02
+    rows = torch.tensor(sorted({0, 1, 255, m // 2, m - 1}), device=DEV)
+    _check_rows_against_f64(outs[0], xq, wq, xs, ws, rows, f"{name or 'auto'} {m}x{n}x{k}")
