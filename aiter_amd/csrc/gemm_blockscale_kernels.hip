@@ -296,6 +296,8 @@ void gemm_describe_choice(int64_t M, int64_t N, int64_t K, bool shuffled, char* 
     const char* name = automatic_choice(p);
     if(strcmp(name, "mid_auto") == 0)
         gemm_mid_describe(p, buf, n);
+    else if(strcmp(name, "prefill_256x256") == 0 && gemm_prefill_plan(p, 256).splits > 1)
+        snprintf(buf, n, "%s:s=%d", name, gemm_prefill_plan(p, 256).splits); // as on a 256-CU part
     else
         snprintf(buf, n, "%s", name);
 }

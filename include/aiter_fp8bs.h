@@ -181,7 +181,7 @@ const char* aiter_fp8bs_gemm_kernel_names(void);
 
 /* The kernel the library takes for contiguous operands of shape M x N x K when kernelName is empty,
  * written to `out` (at least 32 characters) in the form kernelName accepts, e.g. "decode_stream",
- * "prefill_256x256", "mid_128x128:s=2".  Host-only: no device is touched.  The counterpart of the
+ * "prefill_256x256", "prefill_256x256:s=2", "mid_128x128:s=2" (":s=" = K ranges per tile).  Host-only: no device is touched.  The counterpart of the
  * reference's lookup in its tuned tables, get_CKGEMM_config (aiter/ops/gemm_op_a8w8.py:448-490):
  * here the choice is a shape rule inside the library. */
 int aiter_fp8bs_gemm_choice(int64_t M, int64_t N, int64_t K, int preshuffled, char* out, int64_t out_len);

@@ -38,7 +38,8 @@ def test_kernel_choice_query_on_the_headline_shapes():
         for n, k in ((7168, 2048), (24576, 1536), (2112, 7168)):
             assert aiter_amd.get_CKGEMM_config(m, n, k)["kernelName"] == "decode_stream"
     assert aiter_amd.get_CKGEMM_config(8192, 36864, 7168)["kernelName"] == "prefill_256x256"
-    assert aiter_amd.get_CKGEMM_config(2048, 4096, 7168)["kernelName"] == "prefill_256x256"
+    cfg5 = aiter_amd.get_CKGEMM_config(2048, 4096, 7168)  # 128 tiles: two K ranges per tile
+    assert cfg5["kernelName"] == "prefill_256x256:s=2" and cfg5["kRanges"] == 2
     cfg = aiter_amd.get_CKGEMM_config(128, 4096, 7168)  # few tiles, long K: K is split
     assert cfg["kernelName"].startswith("mid_") and cfg["kRanges"] > 1 and cfg["libtype"] == "hip"
     for m, n, k in ((65, 512, 128), (300, 1000, 384), (4096, 2112, 7168), (100000, 128, 128)):
