@@ -51,6 +51,7 @@ EXPORTED_SYMBOLS = sorted(
         "aiter_clear_last_error",
         "aiter_fp8bs_gemm_kernel_names",
         "aiter_fp8bs_gemm_choice",
+        "aiter_fp8bs_gemm_resolve",
     ]
 )
 
@@ -78,6 +79,9 @@ def load_library():
         lib.aiter_fp8bs_gemm_choice.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
                                                 ctypes.c_char_p, ctypes.c_int64]
         lib.aiter_fp8bs_gemm_choice.restype = ctypes.c_int
+        lib.aiter_fp8bs_gemm_resolve.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int,
+                                                 ctypes.c_int64, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int64]
+        lib.aiter_fp8bs_gemm_resolve.restype = ctypes.c_int
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(lib, name)
             fn.argtypes = argtypes + [ctypes.c_void_p]
@@ -139,3 +143,15 @@ def gemm_choice(m: int, n: int, k: int, preshuffled: bool = False) -> str:
         raw = lib.aiter_get_last_error()
         raise RuntimeError(f"aiter_fp8bs_gemm_choice failed: {raw.decode(errors='replace') if raw else '?'}")
     return buf.value.decode()
+
+
+def gemm_resolve(m: int, n: int, k: int, split_k: int = 0, kernel_name: str = "", preshuffled: bool = False):
+    """(kernel, splitK) that a call with this (kernelName, splitK) pair runs; host-only."""
+    lib = load_library()
+    buf = ctypes.create_string_buffer(96)
+    if lib.aiter_fp8bs_gemm_resolve(int(m), int(n), int(k), 1 if preshuffled else 0, int(split_k),
+                                    (kernel_name or "").encode(), buf, 96) != 0:
+        raw = lib.aiter_get_last_error()
+        raise RuntimeError(f"aiter_fp8bs_gemm_resolve failed: {raw.decode(errors='replace') if raw else '?'}")
+    name, _, tail = buf.value.decode().partition(";splitK=")
+    return name, int(tail)

@@ -17,7 +17,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_NAME = "libaiter_fp8bs.so"
 LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 
-SOURCES = ["abi.hip", "norm_quant_kernels.hip", "gemm_blockscale_kernels.hip", "gemm_prefill.hip", "gemm_decode.hip",
+SOURCES = ["abi.hip", "workspace.hip", "norm_quant_kernels.hip", "gemm_blockscale_kernels.hip", "gemm_prefill.hip", "gemm_decode.hip",
            "gemm_mid.hip", "moe_kernels.hip"]
 
 # -ffp-contract=off: the quantiser's rounding sequence must stay one IEEE operation per step.
@@ -62,7 +62,7 @@ def build_library(verbose: bool = False) -> str:
     """Compile every HIP translation unit and link the shared library. Returns its path."""
     obj_dir = os.path.join(PKG_DIR, "build")
     os.makedirs(obj_dir, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=min(6, len(SOURCES))) as ex:
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
         objs = list(ex.map(lambda s: _compile(s, obj_dir, verbose), SOURCES))
     tmp = LIB_PATH + ".tmp"
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]

@@ -391,8 +391,9 @@ static int gemm_blockscale_common(const char* fn, bool preshuffled, aiter_tensor
         check_aligned(fn, w_scale, "w_scale", 4);
         if(M > 0x7fffffffLL / 2 || N > 0x7fffffffLL / 2 || K > 0x7fffffffLL / 2)
             fail(fn, "problem too large");
-        if(splitK < -1 || splitK > 4)
-            fail(fn, "splitK = ", splitK, " outside -1..4");
+        // csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale.cu:82-114 takes 0..30 (KBatch = 1 << splitK)
+        if(splitK < -1 || splitK > 30)
+            fail(fn, "splitK = ", splitK, " outside -1..30");
         if(M == 0 || N == 0)
             return;
 
@@ -443,6 +444,24 @@ int aiter_fp8bs_gemm_choice(int64_t M, int64_t N, int64_t K, int preshuffled, ch
            K > 0x7fffffffLL / 2)
             fail(fn, "M and N must be positive and K a positive multiple of 128, got ", M, " x ", N, " x ", K);
         fp8bs::gemm_describe_choice(M, N, K, preshuffled != 0, out, (size_t)out_len);
+    });
+}
+
+int aiter_fp8bs_gemm_resolve(int64_t M, int64_t N, int64_t K, int preshuffled, int64_t splitK, const char* kernelName,
+                             char* out, int64_t out_len)
+{
+    return guarded([&] {
+        const char* fn = "aiter_fp8bs_gemm_resolve";
+        if(out == nullptr || out_len < 64)
+            fail(fn, "out must hold at least 64 characters");
+        if(M < 1 || N < 1 || K < 128 || K % 128 != 0 || M > 0x7fffffffLL / 2 || N > 0x7fffffffLL / 2 ||
+           K > 0x7fffffffLL / 2)
+            fail(fn, "M and N must be positive and K a positive multiple of 128, got ", M, " x ", N, " x ", K);
+        if(splitK < -1 || splitK > 30)
+            fail(fn, "splitK = ", splitK, " outside -1..30");
+        const char* why = nullptr;
+        if(!fp8bs::gemm_describe_request(M, N, K, preshuffled != 0, (int)splitK, kernelName, out, (size_t)out_len, &why))
+            fail(fn, why ? why : "cannot resolve the request");
     });
 }
 
@@ -779,7 +798,9 @@ int moe_sorting_fwd(aiter_tensor_t* topk_ids, aiter_tensor_t* topk_weights, aite
         if(max_padded >= (1LL << 31))
             fail(fn, "problem too large");
         DeviceGuard guard(topk_ids->device_id);
-        check_hip(fn, fp8bs::launch_moe_sorting(a, (hipStream_t)stream), nullptr);
+        const char* why = nullptr;
+        hipError_t  e   = fp8bs::launch_moe_sorting(a, (hipStream_t)stream, &why);
+        check_hip(fn, e, why);
     });
 }
 
@@ -949,7 +970,9 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
         if(M == 0)
             return; // nothing to do, and no device needed to say so
         DeviceGuard guard(input->device_id);
-        check_hip(fn, fp8bs::launch_fmoe_blockscale(a, (hipStream_t)stream), nullptr);
+        const char* why = nullptr;
+        hipError_t  e   = fp8bs::launch_fmoe_blockscale(a, (hipStream_t)stream, &why);
+        check_hip(fn, e, why);
     });
 }
 

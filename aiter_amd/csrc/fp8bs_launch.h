@@ -79,5 +79,8 @@ hipError_t launch_gemm_blockscale(const GemmArgs& a, hipStream_t stream, const c
 const char* gemm_kernel_names();
 // the kernel (and, for the mid_* family, K range count) taken for contiguous operands of this shape when none is named
 void gemm_describe_choice(int64_t M, int64_t N, int64_t K, bool shuffled, char* buf, size_t n);
+// what a call's (kernelName, splitK) pair resolves to, as "<kernel>;splitK=<n>"; false + *why for an unknown name
+bool gemm_describe_request(int64_t M, int64_t N, int64_t K, bool shuffled, int split_k_log2, const char* kernel_name,
+                           char* buf, size_t n, const char** why);
 
 } // namespace fp8bs

@@ -184,78 +184,138 @@ static const char* automatic_choice(const GemmKernelParams& p)
     return "tile_128x128";
 }
 
+// Names of the reference's own kernel zoo ("a8w8_blockscale_1x128x128_256x16x128x256_..."), as
+// its tuned tables hand them out (aiter/configs/model_configs/a8w8_blockscale_tuned_gemm_ds_v3.csv),
+// say nothing about the kernels here.
+static bool foreign_kernel_name(const char* name) { return strncmp(name, "a8w8_blockscale_", 16) == 0; }
+
+// What a call's (kernelName, splitK) pair asks for.  splitK is a hint, never a reason to fail:
+//  * a foreign name is dropped together with its splitK (tuned for that kernel): the library chooses;
+//  * no name and splitK <= 0: the library chooses kernel and K ranges (the reference's default
+//    splitK = 0 with no name means "nothing tuned", csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale.cu:82-114);
+//  * no name and splitK > 0: the automatic kernel with 2^splitK K ranges where that kernel can
+//    split K (clamped to what the problem allows), ignored where it cannot;
+//  * one of this library's names: that kernel; splitK = 0 keeps K in one range, > 0 as above.
+struct KernelRequest
+{
+    const char* name;         // one of this library's names, never null
+    int         split_k_log2; // -1 = choose
+};
+static KernelRequest resolve_request(const GemmArgs& a, const GemmKernelParams& p)
+{
+    const bool named = a.kernel_name && a.kernel_name[0] && !foreign_kernel_name(a.kernel_name);
+    if(named)
+        return KernelRequest{a.kernel_name, a.split_k_log2};
+    const bool foreign = a.kernel_name && a.kernel_name[0];
+    return KernelRequest{automatic_choice(p), (foreign || a.split_k_log2 <= 0) ? -1 : a.split_k_log2};
+}
+
+// One of this library's kernel names, taken apart.
+enum class Family
+{
+    tile,
+    decode,
+    mid,
+    prefill
+};
+struct ParsedKernel
+{
+    Family      family;
+    int         tile;   // tile: 16256 / 64128 / 128128; mid: 0 (choose) / 64 / 64128 / 128
+    int         splits; // ":s=<n>" of mid_* and prefill_256x256, 0 when absent
+    const char* tuning; // what follows "decode_stream:", or null
+};
+static const char* const kUnknownName = "unknown kernelName (see aiter_fp8bs_gemm_kernel_names())";
+
+static bool parse_kernel_name(const char* name, ParsedKernel* out)
+{
+    *out = ParsedKernel{Family::tile, 0, 0, nullptr};
+    if(strcmp(name, "tile_16x256") == 0 || strcmp(name, "tile_64x128") == 0 || strcmp(name, "tile_128x128") == 0)
+    {
+        out->tile = name[5] == '1' ? (name[6] == '6' ? 16256 : 128128) : 64128;
+        return true;
+    }
+    // "decode_stream" alone, or "decode_stream:r=2,s=4,w=4,g=256" to pin its work split
+    if(strncmp(name, "decode_stream", 13) == 0 && (name[13] == 0 || name[13] == ':'))
+    {
+        out->family = Family::decode;
+        out->tuning = name[13] == ':' ? name + 14 : nullptr;
+        return true;
+    }
+    const char*  colon = strchr(name, ':');
+    const size_t len   = colon ? (size_t)(colon - name) : strlen(name);
+    auto         is    = [&](const char* s) { return strlen(s) == len && strncmp(name, s, len) == 0; };
+    // "mid_128x128" alone, or "mid_128x128:s=7" to pin the number of K ranges
+    if(strncmp(name, "mid_", 4) == 0)
+    {
+        out->family = Family::mid;
+        out->tile   = is("mid_128x128") ? 128 : is("mid_64x128") ? 64128 : is("mid_64x64") ? 64 : is("mid_auto") ? 0 : -1;
+        if(colon && (sscanf(colon, ":s=%d", &out->splits) != 1 || out->splits < 1 || out->splits > 64))
+            return false;
+        return out->tile >= 0;
+    }
+    // "prefill_256x256", or "prefill_256x256:s=2" to pin the number of K ranges per tile
+    if(is("prefill_256x256"))
+    {
+        out->family = Family::prefill;
+        if(colon && (sscanf(colon, ":s=%d", &out->splits) != 1 || out->splits < 1 || out->splits > 16))
+            return false;
+        return true;
+    }
+    return false;
+}
+
 template <In16 DT>
 static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStream_t stream,
                            const char** why)
 {
-    const char* name = (a.kernel_name && a.kernel_name[0]) ? a.kernel_name : automatic_choice(p);
-    if(strcmp(name, "tile_16x256") == 0)
-        return launch_tile<DT, 16, 256, 1, 4>(p, stream);
-    if(strcmp(name, "tile_64x128") == 0)
-        return launch_tile<DT, 64, 128, 2, 2>(p, stream);
-    if(strcmp(name, "tile_128x128") == 0)
-        return launch_tile<DT, 128, 128, 2, 2>(p, stream);
-    // "decode_stream" alone, or "decode_stream:r=2,s=4,w=4,g=256" to pin its work split
-    if(strncmp(name, "decode_stream", 13) == 0 && (name[13] == 0 || name[13] == ':'))
+    const KernelRequest req   = resolve_request(a, p);
+    const bool          named = req.name == a.kernel_name;
+    ParsedKernel        k;
+    if(!parse_kernel_name(req.name, &k))
     {
-        const char* tuning = name[13] == ':' ? name + 14 : nullptr;
+        *why = kUnknownName;
+        return hipErrorInvalidValue;
+    }
+    LaunchCtx ctx;
+    ctx.device_id = a.device_id;
+    ctx.stream    = stream;
+    ctx.why       = why;
+    switch(k.family)
+    {
+    case Family::tile:
+        // (these keep a tile's K in one workgroup: splitK is a hint they have no use for)
+        if(k.tile == 16256)
+            return launch_tile<DT, 16, 256, 1, 4>(p, stream);
+        if(k.tile == 64128)
+            return launch_tile<DT, 64, 128, 2, 2>(p, stream);
+        return launch_tile<DT, 128, 128, 2, 2>(p, stream);
+    case Family::decode:
         if(!gemm_decode_supports(p))
         {
             *why = "decode_stream handles 1 <= M <= 512";
             return hipErrorInvalidValue;
         }
-        return launch_gemm_decode(p, DT, a.split_k_log2, a.device_id, stream, tuning);
-    }
-    if(strncmp(name, "mid_", 4) == 0)
-    {
-        // "mid_128x128" alone, or "mid_128x128:s=7" to pin the number of K ranges
-        const char* colon = strchr(name, ':');
-        const size_t len  = colon ? (size_t)(colon - name) : strlen(name);
-        auto is = [&](const char* s) { return strlen(s) == len && strncmp(name, s, len) == 0; };
-        const int tile = is("mid_128x128")  ? 128
-                         : is("mid_64x128") ? 64128
-                         : is("mid_64x64")  ? 64
-                         : is("mid_auto")   ? 0
-                                            : -1;
-        int splits = 0;
-        if(colon && (sscanf(colon, ":s=%d", &splits) != 1 || splits < 1 || splits > 64))
-            splits = -1;
-        if(tile < 0 || splits < 0)
-        {
-            *why = "unknown kernelName (see aiter_fp8bs_gemm_kernel_names())";
-            return hipErrorInvalidValue;
-        }
+        return launch_gemm_decode(p, DT, req.split_k_log2, ctx, k.tuning);
+    case Family::mid:
         if(!gemm_mid_supports(p))
         {
             *why = "the mid_* kernels need operand matrices below 4 GiB";
             return hipErrorInvalidValue;
         }
-        return launch_gemm_mid(p, DT, a.split_k_log2, a.device_id, stream, tile, splits);
-    }
-    if(a.split_k_log2 > 0)
-    {
-        *why = "splitK > 0 is only available with the decode_stream and mid_* kernels";
-        return hipErrorInvalidValue;
-    }
-    // "prefill_256x256" by name keeps every tile in one workgroup (bitwise the result of the
-    // tile_* kernels); "prefill_256x256:s=2" pins the number of K ranges per tile; chosen
-    // automatically, the launcher decides
-    if(strncmp(name, "prefill_256x256", 15) == 0 && (name[15] == 0 || name[15] == ':'))
-    {
-        int splits = (a.kernel_name && a.kernel_name[0]) ? 1 : 0;
-        if(name[15] == ':' && (sscanf(name + 15, ":s=%d", &splits) != 1 || splits < 1 || splits > 16))
-        {
-            *why = "unknown kernelName (see aiter_fp8bs_gemm_kernel_names())";
-            return hipErrorInvalidValue;
-        }
+        return launch_gemm_mid(p, DT, req.split_k_log2, ctx, k.tile, k.splits);
+    case Family::prefill:
         if(!gemm_prefill_supports(p))
         {
             *why = "prefill_256x256 needs N % 4 == 0 and operand matrices below 4 GiB";
             return hipErrorInvalidValue;
         }
-        return launch_gemm_prefill(p, DT, stream, splits);
+        // by name it keeps every tile in one workgroup (bitwise the result of the tile_* kernels)
+        // unless ":s=" pins the K ranges per tile; chosen automatically, the launcher decides.
+        // splitK is a hint this kernel has no use for.
+        return launch_gemm_prefill(p, DT, ctx, k.splits > 0 ? k.splits : (named ? 1 : 0));
     }
-    *why = "unknown kernelName (see aiter_fp8bs_gemm_kernel_names())";
+    *why = kUnknownName;
     return hipErrorInvalidValue;
 }
 
@@ -300,6 +360,44 @@ void gemm_describe_choice(int64_t M, int64_t N, int64_t K, bool shuffled, char* 
         snprintf(buf, n, "%s:s=%d", name, gemm_prefill_plan(p, 256).splits); // as on a 256-CU part
     else
         snprintf(buf, n, "%s", name);
+}
+
+// "<kernel>;splitK=<n>": what the pair (kernelName, splitK) of a call resolves to for contiguous
+// operands of this shape (n = -1: the kernel chooses its K ranges).  False with *why set when the
+// name is neither one of this library's nor one of the reference's zoo.
+bool gemm_describe_request(int64_t M, int64_t N, int64_t K, bool shuffled, int split_k_log2, const char* kernel_name,
+                           char* buf, size_t n, const char** why)
+{
+    GemmKernelParams p{};
+    p.M          = (int32_t)M;
+    p.N          = (int32_t)N;
+    p.K          = (int32_t)K;
+    p.lda        = K;
+    p.ldb        = K;
+    p.kblocks    = (int32_t)(K / 128);
+    p.w_shuffled = shuffled ? 1 : 0;
+    GemmArgs a{};
+    a.kernel_name        = kernel_name;
+    a.split_k_log2       = split_k_log2;
+    const KernelRequest r = resolve_request(a, p);
+    ParsedKernel        k;
+    if(!parse_kernel_name(r.name, &k))
+    {
+        *why = kUnknownName;
+        return false;
+    }
+    if(r.name != kernel_name) // chosen here: say which tiling and K ranges the choice means
+    {
+        char chosen[48];
+        gemm_describe_choice(M, N, K, shuffled, chosen, sizeof chosen);
+        if(r.split_k_log2 >= 0) // the caller's ranges replace the choice's
+            if(char* colon = strchr(chosen, ':'))
+                *colon = 0;
+        snprintf(buf, n, "%s;splitK=%d", chosen, r.split_k_log2);
+    }
+    else
+        snprintf(buf, n, "%s;splitK=%d", r.name, r.split_k_log2);
+    return true;
 }
 
 } // namespace fp8bs

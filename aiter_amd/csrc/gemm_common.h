@@ -2,6 +2,7 @@
 #pragma once
 
 #include "fp8bs_launch.h"
+#include "workspace.h"
 
 namespace fp8bs {
 
@@ -80,21 +81,15 @@ struct PrefillPlan
 };
 PrefillPlan gemm_prefill_plan(const GemmKernelParams& p, int cus);
 // want_splits: K ranges per tile; 0 lets the launcher choose, 1 keeps a tile in one workgroup
-hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, hipStream_t stream, int want_splits);
+hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, const LaunchCtx& ctx, int want_splits);
 bool       gemm_prefill_supports(const GemmKernelParams& p);
-hipError_t launch_gemm_decode(const GemmKernelParams& p, In16 out_dtype, int split_k_log2, int device_id,
-                              hipStream_t stream, const char* tuning = nullptr);
+hipError_t launch_gemm_decode(const GemmKernelParams& p, In16 out_dtype, int split_k_log2, const LaunchCtx& ctx,
+                              const char* tuning = nullptr);
 bool       gemm_decode_supports(const GemmKernelParams& p);
-hipError_t launch_gemm_mid(const GemmKernelParams& p, In16 out_dtype, int split_k_log2, int device_id,
-                           hipStream_t stream, int tile = 0, int splits = 0);
+hipError_t launch_gemm_mid(const GemmKernelParams& p, In16 out_dtype, int split_k_log2, const LaunchCtx& ctx,
+                           int tile = 0, int splits = 0);
 bool       gemm_mid_supports(const GemmKernelParams& p);
 // modelled duration (us) of the best mid_* tiling, for the choice between kernel families
 void       gemm_mid_describe(const GemmKernelParams& g, char* buf, size_t n);
 float      gemm_mid_estimate_us(const GemmKernelParams& p);
-// Per-device workspace for K split across workgroups (fp32 partial tiles + tickets that are zero
-// between launches), shared by the kernels that split K; grown on demand, kept for the life of
-// the process.  Calls that use it on one device must not overlap.
-hipError_t gemm_split_workspace(int device_id, size_t partial_bytes, size_t n_tickets, hipStream_t stream,
-                                float** partial, uint32_t** tickets);
-
 } // namespace fp8bs

@@ -18,6 +18,7 @@
 // row group (an atomic ticket) adds them in split order, so results never depend on timing.
 #include "gemm_common.h"
 
+#include <atomic>
 #include <stdlib.h>
 #include <string.h>
 
@@ -614,53 +615,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
     flush_prev();
 }
 
-// workspace for split-K partials and tickets, one per device, grown on demand and kept for the
-// life of the process.  Calls that need it on the same device must not overlap.
-struct Workspace
-{
-    float*    partial      = nullptr;
-    size_t    partial_size = 0;
-    uint32_t* tickets      = nullptr;
-    size_t    n_tickets    = 0;
-};
 constexpr int kMaxDevices = 64;
-Workspace     g_ws[kMaxDevices];
-
-hipError_t ensure_workspace(int dev, size_t partial_bytes, size_t n_tickets, hipStream_t stream,
-                            Workspace** out)
-{
-    if(dev < 0 || dev >= kMaxDevices)
-        return hipErrorInvalidDevice;
-    Workspace& w = g_ws[dev];
-    if(w.partial_size < partial_bytes)
-    {
-        if(w.partial)
-            (void)hipFree(w.partial);
-        w.partial      = nullptr;
-        w.partial_size = 0;
-        hipError_t e   = hipMalloc((void**)&w.partial, partial_bytes);
-        if(e != hipSuccess)
-            return e;
-        w.partial_size = partial_bytes;
-    }
-    if(w.n_tickets < n_tickets)
-    {
-        if(w.tickets)
-            (void)hipFree(w.tickets);
-        w.tickets    = nullptr;
-        w.n_tickets  = 0;
-        size_t     n = n_tickets < 4096 ? 4096 : n_tickets;
-        hipError_t e = hipMalloc((void**)&w.tickets, n * sizeof(uint32_t));
-        if(e != hipSuccess)
-            return e;
-        e = hipMemsetAsync(w.tickets, 0, n * sizeof(uint32_t), stream);
-        if(e != hipSuccess)
-            return e;
-        w.n_tickets = n;
-    }
-    *out = &w;
-    return hipSuccess;
-}
 
 // reads "key=value" integers out of a comma-separated tuning string; 0 when absent
 int tuning_value(const char* tuning, const char* key)
@@ -684,7 +639,7 @@ template <int MT, int R, bool SINGLE, bool FULL, bool SHUF, bool CHUNKED = false
 hipError_t launch_one(const DecodeParams& p, dim3 grid, int waves, size_t smem, hipStream_t stream)
 {
     auto        kernel = gemm_decode_kernel<MT, R, SINGLE, FULL, SHUF, CHUNKED>;
-    static bool raised[kMaxDevices]; // dynamic LDS above the default limit needs opting in, once
+    static std::atomic<bool> raised[kMaxDevices]; // dynamic LDS above the default limit needs opting in, once
     int         dev = 0;
     (void)hipGetDevice(&dev);
     if(dev >= 0 && dev < kMaxDevices && !raised[dev])
@@ -729,18 +684,6 @@ hipError_t launch_mt(const DecodeParams& p, int rows, bool single, bool full, di
 
 } // namespace
 
-hipError_t gemm_split_workspace(int device_id, size_t partial_bytes, size_t n_tickets, hipStream_t stream,
-                                float** partial, uint32_t** tickets)
-{
-    Workspace* w = nullptr;
-    hipError_t e = ensure_workspace(device_id, partial_bytes, n_tickets, stream, &w);
-    if(e != hipSuccess)
-        return e;
-    *partial = w->partial;
-    *tickets = w->tickets;
-    return hipSuccess;
-}
-
 bool gemm_decode_supports(const GemmKernelParams& p)
 {
     return p.M >= 1 && p.M <= kDecodeMaxM && p.kblocks >= 1;
@@ -748,9 +691,10 @@ bool gemm_decode_supports(const GemmKernelParams& p)
 
 // split_k_log2 < 0: choose.  Otherwise 2^split_k_log2 K ranges (rounded to whole steps).
 // `tuning` may override the choices: "r=<row tiles per group>,s=<K ranges>,w=<waves>,g=<grid.x>".
-hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int split_k_log2, int device_id,
-                              hipStream_t stream, const char* tuning)
+hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int split_k_log2, const LaunchCtx& ctx,
+                              const char* tuning)
 {
+    const hipStream_t stream = ctx.stream;
     DecodeParams p{};
     p.g           = g;
     p.bf16_out    = out_dtype == In16::bf16 ? 1 : 0;
@@ -818,18 +762,20 @@ hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int spl
         gx = p.n_groups;
 
     const size_t tile_set = (size_t)rows * mt * 64 * 16; // bytes of one group's fp32 tile set
+    WorkspaceLock lock(splits > 1);
     if(splits > 1)
     {
         const size_t bytes = (size_t)splits * p.n_groups * p.m_chunks * tile_set;
         if(bytes >= ((size_t)1 << 31))
+        {
+            if(ctx.why)
+                *ctx.why = "decode_stream: the partial tiles of this many K ranges exceed 2 GiB";
             return hipErrorInvalidValue;
-        Workspace* w = nullptr;
-        hipError_t e = ensure_workspace(device_id, bytes, (size_t)p.n_groups * p.m_chunks, stream, &w);
+        }
+        hipError_t e = split_workspace(ctx, lock, bytes, (size_t)p.n_groups * p.m_chunks, &p.partial, &p.tickets);
         if(e != hipSuccess)
             return e;
-        p.partial       = w->partial;
         p.partial_bytes = (uint32_t)bytes;
-        p.tickets       = w->tickets;
     }
 
     // LDS: a 2 KiB transposition slot per wave, then two slots of parked tile sets

@@ -19,6 +19,7 @@
 // 1 us per K block.
 #include "gemm_common.h"
 
+#include <atomic>
 #include <cstdio>
 
 namespace fp8bs {
@@ -26,6 +27,7 @@ namespace fp8bs {
 namespace {
 
 constexpr int kThreads = 256;
+constexpr size_t kMaxPartialBytes = (size_t)2 << 30; // what the arenas serve for partial tiles
 
 // s_waitcnt immediate for vmcnt(n) alone (expcnt and lgkmcnt left at their maxima)
 constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
@@ -397,7 +399,7 @@ __global__ __launch_bounds__(256) void gemm_mid_reduce_kernel(const float* __res
 }
 
 template <int BM, int BN, bool PAIR = false>
-hipError_t launch_shape(MidParams& p, int split_k_log2, int want_splits, int device_id, hipStream_t stream)
+hipError_t launch_shape(MidParams& p, int split_k_log2, int want_splits, const LaunchCtx& ctx)
 {
     using S = MidShape<BM, BN, PAIR>;
     const GemmKernelParams& g = p.g;
@@ -414,22 +416,32 @@ hipError_t launch_shape(MidParams& p, int split_k_log2, int want_splits, int dev
         splits = 1;
     if(splits > g.kblocks)
         splits = g.kblocks;
+    // The fp32 partial tiles (ranges x M x N x 4 bytes) stay within kMaxPartialBytes, and the
+    // reduction indexes quads of n with 32 bits: a larger request gets fewer ranges.
+    const size_t range_bytes = (size_t)g.M * (size_t)g.N * 4;
+    if(range_bytes / 16 >= ((size_t)1 << 32))
+        splits = 1;
+    while(splits > 1 && (size_t)splits * range_bytes > kMaxPartialBytes)
+        --splits;
     p.kb_per_split = (g.kblocks + splits - 1) / splits;
     splits         = (g.kblocks + p.kb_per_split - 1) / p.kb_per_split;
     p.splits       = splits;
 
+    const int         device_id = ctx.device_id;
+    const hipStream_t stream    = ctx.stream;
+    WorkspaceLock     lock(splits > 1); // from the request to the reduction's launch
     if(splits > 1)
     {
-        const size_t bytes = (size_t)splits * (size_t)g.M * (size_t)g.N * 4;
-        uint32_t*    unused = nullptr;
-        hipError_t   e      = gemm_split_workspace(device_id, bytes, 1, stream, &p.partial, &unused);
+        void*      partial = nullptr;
+        hipError_t e = workspace_acquire(ctx, lock, WsKind::split_partial, (size_t)splits * range_bytes, false, &partial);
         if(e != hipSuccess)
             return e;
+        p.partial = (float*)partial;
     }
 
     auto        kernel = g.w_shuffled ? gemm_mid_kernel<BM, BN, true, S::kOccupancy, PAIR>
                                       : gemm_mid_kernel<BM, BN, false, S::kOccupancy, PAIR>;
-    static bool raised[2][64]; // dynamic LDS above the default limit needs opting in, once
+    static std::atomic<bool> raised[2][64]; // dynamic LDS above the default limit needs opting in, once
     const int   which = g.w_shuffled ? 1 : 0;
     if(device_id >= 0 && device_id < 64 && !raised[which][device_id])
     {
@@ -525,8 +537,8 @@ float gemm_mid_estimate_us(const GemmKernelParams& g) { return best_plan(g, 0).c
 
 // split_k_log2 < 0: choose.  tile: 0 = choose, else 128 (128x128), 64128 (64x128) or 64 (64x64).
 // splits > 0 pins the number of K ranges (any count, not only powers of two).
-hipError_t launch_gemm_mid(const GemmKernelParams& g, In16 out_dtype, int split_k_log2, int device_id,
-                           hipStream_t stream, int tile, int splits)
+hipError_t launch_gemm_mid(const GemmKernelParams& g, In16 out_dtype, int split_k_log2, const LaunchCtx& ctx,
+                           int tile, int splits)
 {
     MidParams p{};
     p.g        = g;
@@ -555,12 +567,12 @@ hipError_t launch_gemm_mid(const GemmKernelParams& g, In16 out_dtype, int split_
     // K blocks requested in pairs (about 0.06 us per K block faster; with two workgroups per
     // compute unit the four-stage ring wins, and the 64x128 tile gains nothing from pairs)
     if(tile == 64 && ((g.M + 63) / 64) * ((g.N + 63) / 64) * splits <= 256)
-        return launch_shape<64, 64, true>(p, -1, splits, device_id, stream);
+        return launch_shape<64, 64, true>(p, -1, splits, ctx);
     switch(tile)
     {
-    case 128: return launch_shape<128, 128>(p, -1, splits, device_id, stream);
-    case 64128: return launch_shape<64, 128>(p, -1, splits, device_id, stream);
-    default: return launch_shape<64, 64>(p, -1, splits, device_id, stream);
+    case 128: return launch_shape<128, 128>(p, -1, splits, ctx);
+    case 64128: return launch_shape<64, 128>(p, -1, splits, ctx);
+    default: return launch_shape<64, 64>(p, -1, splits, ctx);
     }
 }
 

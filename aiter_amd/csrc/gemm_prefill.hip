@@ -11,6 +11,8 @@
 // Workgroups are renumbered so that the 32 tiles resident on one XCD at a time form a compact
 // 8 (m) x 4 (n) patch: each XCD's L2 then serves every operand slab to several CUs.
 #include "gemm_common.h"
+
+#include <atomic>
 #include <algorithm>
 
 namespace fp8bs {
@@ -495,8 +497,9 @@ PrefillPlan gemm_prefill_plan(const GemmKernelParams& p, int cus)
     return best;
 }
 
-hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, hipStream_t stream, int want_splits)
+hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, const LaunchCtx& ctx, int want_splits)
 {
+    const hipStream_t stream = ctx.stream;
     const int    tiles_m = (p.M + kBM - 1) / kBM, tiles_n = (p.N + kBN - 1) / kBN;
     // the two stages, or the eight waves' output blocks of the epilogue, whichever is larger
     const size_t smem    = std::max((size_t)kStages * kStageBytes, (size_t)8 * 64 * kEpiPitch);
@@ -506,8 +509,8 @@ hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, hipStr
     // Per device and instantiation, once: the opt-in to more than 64 KiB of LDS, and the number of
     // compute units.  (Racing first calls repeat the same idempotent set-up.)
     constexpr int kMaxDevices = 64;
-    static int    cus_of[kMaxDevices];
-    static bool   ready[kMaxDevices][4];
+    static std::atomic<int>  cus_of[kMaxDevices];
+    static std::atomic<bool> ready[kMaxDevices][4];
     int           device = 0, cus = 0;
     hipError_t    e = hipGetDevice(&device);
     if(e != hipSuccess)
@@ -540,10 +543,11 @@ hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, hipStr
     float*    partial = nullptr;
     uint32_t* tickets = nullptr;
     size_t    bytes   = 0;
+    WorkspaceLock lock(splits > 1);
     if(splits > 1)
     {
         bytes = (size_t)total * splits * 32 * 512 * 16;
-        if((e = gemm_split_workspace(device, bytes, (size_t)total, stream, &partial, &tickets)) != hipSuccess)
+        if((e = split_workspace(ctx, lock, bytes, (size_t)total, &partial, &tickets)) != hipSuccess)
             return e;
     }
     const int items = total * splits;

@@ -1166,43 +1166,6 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const void* __restrict
     *(u32x2*)dst = u32x2{pack2<DT>(o[0] + acc[0], o[1] + acc[1]), pack2<DT>(o[2] + acc[2], o[3] + acc[3])};
 }
 
-// per-device scratch, grown on demand and kept for the life of the process
-struct Scratch
-{
-    void*  ptr   = nullptr;
-    size_t bytes = 0;
-};
-Scratch g_scratch[64];
-
-hipError_t scratch_for(int device_id, size_t bytes, hipStream_t stream, uint8_t** out)
-{
-    if(device_id < 0 || device_id >= 64)
-        return hipErrorInvalidDevice;
-    Scratch& s = g_scratch[device_id];
-    if(s.bytes < bytes)
-    {
-        if(s.ptr)
-        {
-            // work already enqueued may still use the old buffer
-            hipError_t e = hipStreamSynchronize(stream);
-            if(e != hipSuccess)
-                return e;
-            e = hipFree(s.ptr);
-            if(e != hipSuccess)
-                return e;
-            s.ptr   = nullptr;
-            s.bytes = 0;
-        }
-        const size_t want = bytes + bytes / 4;
-        hipError_t   e    = hipMalloc(&s.ptr, want);
-        if(e != hipSuccess)
-            return e;
-        s.bytes = want;
-    }
-    *out = (uint8_t*)s.ptr;
-    return hipSuccess;
-}
-
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 // The second GEMM's rows wait in memory for the per-token sum: in fp32 while the real rows
@@ -1252,7 +1215,7 @@ hipError_t launch_topk_softmax(const TopkSoftmaxArgs& a, hipStream_t stream)
     return hipGetLastError();
 }
 
-hipError_t launch_moe_sorting(const MoeSortArgs& a, hipStream_t stream)
+hipError_t launch_moe_sorting(const MoeSortArgs& a, hipStream_t stream, const char** why)
 {
     SortParams p{};
     p.topk_ids          = a.topk_ids;
@@ -1279,11 +1242,20 @@ hipError_t launch_moe_sorting(const MoeSortArgs& a, hipStream_t stream)
     p.chunks            = (int32_t)((n + p.chunk_pairs - 1) / p.chunk_pairs);
     if(p.chunks < 1)
         p.chunks = 1;
-    uint8_t*     scratch = nullptr;
-    const size_t counts_bytes = align_up((size_t)p.chunks * a.experts * 4);
-    hipError_t   e = scratch_for(a.device_id, counts_bytes + align_up(((size_t)a.experts + 1) * 4), stream, &scratch);
+    // histograms and expert offsets: a region of their own in the stream's arena (the expert layer
+    // that follows on the same stream uses another)
+    LaunchCtx ctx;
+    ctx.device_id = a.device_id;
+    ctx.stream    = stream;
+    ctx.why       = why;
+    WorkspaceLock lock;
+    void*         block        = nullptr;
+    const size_t  counts_bytes = align_up((size_t)p.chunks * a.experts * 4);
+    hipError_t    e = workspace_acquire(ctx, lock, WsKind::moe_sort, counts_bytes + align_up(((size_t)a.experts + 1) * 4),
+                                        false, &block);
     if(e != hipSuccess)
         return e;
+    uint8_t* const scratch = (uint8_t*)block;
     p.counts       = (int32_t*)scratch;
     p.expert_begin = (int32_t*)(scratch + counts_bytes);
 
@@ -1329,14 +1301,20 @@ size_t moe_workspace_bytes(const MoeArgs& a)
     return b;
 }
 
-hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream)
+hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const char** why)
 {
     if(a.M == 0 || a.max_padded == 0)
         return hipSuccess;
-    uint8_t*   ws = nullptr;
-    hipError_t e  = scratch_for(a.device_id, moe_workspace_bytes(a), stream, &ws);
+    LaunchCtx ctx;
+    ctx.device_id = a.device_id;
+    ctx.stream    = stream;
+    ctx.why       = why;
+    WorkspaceLock lock; // until the layer's last launch is enqueued
+    void*         block = nullptr;
+    hipError_t    e     = workspace_acquire(ctx, lock, WsKind::moe_layer, moe_workspace_bytes(a), false, &block);
     if(e != hipSuccess)
         return e;
+    uint8_t* ws = (uint8_t*)block;
     const size_t slots = (size_t)a.max_padded;
     uint16_t*    h16   = (uint16_t*)ws;
     ws += align_up(slots * a.inter * 2);

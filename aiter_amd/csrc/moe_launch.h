@@ -2,6 +2,7 @@
 #pragma once
 
 #include "fp8bs_launch.h"
+#include "workspace.h"
 
 namespace fp8bs {
 
@@ -35,7 +36,8 @@ struct MoeSortArgs
     int64_t        id_stride, w_stride;
     int            device_id;
 };
-hipError_t launch_moe_sorting(const MoeSortArgs& a, hipStream_t stream);
+// *why receives a static message when scratch memory cannot be had
+hipError_t launch_moe_sorting(const MoeSortArgs& a, hipStream_t stream, const char** why);
 
 struct MoeArgs
 {
@@ -63,6 +65,6 @@ struct MoeArgs
     int64_t        lda, out_stride;
     int            device_id;
 };
-hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream);
+hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const char** why);
 
 } // namespace fp8bs

@@ -1,0 +1,65 @@
+// Scratch memory of the entry points whose kernels need more than their operands: split-K
+// partial tiles and tickets of the GEMM kernels, the intermediates of the expert layer.
+//
+// Eager calls take it from arenas: one set of blocks per (device, stream), allocated on first use
+// and grown on demand.  Work on different streams never shares a block, so calls on different
+// streams cannot touch each other's partial results.  A block that has been handed out is never
+// freed: HIP graphs captured earlier may hold its address.
+// A call whose stream is capturing allocates, clears and synchronises nothing.  It takes its
+// scratch from the device's capture arena, which every eager call keeps at least as large as its
+// own request (up to a cap per kind of buffer): after one eager run of a call, on any stream, the
+// same call can be recorded on any stream; otherwise it fails with a message.  Graphs of one
+// device therefore share scratch with each other (not with eager work): replay them one at a time.
+//
+// A WorkspaceLock must be held from the first request of a call to its last launch: it keeps two
+// host threads that use one stream from interleaving the launches of their calls.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <mutex>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace fp8bs {
+
+enum class WsKind : int
+{
+    split_partial = 0, // fp32 partial tiles of K split across workgroups
+    split_tickets,     // arrival counters, zero between launches
+    moe_sort,          // histograms and expert offsets of the sorting kernels
+    moe_layer,         // intermediates of the expert layer
+    kinds
+};
+
+// What a launcher needs to know about the call it serves besides the operands.
+struct LaunchCtx
+{
+    int          device_id     = 0;
+    hipStream_t  stream        = nullptr;
+    const char** why           = nullptr; // receives a static message when a request fails
+};
+
+class WorkspaceLock
+{
+  public:
+    explicit WorkspaceLock(bool engage = true); // engage = false: a call that needs no scratch
+    ~WorkspaceLock();
+    WorkspaceLock(const WorkspaceLock&)            = delete;
+    WorkspaceLock& operator=(const WorkspaceLock&) = delete;
+    bool engaged() const { return engaged_; }
+
+  private:
+    bool engaged_;
+};
+
+// `bytes` of scratch of one kind for work on ctx.stream, 256-byte aligned.  With `zeroed`, a
+// freshly allocated block is cleared by a fill kernel on that stream before it is handed out
+// (the kernels that use tickets leave them zero).  The caller holds a WorkspaceLock.
+hipError_t workspace_acquire(const LaunchCtx& ctx, const WorkspaceLock& held, WsKind kind, size_t bytes, bool zeroed,
+                             void** out);
+
+// Both split-K buffers at once.
+hipError_t split_workspace(const LaunchCtx& ctx, const WorkspaceLock& held, size_t partial_bytes, size_t n_tickets,
+                           float** partial, uint32_t** tickets);
+
+} // namespace fp8bs

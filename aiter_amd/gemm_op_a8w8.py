@@ -36,10 +36,12 @@ def gemm_a8w8_blockscale_ck(
     splitK: int = 0,
     kernelName: str = "",
 ) -> Tensor:
-    """aiter/ops/gemm_op_a8w8.py:285-298: writes ``Out`` and returns it.  ``splitK`` is the log2
-    of the number of K partitions (-1: the library chooses), ``kernelName`` one of
-    :func:`gemm_kernel_names` or ""."""
-    _blockscale_into(XQ, WQ, x_scale, w_scale, Out, splitK, _own_kernel_name(kernelName))
+    """aiter/ops/gemm_op_a8w8.py:285-298: writes ``Out`` and returns it.  ``kernelName`` is one of
+    :func:`gemm_kernel_names`, "" (the library chooses) or a name of the reference's own zoo as its
+    tuned tables carry them (dropped, together with the ``splitK`` tuned for it).  ``splitK`` (the
+    log2 of the number of K partitions) is a hint: honoured by the kernels that can split K, clamped
+    to what the problem allows, ignored by the others; with no name, 0 and -1 let the library choose."""
+    _blockscale_into(XQ, WQ, x_scale, w_scale, Out, splitK, kernelName or "")
     return Out
 
 
@@ -100,16 +102,8 @@ def gemm_a8w8_blockscale_bpreshuffle_ck(
 ) -> Tensor:
     """aiter/ops/gemm_op_a8w8.py:318-330: ``WQ`` holds ``shuffle_weight(w, layout=(16, 16))`` and
     ``x_scale`` is column-major; writes ``Out`` and returns it."""
-    _bpreshuffle_into(XQ, WQ, x_scale, w_scale, Out, _own_kernel_name(kernelName))
+    _bpreshuffle_into(XQ, WQ, x_scale, w_scale, Out, kernelName or "")
     return Out
-
-
-def _own_kernel_name(kernelName: Optional[str]) -> str:
-    """The reference's tuned tables name kernels of its own zoo ("a8w8_blockscale_..."): tuning
-    hints that mean nothing here and are dropped (the library then chooses).  Anything else goes to
-    the library, which knows its own names and rejects the rest."""
-    name = kernelName or ""
-    return "" if name.startswith("a8w8_blockscale_") else name
 
 
 def gemm_a8w8_blockscale_cktile(
@@ -127,9 +121,9 @@ def gemm_a8w8_blockscale_cktile(
     and x_scale, or, with ``isBpreshuffled``, shuffled weights and column-major x_scale
     (include/gemm_a8w8_blockscale_cktile_common.cuh:334-358).  One library serves both families."""
     if isBpreshuffled:
-        _bpreshuffle_into(XQ, WQ, x_scale, w_scale, Out, _own_kernel_name(kernelName))
+        _bpreshuffle_into(XQ, WQ, x_scale, w_scale, Out, kernelName or "")
     else:
-        _blockscale_into(XQ, WQ, x_scale, w_scale, Out, splitK, _own_kernel_name(kernelName))
+        _blockscale_into(XQ, WQ, x_scale, w_scale, Out, splitK, kernelName or "")
     return Out
 
 

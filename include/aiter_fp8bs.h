@@ -8,11 +8,20 @@
  * memory and keeps it alive until the stream has run the work); `Optional[Tensor]` is NULL;
  * `int` is int64_t, `bool` is int, `float` is float, `str` is const char*; the caller's HIP
  * stream is the last argument.  Functions only enqueue work on that stream and can be captured
- * into a HIP graph.  The GEMM entry points (when K is split across workgroups) and the
- * mixture-of-experts entry points keep scratch buffers that the library allocates on the first
- * call that needs a larger one (hipMalloc; a buffer being replaced is freed after a stream
- * synchronisation): run such a call once before capturing, and do not overlap calls that use
- * the scratch on one device.  Nothing else allocates or synchronises.
+ * into a HIP graph.
+ * Scratch memory: the GEMM entry points (when K is split across workgroups) and the
+ * mixture-of-experts entry points use scratch buffers that the library owns.  Eager calls take
+ * them per (device, stream), allocated (hipMalloc) on the first call on that stream that needs
+ * a larger one: calls on different streams never share scratch, and host threads may call
+ * concurrently (the launches of calls that use scratch are serialised by a lock).  A buffer that
+ * has been handed out is never freed, so graphs captured earlier stay valid.  A call whose
+ * stream is capturing allocates, clears and synchronises nothing: it uses a per-device buffer
+ * reserved for graphs, which every eager call keeps at least as large as its own need (up to
+ * 256 MiB of split-K partial tiles, 1 GiB of expert-layer intermediates).  So: run a call once
+ * eagerly, on any stream of the device, before recording it; a call recorded without that fails
+ * with a message.  Graphs of one device share that buffer with each other (never with eager
+ * work): do not replay two of them concurrently.  Nothing else allocates, and nothing
+ * synchronises.
  * Return value: 0 on success, -1 on failure with the message available from
  * aiter_get_last_error() (thread local).  No C++ exception crosses this boundary.
  *
@@ -150,9 +159,15 @@ int weight_per_128x128_quant(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
  *   Out     bf16|fp16 [M, N] contiguous
  *   Out[m,n] = round16( sum_kb  dot(XQ[m, kb], WQ[n, kb]) * x_scale[m,kb] * w_scale[n/128,kb] )
  *   with exact fp8 products, fp32 accumulation and one final rounding.  K % 128 == 0.
- *   splitK: log2 of the number of K partitions (0..4); -1 lets the library choose.
- *   kernelName: optional tile-kernel name (see aiter_fp8bs_gemm_kernel_names); "" or NULL lets
- *   the library choose.
+ *   kernelName: "" or NULL lets the library choose; one of aiter_fp8bs_gemm_kernel_names() asks
+ *   for that kernel; a name of the reference's own zoo ("a8w8_blockscale_...", as its tuned tables
+ *   carry them) is accepted and dropped together with the splitK that came with it.
+ *   splitK (-1..30, log2 of the number of K partitions in the reference) is a hint and never a
+ *   reason to fail: with no kernelName, <= 0 lets the library choose and > 0 asks the chosen
+ *   kernel for 2^splitK K ranges, clamped to what the problem allows and ignored by kernels that
+ *   keep a tile's K in one workgroup; with one of this library's names, 0 keeps K in one range.
+ *   aiter_fp8bs_gemm_resolve reports what a pair resolves to.  Results are deterministic for a
+ *   given (shape, kernelName, splitK).
  */
 int gemm_a8w8_blockscale(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t* x_scale,
                          aiter_tensor_t* w_scale, aiter_tensor_t* Out, int64_t splitK,
@@ -185,6 +200,14 @@ const char* aiter_fp8bs_gemm_kernel_names(void);
  * reference's lookup in its tuned tables, get_CKGEMM_config (aiter/ops/gemm_op_a8w8.py:448-490):
  * here the choice is a shape rule inside the library. */
 int aiter_fp8bs_gemm_choice(int64_t M, int64_t N, int64_t K, int preshuffled, char* out, int64_t out_len);
+
+/* What the pair (kernelName, splitK) of a gemm_a8w8_blockscale call resolves to for contiguous
+ * operands of shape M x N x K, written to `out` (at least 64 characters) as
+ * "<kernel>;splitK=<n>" with <kernel> in the form kernelName accepts and n = -1 when the kernel
+ * chooses its K ranges.  Host-only.  Fails (-1) for a kernelName that is neither one of this
+ * library's nor one of the reference's zoo, as the GEMM entry points do. */
+int aiter_fp8bs_gemm_resolve(int64_t M, int64_t N, int64_t K, int preshuffled, int64_t splitK, const char* kernelName,
+                             char* out, int64_t out_len);
 
 /*
  * ---- block-scale mixture of experts (gated experts, fp8 e4m3fn, 1x128 / 128x128 scales) ----
@@ -240,8 +263,7 @@ int moe_sorting_fwd(aiter_tensor_t* topk_ids, aiter_tensor_t* topk_weights, aite
  *   else: choose).
  * The product of the first GEMM is quantised 1x128 to fp8 for the second.  Each token's k
  * contributions are added in a fixed order (sorted order up to 128 tokens, slot order beyond):
- * results do not depend on timing.  Scratch memory is
- * allocated by the library on first use and grown on demand.
+ * results do not depend on timing.  Scratch memory: see the top of this file.
  */
 int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_tensor_t* gate, aiter_tensor_t* down,
                              aiter_tensor_t* sorted_token_ids, aiter_tensor_t* sorted_weights,

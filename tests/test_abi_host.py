@@ -131,7 +131,7 @@ def test_gemm_validation(lib):
     assert rc == -1 and "bf16 or fp16" in msg
     rc, msg = go(xq, wq, xs.half(), ws.half(), out)
     assert rc == -1 and "scales must be fp32" in msg
-    rc, msg = go(xq, wq, xs, ws, out, splitk=9)
+    rc, msg = go(xq, wq, xs, ws, out, splitk=31)  # the reference takes 0..30 (gemm_a8w8_blockscale.cu:82-114)
     assert rc == -1 and "splitK" in msg
     rc, msg = go(xq.view(torch.uint8), wq, xs, ws, out)
     assert rc == -1 and "same dtype" in msg  # csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale.cu:90-93
