@@ -35,6 +35,7 @@ _SIGNATURES = {
     ],
     "weight_per_128x128_quant": [_TP, _TP, _TP],
     "gemm_a8w8_blockscale": [_TP, _TP, _TP, _TP, _TP, ctypes.c_int64, ctypes.c_char_p],
+    "gemm_a8w8_blockscale_noalloc": [_TP, _TP, _TP, _TP, _TP, ctypes.c_int64, ctypes.c_char_p],
     "gemm_a8w8_blockscale_bpreshuffle": [_TP, _TP, _TP, _TP, _TP, ctypes.c_char_p],
     "topk_softmax": [_TP, _TP, _TP, _TP, ctypes.c_int],
     "moe_sorting_fwd": [_TP, _TP, _TP, _TP, _TP, _TP, _TP, ctypes.c_int64, ctypes.c_int64, _TP, _TP, ctypes.c_int64],

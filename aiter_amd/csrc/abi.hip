@@ -323,7 +323,8 @@ void rmsnorm_common(const char* fn, aiter_tensor_t* out, aiter_tensor_t* input,
 
 static int gemm_blockscale_common(const char* fn, bool preshuffled, aiter_tensor_t* XQ, aiter_tensor_t* WQ,
                                   aiter_tensor_t* x_scale, aiter_tensor_t* w_scale, aiter_tensor_t* Out,
-                                  int64_t splitK, const char* kernelName, aiter_stream_t stream)
+                                  int64_t splitK, const char* kernelName, aiter_stream_t stream,
+                                  bool static_scratch = false)
 {
     return guarded([&] {
         check_tensor(fn, XQ, "XQ");
@@ -414,6 +415,7 @@ static int gemm_blockscale_common(const char* fn, bool preshuffled, aiter_tensor
         a.device_id    = XQ->device_id;
         a.w_shuffled   = preshuffled;
         a.xs_col_major = preshuffled;
+        a.static_scratch = static_scratch;
         DeviceGuard guard(XQ->device_id);
         const char* why = nullptr;
         hipError_t  e   = fp8bs::launch_gemm_blockscale(a, (hipStream_t)stream, &why);
@@ -633,6 +635,14 @@ int gemm_a8w8_blockscale(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t*
 {
     return gemm_blockscale_common("gemm_a8w8_blockscale", false, XQ, WQ, x_scale, w_scale, Out, splitK,
                                   kernelName, stream);
+}
+
+int gemm_a8w8_blockscale_noalloc(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t* x_scale,
+                                 aiter_tensor_t* w_scale, aiter_tensor_t* Out, int64_t splitK,
+                                 const char* kernelName, aiter_stream_t stream)
+{
+    return gemm_blockscale_common("gemm_a8w8_blockscale_noalloc", false, XQ, WQ, x_scale, w_scale, Out, splitK,
+                                  kernelName, stream, true);
 }
 
 int gemm_a8w8_blockscale_bpreshuffle(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t* x_scale,

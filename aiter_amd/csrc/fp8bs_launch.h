@@ -73,6 +73,7 @@ struct GemmArgs
     int            device_id;
     bool           w_shuffled;   // wq holds shuffle_weight(w, (16,16)); needs N % 16 == 0, ldb == K
     bool           xs_col_major; // xs holds [K/128][M] instead of [M][K/128]
+    bool           static_scratch = false; // split-K scratch from the static buffer: the call allocates nothing
 };
 // Returns hipSuccess, or hipErrorInvalidValue with *why set to a static message.
 hipError_t launch_gemm_blockscale(const GemmArgs& a, hipStream_t stream, const char** why);

@@ -279,8 +279,9 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
     }
     LaunchCtx ctx;
     ctx.device_id = a.device_id;
-    ctx.stream    = stream;
-    ctx.why       = why;
+    ctx.stream      = stream;
+    ctx.why         = why;
+    ctx.static_only = a.static_scratch;
     switch(k.family)
     {
     case Family::tile:

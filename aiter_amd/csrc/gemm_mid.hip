@@ -421,7 +421,7 @@ hipError_t launch_shape(MidParams& p, int split_k_log2, int want_splits, const L
     const size_t range_bytes = (size_t)g.M * (size_t)g.N * 4;
     if(range_bytes / 16 >= ((size_t)1 << 32))
         splits = 1;
-    while(splits > 1 && (size_t)splits * range_bytes > kMaxPartialBytes)
+    while(!ctx.static_only && splits > 1 && (size_t)splits * range_bytes > kMaxPartialBytes)
         --splits;
     p.kb_per_split = (g.kblocks + splits - 1) / splits;
     splits         = (g.kblocks + p.kb_per_split - 1) / p.kb_per_split;

@@ -11,6 +11,11 @@
 // same call can be recorded on any stream; otherwise it fails with a message.  Graphs of one
 // device therefore share scratch with each other (not with eager work): replay them one at a time.
 //
+// Callers that cannot allocate at all have the static buffer instead: a fixed array in device
+// memory, one copy per GPU, shared by every call on that GPU that asks for it (LaunchCtx::
+// static_only).  It serves the split-K buffers up to kStaticPartialBytes / kStaticTickets; a
+// larger request fails.  Calls that use it and overlap on one GPU race.
+//
 // A WorkspaceLock must be held from the first request of a call to its last launch: it keeps two
 // host threads that use one stream from interleaving the launches of their calls.
 #pragma once
@@ -31,11 +36,16 @@ enum class WsKind : int
     kinds
 };
 
+// what the static buffer holds: partial tiles, then tickets
+constexpr size_t kStaticPartialBytes = (size_t)32 << 20;
+constexpr size_t kStaticTickets      = 16384;
+
 // What a launcher needs to know about the call it serves besides the operands.
 struct LaunchCtx
 {
     int          device_id     = 0;
     hipStream_t  stream        = nullptr;
+    bool         static_only   = false;   // scratch from the static buffer only: nothing is allocated
     const char** why           = nullptr; // receives a static message when a request fails
 };
 

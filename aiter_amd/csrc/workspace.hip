@@ -45,6 +45,13 @@ __global__ void __launch_bounds__(256) workspace_fill_zero_kernel(uint4* dst, si
         dst[i] = uint4{0u, 0u, 0u, 0u};
 }
 
+// The static buffer: [partial tiles | tickets].  In host code the array's name is only a handle
+// for hipGetSymbolAddress; g_static_base holds each device's own address of it.
+constexpr size_t kStaticBytes = kStaticPartialBytes + kStaticTickets * sizeof(uint32_t);
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];
+constexpr int  kMaxDevices = 64;
+unsigned char* g_static_base[kMaxDevices]; // guarded by g_mutex
+
 void say(const LaunchCtx& ctx, const char* msg)
 {
     if(ctx.why)
@@ -114,6 +121,36 @@ hipError_t block_for(const LaunchCtx& ctx, Arena& arena, int k, size_t bytes, bo
     return hipSuccess;
 }
 
+// This device's copy of the static buffer.  First use on a device (which must be current): look
+// the address up and clear the tickets with a fill kernel on the caller's stream.
+hipError_t static_base(const LaunchCtx& ctx, unsigned char** base)
+{
+    if(ctx.device_id < 0 || ctx.device_id >= kMaxDevices)
+    {
+        say(ctx, "device ordinal outside 0..63");
+        return hipErrorInvalidDevice;
+    }
+    if(g_static_base[ctx.device_id] == nullptr)
+    {
+        void*      ptr = nullptr;
+        hipError_t e   = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if(e != hipSuccess || ptr == nullptr)
+        {
+            say(ctx, "hipGetSymbolAddress of the static scratch buffer failed");
+            return e != hipSuccess ? e : hipErrorInvalidSymbol;
+        }
+        unsigned char* const tickets = (unsigned char*)ptr + kStaticPartialBytes;
+        const size_t         vecs    = kStaticTickets * sizeof(uint32_t) / 16;
+        hipLaunchKernelGGL(workspace_fill_zero_kernel, dim3((unsigned)((vecs + 255) / 256)), dim3(256), 0, ctx.stream,
+                           (uint4*)tickets, vecs);
+        if((e = hipGetLastError()) != hipSuccess)
+            return e;
+        g_static_base[ctx.device_id] = (unsigned char*)ptr;
+    }
+    *base = g_static_base[ctx.device_id];
+    return hipSuccess;
+}
+
 Arena* find_arena(int device, hipStream_t stream, bool capture)
 {
     for(Arena& a : g_arenas)
@@ -146,6 +183,30 @@ hipError_t workspace_acquire(const LaunchCtx& ctx, const WorkspaceLock& held, Ws
     *out        = nullptr;
     if(!held.engaged())
         return hipErrorInvalidValue;
+    if(ctx.static_only)
+    {
+        const bool partial = kind == WsKind::split_partial, tickets = kind == WsKind::split_tickets;
+        if(!partial && !tickets)
+        {
+            say(ctx, "this kind of scratch memory is not served from the static buffer");
+            return hipErrorInvalidValue;
+        }
+        if(bytes > (partial ? kStaticPartialBytes : kStaticTickets * sizeof(uint32_t)))
+        {
+            say(ctx, partial ? "the kernel for this problem needs more than the 32 MiB of split-K partial tiles that "
+                               "the static scratch buffer holds: use the allocating entry point, or ask for fewer K "
+                               "ranges (kernelName / splitK)"
+                             : "the kernel for this problem needs more than the 16384 split-K tickets that the static "
+                               "scratch buffer holds: use the allocating entry point");
+            return hipErrorInvalidValue;
+        }
+        unsigned char* base = nullptr;
+        hipError_t     e    = static_base(ctx, &base);
+        if(e != hipSuccess)
+            return e;
+        *out = partial ? base : base + kStaticPartialBytes;
+        return hipSuccess;
+    }
     if(bytes > kMaxBytes[k])
     {
         say(ctx, "the call needs more scratch memory than the library serves for this kind of buffer");

@@ -174,6 +174,23 @@ int gemm_a8w8_blockscale(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t*
                          const char* kernelName, aiter_stream_t stream);
 
 /*
+ * gemm_a8w8_blockscale for callers that cannot allocate device memory (code under HIP graph
+ * capture that was never run eagerly, tight serving loops, harnesses that forbid hipMalloc).  It
+ * has no counterpart in the reference.  Same operands, same kernels, same results bit for bit;
+ * the split-K scratch (fp32 partial tiles, tickets) comes from a fixed buffer in device memory
+ * that the library's code object carries: 32 MiB of partial tiles and 16384 tickets per GPU, held
+ * until the process ends.  The call allocates nothing (no hipMalloc, hipFree or allocating
+ * library routine).  A problem whose kernel needs more than the buffer holds is rejected with a
+ * message (status -1).  Every call on a GPU uses that GPU's one buffer: calls that overlap on one
+ * GPU (different streams, or a graph replay beside eager calls) race; calls on one stream are
+ * ordered and safe.  The first call on a GPU enqueues one small fill kernel (which clears the
+ * tickets) before the GEMM, on the caller's stream.
+ */
+int gemm_a8w8_blockscale_noalloc(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t* x_scale,
+                                 aiter_tensor_t* w_scale, aiter_tensor_t* Out, int64_t splitK,
+                                 const char* kernelName, aiter_stream_t stream);
+
+/*
  * The same GEMM on pre-shuffled weights.  Replaces gemm_a8w8_blockscale_bpreshuffle,
  * csrc/ck_gemm_a8w8_blockscale_bpreshuffle/gemm_a8w8_blockscale_bpreshuffle.cu:64-89 (declared
  * include/gemm_a8w8_blockscale_bpreshuffle.h:7-13, binding aiter/ops/gemm_op_a8w8.py:318-330).
