@@ -40,6 +40,25 @@ def per_1x128_quant(x: torch.Tensor, group: int = 128, quant_dtype=FP8):
     return y.view(*lead, n), s.view(*lead, n // group)
 
 
+def per_1x128_quant_device_formula(x: torch.Tensor, group: int = 128, quant_dtype=FP8):
+    """The arithmetic of the reference's HIP kernel behind the same entry point,
+    csrc/kernels/quant_kernels.cu:87-166 (with aiter_opus_plus.h:49-75 for the store): amax floored
+    at 1e-10, scale = amax * float(1/448), codes = fp8(clamp(x * (1 / scale), +-448)).  It differs
+    from :func:`per_1x128_quant` (the torch definition this build matches bit for bit) by
+    reciprocal-multiply roundings and on all-zero groups; kept so that a test can bound that
+    difference.  Bitwise parity with the reference's kernel itself is unpinned: it needs a GPU run
+    of the reference, and its 1/scale may be compiled as an approximate reciprocal."""
+    assert x.shape[-1] % group == 0
+    lead, n = x.shape[:-1], x.shape[-1]
+    xf = x.reshape(-1, group).to(torch.float32)
+    dtype_max = torch.finfo(quant_dtype).max
+    amax = torch.clamp(xf.abs().amax(dim=-1, keepdim=True), min=1e-10)
+    scale = amax * torch.tensor(1.0 / dtype_max, dtype=torch.float32)
+    inv = torch.tensor(1.0, dtype=torch.float32) / scale
+    y = torch.clamp(xf * inv, -dtype_max, dtype_max).to(quant_dtype)
+    return y.view(*lead, n), scale.view(*lead, n // group)
+
+
 def weight_per_128x128_quant(w: torch.Tensor, block=(128, 128), quant_dtype=FP8):
     """op_tests/multigpu_tests/test_dispatch_combine.py:180-204 for one [N,K] matrix.
 

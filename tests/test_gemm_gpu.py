@@ -376,7 +376,9 @@ def test_prefill_kernel_more_tiles_than_compute_units(m, n, k):
 def test_config4_full_size(layout):
     # BASELINE config 4: M=8192, N=36864, K=7168 through the library's own kernel choice.  Every
     # output is compared bit for bit with the generic tile kernel (same products, same order of
-    # additions), and 16 rows x all N with the fp64 reference on the CPU.
+    # additions), and 72 rows x all N with the fp64 reference on the CPU: two rows out of each of the
+    # 32 tiles of 256 rows, 96 rows apart (another 64-row wave quarter and the other 32-row half of
+    # it), at offsets that walk through all 16 lanes and 4 accumulator rows, plus the corners.
     m, n, k = 8192, 36864, 7168
     xq, wq, xs, ws = _gpu_problem(m, n, k, seed=4, outliers=True)
     out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
@@ -392,8 +394,12 @@ def test_config4_full_size(layout):
     torch.cuda.synchronize()
     assert torch.equal(out.view(torch.int16), tile.view(torch.int16))
     del tile
-    rows = torch.tensor([0, 1, 255, 256, 1000, 2047, 2048, 3333, 4095, 4096, 5000, 6143, 6144, 7777, 8190, 8191],
-                        device=DEV)
+    picked = {0, 1, 255, 256, 4095, 4096, 8190, 8191}
+    for t in range(m // 256):
+        r = (t * 37 + 5) % 256
+        picked |= {t * 256 + r, t * 256 + (r + 96) % 256}
+    assert len(picked) >= 64
+    rows = torch.tensor(sorted(picked), device=DEV)
     _check_rows_against_f64(out, xq, wq, xs, ws, rows, f"config 4 {layout}")
 
 

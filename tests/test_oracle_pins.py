@@ -250,3 +250,35 @@ def test_rmsnorm_closed_form_and_add():
     assert np.array_equal(out, co.rmsnorm_bf16(res_out, co.codes16(w), 1e-6))
     ref, _ = tr.rmsnorm_ref(x, w, 1e-6, residual=r)
     assert np.abs(out.astype(np.int32) - co.codes16(ref).astype(np.int32)).max() <= 1
+
+
+def test_device_kernel_formula_stays_within_one_rounding_of_the_torch_definition():
+    """The reference has two definitions of the 1x128 quant: the torch one (aiter/ops/quant.py:64-94,
+    matched here bit for bit) and its HIP kernel's (csrc/kernels/quant_kernels.cu:87-166: amax floored
+    at 1e-10, scale = amax * (1/448), multiply by 1/scale, clamp).  They may differ by one ulp in the
+    scale and by one code where a quotient sits on a rounding boundary; nothing more."""
+    x = tr.make_activation(512, 7168, seed=5, outlier_frac=0.01)
+    x[7, 256:384] = 0                      # an all-zero group
+    y_t, s_t = tr.per_1x128_quant(x)
+    y_d, s_d = tr.per_1x128_quant_device_formula(x)
+    st = s_t.numpy().view(np.uint32).astype(np.int64)
+    sd = s_d.numpy().view(np.uint32).astype(np.int64)
+    zero_group = (7, 2)
+    mask = np.ones(st.shape, dtype=bool)
+    mask[zero_group] = False
+    assert np.abs(st - sd)[mask].max() <= 1, "scales differ by more than one ulp"
+    # (about half of the scales do differ by that ulp: amax * fl(1/448) is not the rounded amax / 448)
+    assert s_t[zero_group].item() == 1.0 and abs(s_d[zero_group].item() - 1e-10 / 448) < 1e-17
+    ct = y_t.view(torch.uint8).numpy().astype(np.int32)
+    cd = y_d.view(torch.uint8).numpy().astype(np.int32)
+    assert not ct[7, 256:384].any() and not cd[7, 256:384].any()
+    differ = ct != cd
+    assert differ.mean() < 2e-3, f"{differ.mean():.2e} of the codes differ"
+    # every differing pair is a pair of neighbouring codes of the same sign ...
+    assert np.all(np.abs(ct[differ] - cd[differ]) == 1)
+    # ... and its exact quotient lies within a few fp32 roundings of the midpoint between them
+    table = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).double().numpy()
+    xq = x.double().numpy()[differ]
+    sc = np.repeat(s_t.double().numpy(), 128, axis=-1)[differ]
+    mid = (table[ct[differ]] + table[cd[differ]]) / 2
+    assert np.all(np.abs(xq / sc - mid) <= 4 * 2.0**-24 * np.abs(mid))
