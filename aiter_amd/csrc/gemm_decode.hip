@@ -97,7 +97,8 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
     // 16-row x 128-byte unit into MFMA fragments through a private 2 KiB LDS slot: written as
     // loaded, read back fragment-wise; the bank swizzle of that slot is applied on the global
     // side, by which 16-byte chunk of its row a lane fetches.
-    const int crow = lane >> 3, cchunk = (lane & 7) ^ crow;
+    const int crow = lane >> 3;
+    const int cchunk[2] = {(int)((lane & 7) ^ lds_swizzle(crow)), (int)((lane & 7) ^ lds_swizzle(8 + crow))};
     uint8_t*  slot = smem + (size_t)wave * 2048;
     auto      as_fragment = [&](const u32x4(&raw)[2]) -> i32x8 {
         return i32x8{(int)raw[0][0], (int)raw[0][1], (int)raw[0][2], (int)raw[0][3],
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
 #pragma unroll
             for(int h = 0; h < 2; ++h)
                 xrow[j][h] =
-                    g.xq + (size_t)min(m_base + j * 16 + h * 8 + crow, g.M - 1) * g.lda + cchunk * 16;
+                    g.xq + (size_t)min(m_base + j * 16 + h * 8 + crow, g.M - 1) * g.lda + cchunk[h] * 16;
             xsrow[j] = g.xs + (size_t)min(m_base + j * 16 + l16, g.M - 1) * g.xs_m;
         }
     };
@@ -164,7 +165,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                 for(int h = 0; h < 2; ++h)
                 {
                     const int      n  = min(tile * 16 + h * 8 + crow, g.N - 1);
-                    const uint8_t* wp = g.wq + (size_t)n * g.ldb + cchunk * 16;
+                    const uint8_t* wp = g.wq + (size_t)n * g.ldb + cchunk[h] * 16;
 #pragma unroll
                     for(int i = 0; i < kStepKb; ++i)
                         raw[r][i][h] = __builtin_nontemporal_load(

@@ -126,7 +126,7 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
 
     // ---- global -> LDS plan: a stage is BN/8 + BM/8 units of 1 KiB (8 rows each); wave w moves
     // units 4 i + w of either slab.  Lane p of a unit fills LDS chunk p: stage row 8 u + p/8,
-    // stored chunk p%8, which must hold the row's logical chunk (p%8) ^ ((row>>1)&7).
+    // stored chunk p%8, which must hold the row's logical chunk (p%8) ^ lds_swizzle(row).
     // Pre-shuffled weights: unit u is half of 16-row tile u/2's K block, copied as it lies.
     uint32_t goff_w[S::kWUnits], goff_x[S::kXUnits];
 #pragma unroll
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
     {
         const uint32_t u = 4u * i + wave;
         const uint32_t r = 8u * u + (lane >> 3);
-        const uint32_t c = (lane & 7u) ^ ((r >> 1) & 7u);
+        const uint32_t c = (lane & 7u) ^ lds_swizzle(r);
         if(SHUF)
         {
             uint32_t tl = ((uint32_t)n0 >> 4) + (u >> 1);
@@ -152,7 +152,7 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
     {
         const uint32_t u = 4u * i + wave;
         const uint32_t r = 8u * u + (lane >> 3);
-        const uint32_t c = (lane & 7u) ^ ((r >> 1) & 7u);
+        const uint32_t c = (lane & 7u) ^ lds_swizzle(r);
         const uint32_t m = min((uint32_t)m0 + r, (uint32_t)g.M - 1u);
         goff_x[i]        = m * (uint32_t)g.lda + c * 16u;
     }
@@ -214,7 +214,7 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
 
     // ---- LDS read offsets of this lane's fragment halves (tile rows start at multiples of 16,
     // so the swizzle term depends on l16 only)
-    const uint32_t sw      = (uint32_t)(l16 >> 1) & 7u;
+    const uint32_t sw      = lds_swizzle((uint32_t)l16);
     const uint32_t lo_off  = (uint32_t)l16 * 128u + (((2u * kg) ^ sw) << 4);
     const uint32_t hi_off  = (uint32_t)l16 * 128u + (((2u * kg + 1u) ^ sw) << 4);
     const uint32_t wlo_off = SHUF ? (uint32_t)kg * 512u + (uint32_t)l16 * 16u : lo_off;

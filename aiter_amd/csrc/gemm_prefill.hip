@@ -26,12 +26,9 @@ constexpr int kStages = 2;
 constexpr uint32_t kEpiPitch = 272; // bytes per row of a wave's 64 x 128 16-bit output block in LDS
 constexpr int kGroupN = 4; // n tiles swept together by consecutive workgroups
 
-// 16-byte chunk c of stage row r is stored at chunk c ^ ((r >> 1) & 7): the 16 rows one
-// quarter-wave reads with a ds_read_b128 then fall on 16 different 16-byte bank groups.
-__device__ __forceinline__ uint32_t swz(uint32_t row, uint32_t chunk)
-{
-    return row * 128u + ((chunk ^ ((row >> 1) & 7u)) << 4);
-}
+// 16-byte chunk c of stage row r is stored at chunk c ^ lds_swizzle(r): every group of 16 lanes
+// that the LDS serves together in a fragment read then falls on 16 different 16-byte bank groups.
+__device__ __forceinline__ uint32_t swz(uint32_t row, uint32_t chunk) { return lds_off(row, chunk); }
 
 __device__ __forceinline__ i32x8 read_frag(const uint8_t* base, uint32_t row, uint32_t kg)
 {
@@ -88,13 +85,13 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
 
     // ---- global -> LDS plan: per stage 64 units of 8 rows (1 KiB); wave w moves units i*8+w.
     // Lane p of a unit fills LDS chunk p, i.e. stage row 8u + p/8, stored chunk p%8, which must
-    // hold the row's logical chunk (p%8) ^ ((row>>1)&7).
+    // hold the row's logical chunk (p%8) ^ lds_swizzle(row).
     uint32_t goff[8];
 #pragma unroll
     for(int i = 0; i < 8; ++i)
     {
         const uint32_t r = 64u * i + 8u * wave + (lane >> 3);
-        const uint32_t c = (lane & 7u) ^ ((r >> 1) & 7u);
+        const uint32_t c = (lane & 7u) ^ lds_swizzle(r);
         if(i < 4 && SHUF)
         {
             // unit U = 8 i + wave is half of tile U/2's K block: 1 KiB, copied as it lies
@@ -151,7 +148,7 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     // ---- LDS read addresses.  A fragment is 32 bytes of one row: logical chunks 2kg and 2kg+1.
     // Tile rows start at multiples of 16, so the swizzle term depends on l16 only and every
     // tile is reached with an immediate offset from these four per-lane bases.
-    const uint32_t sw     = (uint32_t)(l16 >> 1) & 7u;
+    const uint32_t sw     = lds_swizzle((uint32_t)l16);
     const uint32_t lo_off = (uint32_t)l16 * 128u + (((2u * kg) ^ sw) << 4);
     const uint32_t hi_off = (uint32_t)l16 * 128u + (((2u * kg + 1u) ^ sw) << 4);
     const uint32_t wlo_off = SHUF ? (uint32_t)kg * 512u + (uint32_t)l16 * 16u : lo_off;
