@@ -63,10 +63,21 @@ def parse_args():
     return ap.parse_args()
 
 
-def time_steps(torch, fn, steps, warmup):
-    """Average seconds per call of fn over exactly `steps` calls, HIP events on the current stream."""
+WARM_SECONDS = 0.05  # untimed work before the side measurements (`also`, per-shape tables)
+
+
+def time_steps(torch, fn, steps, warmup, settle=False):
+    """Average seconds per call of fn over exactly `steps` calls, HIP events on the current stream.
+    `settle`: besides the `warmup` calls, keep calling for WARM_SECONDS first, so that a short
+    timed region is not measured while the clocks still ramp up from idle."""
     for _ in range(warmup):
         fn()
+    if settle:
+        torch.cuda.synchronize()
+        t_warm = time.perf_counter()
+        while time.perf_counter() - t_warm < WARM_SECONDS:
+            fn()
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
@@ -94,8 +105,14 @@ def time_launches(torch, fn, steps, warmup):
         with torch.cuda.graph(graph, stream=side):
             for _ in range(steps):
                 fn()
-        graph.replay()  # first replay: not timed
-        side.synchronize()
+        # untimed replays until the clocks have settled (a launch sequence that starts on an idle
+        # chip runs its first tens of milliseconds at lower clocks)
+        t_warm = time.perf_counter()
+        while True:
+            graph.replay()
+            side.synchronize()
+            if time.perf_counter() - t_warm > WARM_SECONDS:
+                break
         times = []
         for _ in range(5):
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -680,14 +697,14 @@ def main():
             w2 = make_workload(name)
             w2.setup(torch, dev)
             steps2 = 10 if name == "prefill" else 30
-            s2 = time_steps(torch, w2.step, steps2, 3)
+            s2 = time_steps(torch, w2.step, steps2, 3, settle=True)
             v2, u2, r2 = w2.result(s2)
             entry = {"value": v2, "unit": u2, "us_per_step": s2 * 1e6, "steps": steps2, "roofline": r2,
                      "config": w2.describe()}
             if name == "prefill":
                 entry["vs_reference_tuned_csv"] = v2 / REF_PREFILL_TFLOPS
             if name == "fused":
-                sn = time_steps(torch, w2.step_norm_only, 30, 3)
+                sn = time_steps(torch, w2.step_norm_only, 30, 3, settle=True)
                 gb = w2.norm_bytes() / sn / 1e9
                 entry["norm_quant"] = {"us": sn * 1e6, "GB/s": gb, "frac_of_hbm_peak": gb / HBM_PEAK_GBS}
             if not args.no_cpu and name in ("prefill", "fused"):
