@@ -707,11 +707,13 @@ hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int spl
     const int kChipCus  = 256;
 
     // Two row tiles per group halve the activation traffic and double what a wave keeps in
-    // flight: taken when the activations are wide (their re-reads then cost more than idle
-    // compute units) or when that still leaves a workgroup for nearly every compute unit.
+    // flight: taken when the activations are wide (from 33 rows; their re-reads then cost more
+    // than anything else).  Up to 32 rows single tiles are faster at every N measured, walked two
+    // or three to a workgroup with the next tile's weights already requested ((1, 7168, 2048):
+    // 5.8 us against 6.2, (1, 24576, 1536): 9.4 against 10.4, (32, 24576, 1536): 11.1 against 12.2).
     int rows = tuning_value(tuning, "r");
     if(rows != 1 && rows != 2)
-        rows = (mt >= 3 || p.n_tiles >= 2 * (kChipCus - kChipCus / 8)) ? 2 : 1;
+        rows = mt >= 3 ? 2 : 1;
     p.n_groups = (p.n_tiles + rows - 1) / rows;
 
     int splits = tuning_value(tuning, "s");
@@ -752,7 +754,15 @@ hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int spl
     if(gx <= 0)
     {
         gx = p.n_groups;
-        if(single && p.n_groups * splits > 2 * kChipCus)
+        if(single && rows == 1 && mt <= 2 && splits == 1 && p.n_groups >= 2 * (kChipCus - kChipCus / 8))
+        {
+            // single tiles, short K: at least two tiles per workgroup, at most two workgroups per
+            // compute unit at a time
+            int iters = (p.n_groups + 2 * kChipCus - 1) / (2 * kChipCus);
+            iters     = iters < 2 ? 2 : iters;
+            gx        = (p.n_groups + iters - 1) / iters;
+        }
+        else if(single && p.n_groups * splits > 2 * kChipCus)
         {
             const int per_split = (kChipCus + splits - 1) / splits;
             const int iters     = (p.n_groups + per_split - 1) / per_split;
