@@ -96,6 +96,7 @@ def time_launches(torch, fn, steps, warmup):
     stream it is launched on; the median of five replays is returned.  Kernels replayed back to
     back overlap one launch's tail with the next one's head, so this figure can be below the
     duration a profiler reports for the kernel alone: the fields that carry it say "replay"."""
+    torch.zeros(1, device="cuda")  # a fill kernel: cuts a kernel trace of the run into its measurements
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
