@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the FP8 block-scale path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload quant|prefill|decode|decode9|sweep|moe|fused]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload quant|prefill|decode|decode9|sweep|moe|fused|stream]
                     [--no-also] [--no-cpu]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
@@ -18,6 +18,8 @@ Workloads (BASELINE.json configs):
                      duration the reference's tuner recorded for it
   moe      (beyond the configs) block-scale expert layer of DeepSeek-V3, 1..1024 tokens
   fused    config 5  RMSNorm + 1x128 quant on [2048,7168], then GEMM N=4096
+  stream   (calibration) read-only / write-only / 2:1 mixed streaming rates of the quant kernel's
+                     access pattern without its arithmetic, on config 2's byte counts
 
 Timing uses HIP events recorded on the stream the kernels are launched on (torch's current
 stream) around exactly K launches-worth of steps, bracketed by device synchronisation.
@@ -48,7 +50,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="quant", choices=["quant", "prefill", "decode", "decode9", "sweep", "moe", "fused", "copy"],
+    ap.add_argument("--workload", default="quant", choices=["quant", "prefill", "decode", "decode9", "sweep", "moe", "fused", "copy", "stream"],
                     help="'copy' is a plain 1 GiB device copy used to calibrate the rocprofv3 FETCH_SIZE / "
                     "WRITE_SIZE counters; it is not part of the path")
     ap.add_argument("--no-also", action="store_true", help="time only the primary workload")
@@ -414,6 +416,63 @@ class CopyCalibration:
         return None
 
 
+class StreamCeilings:
+    """The quant kernel with its arithmetic taken out (aiter_fp8bs_stream_probe: same grid, same
+    32 bytes in and 16 bytes out per lane, same cache policy) on config 2's byte counts: a
+    read-only pass over the 235 MB input, a write-only pass over the 117 MB output, and the 2 : 1
+    mix of both.  The ceiling the quant kernel is held against."""
+
+    name = "stream"
+    M, K = 16384, 7168
+
+    def setup(self, torch, dev):
+        from aiter_amd import _ffi
+
+        self.call = _ffi.call
+        n = self.M * self.K
+        self.xs = [torch.randn(n, device=dev).bfloat16() for _ in range(3)]
+        self.y = torch.empty(n, dtype=torch.uint8, device=dev)
+        self.i = 0
+
+    def _next(self):
+        self.i = (self.i + 1) % len(self.xs)
+        return self.xs[self.i]
+
+    def step(self):  # the mix
+        self.call("aiter_fp8bs_stream_probe", self.y, self._next(), 2)
+
+    def step_read(self):
+        self.call("aiter_fp8bs_stream_probe", self.y, self._next(), 0)
+
+    def step_write(self):
+        self.call("aiter_fp8bs_stream_probe", self.y, self._next(), 1)
+
+    def describe(self):
+        return {"workload": "streaming ceilings for config 2's byte mix (the quant kernel without arithmetic): "
+                            "headline value is the 2:1 read/write mix; read-only and write-only ride in per_shape",
+                "kernel": "stream_probe_kernel"}
+
+    def result(self, sec):
+        by = self.M * self.K * 3
+        gbs = by / sec / 1e9
+        return gbs, "GB/s", {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": gbs / HBM_PEAK_GBS, "traffic": None}
+
+    def per_shape(self, torch, steps, warmup):
+        n = self.M * self.K
+        out = []
+        for what, fn, by in (("read-only, 2 B per element", self.step_read, 2 * n),
+                             ("write-only, 1 B per element", self.step_write, n),
+                             ("2 B read + 1 B written per element", self.step, 3 * n)):
+            sec = time_steps(torch, fn, steps, warmup, settle=True)
+            out.append({"what": what, "bytes": by, "us": sec * 1e6, "GB/s": by / sec / 1e9,
+                        "frac_of_hbm_peak": by / sec / 1e9 / HBM_PEAK_GBS})
+        return out
+
+    def cpu_baseline(self, torch):
+        return None
+
+
 class DecodeAllWorkload:
     """All nine decode shapes of config 3, one launch each per step (shape after shape, so a kernel
     trace of the run lists them in DECODE_SHAPES order)."""
@@ -619,6 +678,8 @@ def make_workload(name):
         return SweepWorkload()
     if name == "copy":
         return CopyCalibration()
+    if name == "stream":
+        return StreamCeilings()
     if name == "quant":
         return QuantWorkload()
     if name == "prefill":
@@ -679,12 +740,12 @@ def main():
     }
     if args.workload == "prefill":
         line["vs_reference_tuned_csv"] = value / REF_PREFILL_TFLOPS
-    if args.workload in ("decode9", "sweep", "moe"):
+    if args.workload in ("decode9", "sweep", "moe", "stream"):
         # shape after shape: steps + warmup launches each, in DECODE_SHAPES order
         line["per_shape"] = wl.per_shape(torch, args.steps, args.warmup)
         args.no_also = True
 
-    if not args.no_cpu and args.workload != "copy":
+    if not args.no_cpu and args.workload not in ("copy", "stream"):
         torch.set_num_threads(os.cpu_count() or 1)
         line["cpu_baseline"] = wl.cpu_baseline(torch)
 
