@@ -864,8 +864,10 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
             fail(fn, "fc2_smooth_scale is not supported");
         if(fc_scale_blkn != 128 || fc_scale_blkk != 128)
             fail(fn, "only 128 x 128 weight scale blocks are supported, got ", fc_scale_blkn, " x ", fc_scale_blkk);
-        if(block_size_M != 32)
-            fail(fn, "block_size_M must be 32, got ", block_size_M);
+        // the block size the arrays were sorted with (the reference's kernels exist for 16, 32 and 64:
+        // hsa/gfx950/fmoe/silu/fmoe_bf16_blockscaleFp8_g1u1_silu.csv, column subGU_m)
+        if(block_size_M != 16 && block_size_M != 32 && block_size_M != 64 && block_size_M != 128)
+            fail(fn, "block_size_M must be 16, 32, 64 or 128, got ", block_size_M);
         if(activation != 0 && activation != 1)
             fail(fn, "activation must be 0 (silu) or 1 (gelu), got ", activation);
         if(!is_f16_like(out->dtype_))
@@ -907,16 +909,20 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
         if(!contiguous(sorted_token_ids) || !contiguous(sorted_expert_ids) || !contiguous(sorted_weights) ||
            num_valid_ids->numel_ < 1)
             fail(fn, "the sorted arrays must be contiguous");
+        const int64_t unit       = block_size_M;
+        const int64_t block_rows = unit < 32 ? unit : 32; // rows of the blocks the kernels walk
         const int64_t max_blocks = (int64_t)sorted_expert_ids->numel_;
-        const int64_t max_padded = max_blocks * 32;
-        if((int64_t)sorted_token_ids->numel_ < max_padded - 31 || (int64_t)sorted_weights->numel_ < max_padded - 31)
+        const int64_t max_padded = max_blocks * unit;
+        if((int64_t)sorted_token_ids->numel_ < max_padded - (unit - 1) ||
+           (int64_t)sorted_weights->numel_ < max_padded - (unit - 1))
             fail(fn, "sorted_token_ids and sorted_weights must cover the ", max_blocks,
                  " blocks of sorted_expert_ids");
         // the kernels read whole blocks: the last block may only be addressed if it is backed
         const int64_t backed = (int64_t)sorted_token_ids->numel_ < (int64_t)sorted_weights->numel_
                                    ? (int64_t)sorted_token_ids->numel_
                                    : (int64_t)sorted_weights->numel_;
-        const int64_t use_blocks = backed / 32 < max_blocks ? backed / 32 : max_blocks;
+        const int64_t use_sorted = backed / unit < max_blocks ? backed / unit : max_blocks;
+        const int64_t use_blocks = use_sorted * (unit / block_rows);
         if(max_padded >= (1LL << 31) || max_padded * dim >= (1LL << 40))
             fail(fn, "problem too large");
 
@@ -975,7 +981,9 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
         a.experts           = (int32_t)E;
         a.topk              = (int32_t)topk;
         a.max_blocks        = (int32_t)use_blocks;
-        a.max_padded        = (int32_t)(use_blocks * 32);
+        a.max_padded        = (int32_t)(use_blocks * block_rows);
+        a.block_rows        = (int32_t)block_rows;
+        a.expert_shift      = unit == 128 ? 2 : unit == 64 ? 1 : 0;
         a.activation        = (int32_t)activation;
         // the reference's names pick among its tuned kernels; here "nt=1|2|4" pins the first GEMM's
         // columns per workgroup, "dw=" / "dc=" / "down=rows" pick the second GEMM that writes rows

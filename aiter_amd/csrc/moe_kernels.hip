@@ -504,6 +504,8 @@ struct MoeGemmParams
     float*         row_info;   // first GEMM only: [slots][kRowInfo] records, see below (null: not wanted)
     const float*   sorted_weights; // first GEMM only, for row_info
     int32_t        xs_stride;  // second GEMM only: floats between the scale rows of two slots
+    int32_t        block_rows;   // sorted rows a workgroup's block covers: 32, or 16 when the arrays were sorted in blocks of 16
+    int32_t        expert_shift; // such a block's entry in sorted_expert_ids is block >> expert_shift (sorting blocks of 64, 128)
     int64_t        lda;
 };
 
@@ -553,7 +555,7 @@ __device__ __forceinline__ void gate_up_body(const MoeGemmParams& p, float* red,
 #pragma unroll
     for(int j = 0; j < MT; ++j)
     {
-        const int id  = p.sorted_ids[blk * 32 + j * 16 + l16] & 0xffffff;
+        const int id  = p.sorted_ids[blk * p.block_rows + j * 16 + l16] & 0xffffff;
         const int tok = id < p.M ? id : 0; // padding rows compute on token 0 and are never read
         xrow[j]       = p.xq + (size_t)tok * p.lda;
         xsr[j]        = p.xs + tok;
@@ -626,7 +628,7 @@ __device__ __forceinline__ void gate_up_body(const MoeGemmParams& p, float* red,
 #pragma unroll
             for(int c = 0; c < 4; ++c)
                 h[c] = activate(g[c], p.activation) * u[c];
-            const int slot = blk * 32 + j * 16 + l16;
+            const int slot = blk * p.block_rows + j * 16 + l16;
             const int col  = (grp * NT + i) * 16 + kg * 4;
             *(u32x2*)(p.out + (size_t)slot * p.inter + col) =
                 u32x2{pack2<In16::bf16>(h[0], h[1]), pack2<In16::bf16>(h[2], h[3])};
@@ -639,17 +641,17 @@ __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmP
 {
     __shared__ __attribute__((aligned(16))) float red_dyn[kGateUpWaves * 2 * NT * 64 * 4];
     const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
-    if(blk * 32 >= p.num_valid[0])
+    if(blk * p.block_rows >= p.num_valid[0])
         return;
-    const int expert = p.sorted_expert_ids[blk];
+    const int expert = p.sorted_expert_ids[blk >> p.expert_shift];
     if(expert < 0 || expert >= p.experts)
         return;
     if(grp == 0 && threadIdx.x < 64) // record which rows are real pairs, and where each pair sits, for the final sum
     {
         bool real = false;
-        if(threadIdx.x < 32)
+        if((int)threadIdx.x < p.block_rows)
         {
-            const int at = blk * 32 + threadIdx.x;
+            const int at = blk * p.block_rows + threadIdx.x;
             const int id = p.sorted_ids[at], token = id & 0xffffff, slot = (id >> 24) & 0xff;
             real         = token < p.M && slot < p.topk;
             if(real && p.where)
@@ -665,7 +667,7 @@ __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmP
             p.block_mask[blk] = (uint32_t)rows;
     }
     // rows of a block are real pairs first, padding after: the second 16 rows matter only if row 16 is real
-    const bool second_half = (p.sorted_ids[blk * 32 + 16] & 0xffffff) < p.M;
+    const bool second_half = p.block_rows == 32 && (p.sorted_ids[blk * 32 + 16] & 0xffffff) < p.M;
     if(second_half)
         gate_up_body<2, NT>(p, red_dyn, blk, grp, expert);
     else
@@ -688,7 +690,7 @@ __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int g
 #pragma unroll
     for(int j = 0; j < MT; ++j)
     {
-        const size_t slot = (size_t)blk * 32 + j * 16 + l16;
+        const size_t slot = (size_t)blk * p.block_rows + j * 16 + l16;
         real[j]           = (p.sorted_ids[slot] & 0xffffff) < p.M;
 #pragma unroll
         for(int kb = 0; kb < KB; ++kb)
@@ -729,7 +731,7 @@ __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int g
                     for(int c = 0; c < 4; ++c)
                         acc[c] = __builtin_fmaf(prod[c], sc, acc[c]);
                 }
-                const size_t slot = (size_t)blk * 32 + j * 16 + l16;
+                const size_t slot = (size_t)blk * p.block_rows + j * 16 + l16;
                 const int    col  = n + kg * 4;
                 if(!real[j])
                     continue;
@@ -760,12 +762,12 @@ template <int KB>
 __global__ __launch_bounds__(512) void moe_down_kernel(MoeGemmParams p)
 {
     const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
-    if(blk * 32 >= p.num_valid[0])
+    if(blk * p.block_rows >= p.num_valid[0])
         return;
-    const int expert = p.sorted_expert_ids[blk];
+    const int expert = p.sorted_expert_ids[blk >> p.expert_shift];
     if(expert < 0 || expert >= p.experts)
         return;
-    const bool second_half = (p.sorted_ids[blk * 32 + 16] & 0xffffff) < p.M;
+    const bool second_half = p.block_rows == 32 && (p.sorted_ids[blk * 32 + 16] & 0xffffff) < p.M;
     if(second_half)
         down_body<2, KB>(p, blk, grp, expert);
     else
@@ -776,9 +778,9 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeGemmParams p)
 __global__ __launch_bounds__(256) void moe_down_long_k_kernel(MoeGemmParams p)
 {
     const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
-    if(blk * 32 >= p.num_valid[0])
+    if(blk * p.block_rows >= p.num_valid[0])
         return;
-    const int expert = p.sorted_expert_ids[blk];
+    const int expert = p.sorted_expert_ids[blk >> p.expert_shift];
     if(expert < 0 || expert >= p.experts)
         return;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
@@ -791,10 +793,12 @@ __global__ __launch_bounds__(256) void moe_down_long_k_kernel(MoeGemmParams p)
 #pragma unroll
     for(int j = 0; j < 2; ++j)
     {
-        const size_t slot = (size_t)blk * 32 + j * 16 + l16;
+        // a block of 16 rows has no second tile: it repeats the first and stores nothing
+        const bool   have = j * 16 < p.block_rows;
+        const size_t slot = (size_t)blk * p.block_rows + (have ? j * 16 : 0) + l16;
         xrow[j]           = p.xq + slot * p.lda;
         xsr[j]            = p.xs + slot * p.xs_stride;
-        real[j]           = (p.sorted_ids[slot] & 0xffffff) < p.M;
+        real[j]           = have && (p.sorted_ids[slot] & 0xffffff) < p.M;
     }
     const uint8_t* wt  = p.w + (size_t)expert * (size_t)p.N * (size_t)p.K + (size_t)(n0 >> 4) * 16 * (size_t)p.K;
     const float*   wsr = p.wsc + ((size_t)expert * (p.N / 128) + n0 / 128) * p.kblocks;
@@ -835,7 +839,7 @@ __global__ __launch_bounds__(256) void moe_down_long_k_kernel(MoeGemmParams p)
 #pragma unroll
         for(int i = 0; i < 4; ++i)
         {
-            const size_t slot = (size_t)blk * 32 + j * 16 + l16;
+            const size_t slot = (size_t)blk * p.block_rows + j * 16 + l16;
             const int    col  = n0 + i * 16 + kg * 4;
             if(!real[j])
                 continue;
@@ -869,6 +873,7 @@ struct DownColsParams
     uint16_t*       out;        // [M][N], row stride out_stride
     int64_t         out_stride;
     int32_t         M, K, N, kblocks, max_blocks, experts;
+    int32_t         block_rows, expert_shift; // as in MoeGemmParams
 };
 
 constexpr int kColsDepth     = 8;
@@ -943,7 +948,7 @@ __global__ __launch_bounds__(512) void moe_down_cols_kernel(DownColsParams p)
     if(wave == 0) // list the units in sorted order
     {
         const int nv    = p.num_valid[0];
-        int       valid = (nv + 31) / 32;
+        int       valid = (nv + p.block_rows - 1) / p.block_rows;
         valid           = valid < p.max_blocks ? valid : p.max_blocks;
         int      e[kColsMaxBlocks / 64];
         uint32_t m[kColsMaxBlocks / 64];
@@ -951,7 +956,7 @@ __global__ __launch_bounds__(512) void moe_down_cols_kernel(DownColsParams p)
         for(int c = 0; c < kColsMaxBlocks / 64; ++c)
         {
             const int b = c * 64 + lane;
-            e[c]        = b < valid ? p.sorted_expert_ids[b] : -1;
+            e[c]        = b < valid ? p.sorted_expert_ids[b >> p.expert_shift] : -1;
             m[c]        = b < valid ? p.block_mask[b] : 0u;
         }
         int            base = 0;
@@ -1006,7 +1011,7 @@ __global__ __launch_bounds__(512) void moe_down_cols_kernel(DownColsParams p)
         cols_load4(s.ws, wslane + (size_t)expert * wsexp);
         // rows that are padding read the unit's first real row instead: same cache lines, no traffic
         const int    row  = (s.mask >> l16) & 1u ? l16 : __builtin_ctz(s.mask);
-        const size_t slot = (size_t)(a >> 1) * 32 + (a & 1u) * 16 + row;
+        const size_t slot = (size_t)(a >> 1) * p.block_rows + (a & 1u) * 16 + row;
         const uint8_t* xp = p.xq + slot * (size_t)p.K + (size_t)kb * 128 + kg * 32;
         cols_load16(s.xlo, xp);
         cols_load16_at16(s.xhi, xp);
@@ -1377,6 +1382,8 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
     p.row_info          = a.inter / 128 <= 4 ? hs : nullptr;
     p.sorted_weights    = a.sorted_weights;
     p.max_blocks        = a.max_blocks;
+    p.block_rows        = a.block_rows;
+    p.expert_shift      = a.expert_shift;
     p.experts           = a.experts;
     p.activation        = a.activation;
     p.lda               = a.x16 ? a.dim : a.lda;
@@ -1430,6 +1437,8 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
         c.N                 = a.dim;
         c.kblocks           = a.inter / 128;
         c.max_blocks        = a.max_blocks;
+        c.block_rows        = a.block_rows;
+        c.expert_shift      = a.expert_shift;
         c.experts           = a.experts;
         const size_t lds    = (size_t)a.max_blocks * 16 + (size_t)kColsTiles * c.kblocks * (a.M + 16) * 64;
         const dim3   grid((unsigned)(a.dim / (16 * kColsTiles))), block((unsigned)(64 * c.kblocks * kColsTiles));

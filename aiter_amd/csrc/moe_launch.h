@@ -56,6 +56,10 @@ struct MoeArgs
     void*          out; // [M][dim] 16-bit, row stride out_stride; accumulated into
     In16           out_dtype;
     int32_t        M, dim, inter, experts, topk, max_padded, max_blocks;
+    // The kernels walk the sorted rows in blocks of block_rows (32; 16 when the arrays were sorted in
+    // blocks of 16); max_blocks and max_padded count those.  A block's expert is
+    // sorted_expert_ids[block >> expert_shift] (arrays sorted in blocks of 64 or 128: shift 1 or 2).
+    int32_t        block_rows, expert_shift;
     int32_t        activation; // 0 silu, 1 gelu
     int32_t        gate_tiles; // first GEMM: 16-column tiles per workgroup (1, 2, 4), 0 = choose
     int32_t        down_waves; // second GEMM: waves per workgroup (2, 4, 8), 0 = choose

@@ -157,8 +157,11 @@ def fused_moe(hidden_states, w1, w2, topk_weight, topk_ids, expert_mask=None, ac
     unsupported = {k: v for k, v in other.items() if not neutral(v)}
     if unsupported:
         raise NotImplementedError(f"fused_moe: unsupported options {sorted(unsupported)}")
-    if block_size_M not in (None, -1, 0, BLOCK_SIZE_M):
-        raise NotImplementedError(f"fused_moe: block_size_M must be {BLOCK_SIZE_M}")
+    # the reference's block-scale kernels exist for blocks of 16, 32 and 64 sorted rows
+    # (hsa/gfx950/fmoe/silu/fmoe_bf16_blockscaleFp8_g1u1_silu.csv); 128 is taken as well
+    block_m = BLOCK_SIZE_M if block_size_M in (None, -1, 0) else int(block_size_M)
+    if block_m not in (16, 32, 64, 128):
+        raise NotImplementedError(f"fused_moe: block_size_M must be 16, 32, 64 or 128, got {block_size_M}")
     if w1_scale is None or w2_scale is None:
         raise ValueError("fused_moe: w1_scale and w2_scale are required for per_1x128")
     tokens, dim = hidden_states.shape
@@ -170,7 +173,7 @@ def fused_moe(hidden_states, w1, w2, topk_weight, topk_ids, expert_mask=None, ac
         dtype = hidden_states.dtype if hidden_states.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
     num_experts = E if expert_mask is None else expert_mask.numel()
     sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, out = moe_sorting(
-        topk_ids, topk_weight, num_experts, dim, dtype, BLOCK_SIZE_M, expert_mask, num_local_tokens,
+        topk_ids, topk_weight, num_experts, dim, dtype, block_m, expert_mask, num_local_tokens,
         moe_sorting_dispatch_policy)
     if hidden_states.dtype in (torch.bfloat16, torch.float16):
         a1, scale_t = hidden_states, None
@@ -181,5 +184,5 @@ def fused_moe(hidden_states, w1, w2, topk_weight, topk_ids, expert_mask=None, ac
         scale_t = a1_scale.reshape(tokens, dim // 128).t().contiguous()
     fmoe_fp8_blockscale_g1u1(out, a1, w1, w2, sorted_ids, sorted_weights, sorted_expert_ids, num_valid_ids, topk,
                              scale_t, w1_scale.reshape(E, -1), w2_scale.reshape(E, -1), "", 128, 128, None,
-                             int(ActivationType(activation)), BLOCK_SIZE_M)
+                             int(ActivationType(activation)), block_m)
     return out

@@ -284,8 +284,10 @@ int moe_sorting_fwd(aiter_tensor_t* topk_ids, aiter_tensor_t* topk_weights, aite
  *          [experts, 2*inter_dim/128 * dim/128]
  *   down   fp8 [experts, dim, inter_dim], pre-shuffled likewise; fc2_scale fp32
  *          [experts, dim/128 * inter_dim/128]
- *   the four sorted arrays as moe_sorting_fwd writes them with unit_size 32
- *   activation 0 = silu, 1 = gelu; fc_scale_blkn = fc_scale_blkk = 128; block_size_M = 32;
+ *   the four sorted arrays as moe_sorting_fwd writes them with unit_size = block_size_M
+ *   activation 0 = silu, 1 = gelu; fc_scale_blkn = fc_scale_blkk = 128; block_size_M = 16, 32, 64
+ *   (the sizes the reference has kernels for: hsa/gfx950/fmoe/silu/fmoe_bf16_blockscaleFp8_g1u1_silu.csv,
+ *   column subGU_m) or 128;
  *   fc2_smooth_scale must be NULL; kernel_name names the reference's tuned kernels and is only a
  *   tuning hint here ("nt=1|2|4", "dw=2|4|8", "dc=2|4|8", "down=rows", "down=cols"; anything
  *   else: choose).

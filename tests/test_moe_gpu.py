@@ -222,6 +222,35 @@ def test_fmoe_other_shapes(tokens, dim, inter, experts, topk):
     assert_close(run_moe(p, kernel_name="down=cols"), refs, f"{tokens}x{dim}x{inter} E={experts} k={topk}, cols")
 
 
+@pytest.mark.parametrize("block", [16, 64, 128])
+@pytest.mark.parametrize("tokens,dim,inter,experts,topk", [(5, 7168, 256, 32, 8), (48, 7168, 256, 32, 8),
+                                                           (300, 512, 128, 4, 2), (40, 1024, 640, 8, 3)])
+def test_fmoe_sorted_in_other_block_sizes(block, tokens, dim, inter, experts, topk):
+    # the reference's kernels exist for arrays sorted in blocks of 16, 32 and 64 rows
+    # (hsa/gfx950/fmoe/silu/fmoe_bf16_blockscaleFp8_g1u1_silu.csv, subGU_m; its tuned table uses all three);
+    # the products are the same, so with either second GEMM the result must not depend on the block size
+    p = make_moe(tokens, dim, inter, experts, topk, seed=block + tokens)
+    w1 = aiter_amd.shuffle_weight(p["w1q"].view(torch.uint8)).view(dtypes.fp8)
+    w2 = aiter_amd.shuffle_weight(p["w2q"].view(torch.uint8)).view(dtypes.fp8)
+    a, a_scale = p["aq"].to(DEV), p["asc"].t().contiguous().to(DEV)
+    ti, tw = p["ti"].to(DEV), p["tw"].to(DEV)
+    refs = reference(p)
+    for hint in ("down=rows", "down=cols", ""):
+        outs = {}
+        for b in (32, block):
+            s_ids, s_w, s_e, nv, out = aiter_amd.moe_sorting(ti, tw, experts, dim, torch.bfloat16, block_size=b)
+            aiter_amd.fmoe_fp8_blockscale_g1u1(out, a, w1, w2, s_ids, s_w, s_e, nv, topk, a_scale, p["w1s"], p["w2s"],
+                                               hint, 128, 128, None, 0, b)
+            torch.cuda.synchronize()
+            outs[b] = out
+        assert_close(outs[block], refs, f"block {block}, {hint or 'auto'}")
+        if hint == "down=rows":  # per token the k rows are added in slot order whatever the sorting
+            assert torch.equal(outs[block].view(torch.int16), outs[32].view(torch.int16)), f"block {block}"
+    out = aiter_amd.fused_moe(p["x"], w1, w2, tw, ti, w1_scale=p["w1s"], w2_scale=p["w2s"], block_size_M=block)
+    torch.cuda.synchronize()
+    assert_close(out, refs, f"fused_moe, block {block}")
+
+
 def test_fmoe_both_second_gemms_on_the_reference_shape():
     p = make_moe(48, 7168, 256, 32, 8, seed=3)
     refs = reference(p)
@@ -362,7 +391,7 @@ def test_fmoe_rejects_what_it_cannot_do():
     with pytest.raises(RuntimeError, match="128 x 128"):
         aiter_amd.fmoe_fp8_blockscale_g1u1(*args, "", 64, 128)
     with pytest.raises(RuntimeError, match="block_size_M"):
-        aiter_amd.fmoe_fp8_blockscale_g1u1(*args, "", 128, 128, None, 0, 64)
+        aiter_amd.fmoe_fp8_blockscale_g1u1(*args, "", 128, 128, None, 0, 48)
     with pytest.raises(RuntimeError, match="fc2_smooth_scale"):
         aiter_amd.fmoe_fp8_blockscale_g1u1(*args, "", 128, 128, torch.ones(4, device=DEV))
     with pytest.raises(RuntimeError, match="input_scale"):
