@@ -179,7 +179,7 @@ def test_moe_validation(lib):
     assert rc == -1 and "gate must be [experts, 2*inter_dim, dim]" in msg
     rc, msg = fmoe(blkn=64)
     assert rc == -1 and "128 x 128" in msg
-    rc, msg = fmoe(block_m=16)
+    rc, msg = fmoe(block_m=48)
     assert rc == -1 and "block_size_M" in msg
     rc, msg = fmoe(act=7)
     assert rc == -1 and "activation" in msg
