@@ -38,6 +38,8 @@ _SIGNATURES = {
     "gemm_a8w8_blockscale": [_TP, _TP, _TP, _TP, _TP, ctypes.c_int64, ctypes.c_char_p],
     "gemm_a8w8_blockscale_noalloc": [_TP, _TP, _TP, _TP, _TP, ctypes.c_int64, ctypes.c_char_p],
     "gemm_a8w8_blockscale_bpreshuffle": [_TP, _TP, _TP, _TP, _TP, ctypes.c_char_p],
+    "gemm_a8w8_blockscale_bpreshuffle_asm": [_TP, _TP, _TP, _TP, _TP, _TP, ctypes.c_int, ctypes.c_char_p, ctypes.c_int,
+                                             _TP],
     "topk_softmax": [_TP, _TP, _TP, _TP, ctypes.c_int],
     "moe_sorting_fwd": [_TP, _TP, _TP, _TP, _TP, _TP, _TP, ctypes.c_int64, ctypes.c_int64, _TP, _TP, ctypes.c_int64],
     "fmoe_fp8_blockscale_g1u1": [

@@ -324,7 +324,7 @@ void rmsnorm_common(const char* fn, aiter_tensor_t* out, aiter_tensor_t* input,
 static int gemm_blockscale_common(const char* fn, bool preshuffled, aiter_tensor_t* XQ, aiter_tensor_t* WQ,
                                   aiter_tensor_t* x_scale, aiter_tensor_t* w_scale, aiter_tensor_t* Out,
                                   int64_t splitK, const char* kernelName, aiter_stream_t stream,
-                                  bool static_scratch = false)
+                                  bool static_scratch = false, aiter_tensor_t* bias = nullptr)
 {
     return guarded([&] {
         check_tensor(fn, XQ, "XQ");
@@ -395,6 +395,17 @@ static int gemm_blockscale_common(const char* fn, bool preshuffled, aiter_tensor
         // csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale.cu:82-114 takes 0..30 (KBatch = 1 << splitK)
         if(splitK < -1 || splitK > 30)
             fail(fn, "splitK = ", splitK, " outside -1..30");
+        if(bias)
+        {
+            check_tensor(fn, bias, "bias");
+            same_device(fn, {XQ, bias});
+            if(bias->dtype_ != AITER_DTYPE_fp32 || (int64_t)bias->numel_ != N || !contiguous(bias))
+                fail(fn, "bias must be a contiguous fp32 tensor of N = ", N, " elements, got ", bias->numel_, " of ",
+                     dtype_name(bias->dtype_));
+            if(N % 4 != 0)
+                fail(fn, "a bias needs N % 4 == 0, got N = ", N);
+            check_aligned(fn, bias, "bias", 16);
+        }
         if(M == 0 || N == 0)
             return;
 
@@ -420,6 +431,9 @@ static int gemm_blockscale_common(const char* fn, bool preshuffled, aiter_tensor
         const char* why = nullptr;
         hipError_t  e   = fp8bs::launch_gemm_blockscale(a, (hipStream_t)stream, &why);
         check_hip(fn, e, why);
+        if(bias)
+            check_hip(fn, fp8bs::launch_gemm_bias_add(Out->ptr, a.out_dtype, (const float*)bias->ptr, M, N,
+                                                      (hipStream_t)stream), nullptr);
     });
 }
 
@@ -673,6 +687,24 @@ int gemm_a8w8_blockscale_bpreshuffle(aiter_tensor_t* XQ, aiter_tensor_t* WQ, ait
 {
     return gemm_blockscale_common("gemm_a8w8_blockscale_bpreshuffle", true, XQ, WQ, x_scale, w_scale, Out,
                                   -1, kernelName, stream);
+}
+
+int gemm_a8w8_blockscale_bpreshuffle_asm(aiter_tensor_t* A, aiter_tensor_t* B, aiter_tensor_t* out,
+                                         aiter_tensor_t* A_scale, aiter_tensor_t* B_scale, aiter_tensor_t* bias,
+                                         int splitK, const char* kernelName, int bpreshuffle,
+                                         aiter_tensor_t* zero_bias_buf, aiter_stream_t stream)
+{
+    (void)zero_bias_buf; // the reference's kernel always reads a bias and wants zeros when there is none
+    if(!bpreshuffle)
+        return guarded([&] {
+            fail("gemm_a8w8_blockscale_bpreshuffle_asm",
+                 "bpreshuffle = 0 is not supported: row-major weights go through gemm_a8w8_blockscale");
+        });
+    // splitK and kernelName tune the reference's kernel: the name is foreign here and dropped with its split
+    (void)splitK;
+    (void)kernelName;
+    return gemm_blockscale_common("gemm_a8w8_blockscale_bpreshuffle_asm", true, A, B, A_scale, B_scale, out, -1,
+                                  nullptr, stream, false, bias);
 }
 
 // ---- mixture of experts -------------------------------------------------------------------

@@ -81,6 +81,8 @@ struct GemmArgs
 };
 // Returns hipSuccess, or hipErrorInvalidValue with *why set to a static message.
 hipError_t launch_gemm_blockscale(const GemmArgs& a, hipStream_t stream, const char** why);
+// out[m][n] += bias[n] on a stored, contiguous [M][N] result of 16-bit values (N a multiple of 4)
+hipError_t launch_gemm_bias_add(void* out, In16 dtype, const float* bias, int64_t M, int64_t N, hipStream_t stream);
 const char* gemm_kernel_names();
 // the kernel (and, for the mid_* family, K range count) taken for contiguous operands of this shape when none is named
 void gemm_describe_choice(int64_t M, int64_t N, int64_t K, bool shuffled, char* buf, size_t n);

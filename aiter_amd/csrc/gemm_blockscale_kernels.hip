@@ -401,4 +401,47 @@ bool gemm_describe_request(int64_t M, int64_t N, int64_t K, bool shuffled, int s
     return true;
 }
 
+
+namespace {
+// out[m][n] = round16(float(out[m][n]) + bias[n]), four columns per thread
+template <In16 DT>
+__global__ __launch_bounds__(256) void gemm_bias_add_kernel(uint16_t* __restrict__ out, const float* __restrict__ bias,
+                                                            int64_t quads, int32_t quads_per_row)
+{
+    const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if(q >= quads)
+        return;
+    const int   n = (int)(q % quads_per_row) * 4;
+    const u32x2 v = *(const u32x2*)(out + q * 4);
+    const f32x4 b = *(const f32x4*)(bias + n);
+    float       f[4];
+#pragma unroll
+    for(int c = 0; c < 4; ++c)
+    {
+        const unsigned short h = (unsigned short)((v[c >> 1] >> (16 * (c & 1))) & 0xffffu);
+        if constexpr(DT == In16::bf16)
+            f[c] = __uint_as_float((uint32_t)h << 16) + b[c];
+        else
+            f[c] = (float)__builtin_bit_cast(_Float16, h) + b[c];
+    }
+    *(u32x2*)(out + q * 4) = u32x2{pack2<DT>(f[0], f[1]), pack2<DT>(f[2], f[3])};
+}
+} // namespace
+
+// Adds a per-column fp32 bias onto a stored [M][N] result (N a multiple of 4, rows contiguous).
+hipError_t launch_gemm_bias_add(void* out, In16 dtype, const float* bias, int64_t M, int64_t N, hipStream_t stream)
+{
+    const int64_t quads = M * N / 4;
+    if(quads == 0)
+        return hipSuccess;
+    const dim3 grid((unsigned)((quads + 255) / 256));
+    if(dtype == In16::bf16)
+        hipLaunchKernelGGL(gemm_bias_add_kernel<In16::bf16>, grid, dim3(256), 0, stream, (uint16_t*)out, bias, quads,
+                           (int32_t)(N / 4));
+    else
+        hipLaunchKernelGGL(gemm_bias_add_kernel<In16::fp16>, grid, dim3(256), 0, stream, (uint16_t*)out, bias, quads,
+                           (int32_t)(N / 4));
+    return hipGetLastError();
+}
+
 } // namespace fp8bs

@@ -155,12 +155,12 @@ def gemm_a8w8_blockscale_bpreshuffle_asm(
     """aiter/ops/gemm_op_a8w8.py:404-430: the reference's hand-scheduled kernel for the same
     operands as :func:`gemm_a8w8_blockscale_bpreshuffle_ck` (argument order differs: ``out``
     third).  ``splitK`` and the reference's kernel names are tuning hints of that kernel and are
-    not interpreted; a bias is not supported."""
-    if bias is not None:
-        raise NotImplementedError("gemm_a8w8_blockscale_bpreshuffle_asm: bias is not part of this library")
+    not interpreted.  ``bias`` (fp32 [N] or [1, N]) is added onto the stored result by a second
+    launch: ``out = round(float(round(acc)) + bias)``."""
     if not bpreshuffle:
         raise NotImplementedError("gemm_a8w8_blockscale_bpreshuffle_asm: only pre-shuffled weights (bpreshuffle=True)")
-    _bpreshuffle_into(A, B, A_scale, B_scale, out, "")
+    _ffi.call("gemm_a8w8_blockscale_bpreshuffle_asm", A, B, out, A_scale, B_scale, bias,
+              -1 if splitK is None else int(splitK), kernelName or "", 1, None)
     return out
 
 

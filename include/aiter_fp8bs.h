@@ -217,6 +217,22 @@ int gemm_a8w8_blockscale_bpreshuffle(aiter_tensor_t* XQ, aiter_tensor_t* WQ, ait
                                      aiter_tensor_t* w_scale, aiter_tensor_t* Out,
                                      const char* kernelName, aiter_stream_t stream);
 
+/*
+ * The entry point of the reference's hand-scheduled gfx950 kernel for the same operands.  Replaces
+ * gemm_a8w8_blockscale_bpreshuffle_asm, csrc/py_itfs_cu/asm_a8w8_blockscale_bpreshuffle.cu:253-266
+ * (binding aiter/ops/gemm_op_a8w8.py:371-430; note the argument order: out third).
+ *   A, B, A_scale, B_scale, out: XQ, WQ, x_scale, w_scale, Out of gemm_a8w8_blockscale_bpreshuffle,
+ *           without that kernel's M >= 16, K >= 512, bf16 limits.
+ *   bias    optional fp32 [N] or [1, N]: out[m][n] = round16(float(round16(acc[m][n])) + bias[n]),
+ *           added by a second launch onto the stored result (two roundings; N % 4 == 0).
+ *   splitK, kernelName: tuning of the reference's kernel, not interpreted.  bpreshuffle must be
+ *           non-zero.  zero_bias_buf (the zeros that kernel reads when there is no bias) is ignored.
+ */
+int gemm_a8w8_blockscale_bpreshuffle_asm(aiter_tensor_t* A, aiter_tensor_t* B, aiter_tensor_t* out,
+                                         aiter_tensor_t* A_scale, aiter_tensor_t* B_scale, aiter_tensor_t* bias,
+                                         int splitK, const char* kernelName, int bpreshuffle,
+                                         aiter_tensor_t* zero_bias_buf, aiter_stream_t stream);
+
 /* Comma-separated list of the tile kernels gemm_a8w8_blockscale can be asked for by name
  * (the counterpart of the reference's generated kernel zoo,
  * csrc/ck_gemm_a8w8_blockscale/gemm_a8w8_blockscale_instance.py:73-117). */

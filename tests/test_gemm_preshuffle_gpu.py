@@ -98,3 +98,41 @@ def test_rejects_what_the_layout_cannot_express():
     bad = torch.empty(4, 3, device=DEV)  # wrong number of scales
     with pytest.raises(RuntimeError, match="column-major"):
         aiter_amd.gemm_a8w8_blockscale_bpreshuffle(xq.to(DEV), wq.to(DEV), bad, ws.to(DEV))
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 7168, 2048), (16, 2112, 7168), (64, 512, 512), (300, 1008, 384), (1024, 2112, 512)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_asm_spelling_with_and_without_bias(m, n, k, dtype):
+    # aiter/ops/gemm_op_a8w8.py:404-430 (csrc/py_itfs_cu/asm_a8w8_blockscale_bpreshuffle.cu:253-266): same
+    # operands, out third, optional fp32 bias per column; splitK and the reference's kernel names are its
+    # own kernel's tuning and must not change anything here
+    xq, wq, xs, ws = make_problem(m, n, k, seed=m + n + k, outliers=0.01)
+    wsh = aiter_amd.shuffle_weight(wq.view(torch.uint8)).view(wq.dtype).to(DEV)
+    a, b_scale = xq.to(DEV), ws.to(DEV)
+    a_scale = col_major(xs.to(DEV), "view")
+    base = aiter_amd.gemm_a8w8_blockscale_bpreshuffle(a, wsh, a_scale, b_scale, dtype=dtype)
+    out = torch.full((m, n), 3.0, dtype=dtype, device=DEV)
+    ret = aiter_amd.gemm_a8w8_blockscale_bpreshuffle_asm(a, wsh, out, a_scale, b_scale, splitK=2,
+                                                         kernelName="_ZN5aiter42f8_block_scale_mi350_x128_splitk")
+    assert ret.data_ptr() == out.data_ptr()
+    assert torch.equal(out.view(torch.int16), base.view(torch.int16))
+    g = torch.Generator().manual_seed(7)
+    for shape in ((n,), (1, n)):
+        bias = torch.randn(shape, generator=g).to(DEV)
+        aiter_amd.gemm_a8w8_blockscale_bpreshuffle_asm(a, wsh, out, a_scale, b_scale, bias=bias)
+        torch.cuda.synchronize()
+        # the definition: the stored result, widened, plus the bias, rounded once more
+        want = (base.float() + bias.reshape(1, n)).to(dtype)
+        assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+        # and against the exact sum: the stored product was already rounded, so the bound follows the
+        # product's magnitude, not the (possibly cancelled) sum's
+        product, b64 = tr.gemm_a8w8_blockscale_ref_f64(xq, wq, xs, ws), bias.reshape(1, n).double().cpu()
+        err = (out.double().cpu() - (product + b64)).abs()
+        assert (err <= 1e-2 + 1e-2 * (product.abs() + b64.abs())).all(), f"{m}x{n}x{k}: max error {err.max().item():.3e}"
+    with pytest.raises(RuntimeError, match="bias"):
+        aiter_amd.gemm_a8w8_blockscale_bpreshuffle_asm(a, wsh, out, a_scale, b_scale, bias=torch.zeros(n + 4, device=DEV))
+    with pytest.raises(RuntimeError, match="bias"):
+        aiter_amd.gemm_a8w8_blockscale_bpreshuffle_asm(a, wsh, out, a_scale, b_scale,
+                                                       bias=torch.zeros(n, device=DEV, dtype=torch.bfloat16))
+    with pytest.raises(NotImplementedError):
+        aiter_amd.gemm_a8w8_blockscale_bpreshuffle_asm(a, wsh, out, a_scale, b_scale, bpreshuffle=False)
