@@ -161,7 +161,8 @@ static hipError_t launch_tile(const GemmKernelParams& p, hipStream_t stream)
 }
 
 static const char* const kKernelNames =
-    "tile_16x256,tile_64x128,tile_128x128,mid_64x64,mid_64x128,mid_128x128,prefill_256x256,decode_stream";
+    "tile_16x256,tile_64x128,tile_128x128,mid_64x64,mid_64x128,mid_128x128,prefill_256x256,prefill_256x128,"
+    "decode_stream";
 
 const char* gemm_kernel_names() { return kKernelNames; }
 
@@ -180,7 +181,7 @@ static const char* automatic_choice(const GemmKernelParams& p)
     if(gemm_mid_supports(p) && (!gemm_prefill_supports(p) || gemm_mid_estimate_us(p) * 1.03f < prefill_us))
         return "mid_auto";
     if(gemm_prefill_supports(p))
-        return "prefill_256x256";
+        return gemm_prefill_plan(p, 256).tile_n == 128 ? "prefill_256x128" : "prefill_256x256";
     return "tile_128x128";
 }
 
@@ -222,7 +223,7 @@ struct ParsedKernel
 {
     Family      family;
     int         tile;   // tile: 16256 / 64128 / 128128; mid: 0 (choose) / 64 / 64128 / 128
-    int         splits; // ":s=<n>" of mid_* and prefill_256x256, 0 when absent
+    int         splits; // ":s=<n>" of mid_* and prefill_*, 0 when absent
     const char* tuning; // what follows "decode_stream:", or null
 };
 static const char* const kUnknownName = "unknown kernelName (see aiter_fp8bs_gemm_kernel_names())";
@@ -254,10 +255,11 @@ static bool parse_kernel_name(const char* name, ParsedKernel* out)
             return false;
         return out->tile >= 0;
     }
-    // "prefill_256x256", or "prefill_256x256:s=2" to pin the number of K ranges per tile
-    if(is("prefill_256x256"))
+    // "prefill_256x256" / "prefill_256x128", or "prefill_256x256:s=2" to pin the number of K ranges per tile
+    if(is("prefill_256x256") || is("prefill_256x128"))
     {
         out->family = Family::prefill;
+        out->tile   = is("prefill_256x128") ? 128 : 256;
         if(colon && (sscanf(colon, ":s=%d", &out->splits) != 1 || out->splits < 1 || out->splits > 16))
             return false;
         return true;
@@ -308,13 +310,13 @@ static hipError_t dispatch(const GemmArgs& a, const GemmKernelParams& p, hipStre
     case Family::prefill:
         if(!gemm_prefill_supports(p))
         {
-            *why = "prefill_256x256 needs N % 4 == 0 and operand matrices below 4 GiB";
+            *why = "the prefill_* kernels need N % 4 == 0 and operand matrices below 4 GiB";
             return hipErrorInvalidValue;
         }
         // by name it keeps every tile in one workgroup (bitwise the result of the tile_* kernels)
         // unless ":s=" pins the K ranges per tile; chosen automatically, the launcher decides.
         // splitK is a hint this kernel has no use for.
-        return launch_gemm_prefill(p, DT, ctx, k.splits > 0 ? k.splits : (named ? 1 : 0));
+        return launch_gemm_prefill(p, DT, ctx, k.splits > 0 ? k.splits : (named ? 1 : 0), named ? k.tile : 0);
     }
     *why = kUnknownName;
     return hipErrorInvalidValue;
@@ -357,7 +359,7 @@ void gemm_describe_choice(int64_t M, int64_t N, int64_t K, bool shuffled, char* 
     const char* name = automatic_choice(p);
     if(strcmp(name, "mid_auto") == 0)
         gemm_mid_describe(p, buf, n);
-    else if(strcmp(name, "prefill_256x256") == 0 && gemm_prefill_plan(p, 256).splits > 1)
+    else if(strncmp(name, "prefill_", 8) == 0 && gemm_prefill_plan(p, 256).splits > 1)
         snprintf(buf, n, "%s:s=%d", name, gemm_prefill_plan(p, 256).splits); // as on a 256-CU part
     else
         snprintf(buf, n, "%s", name);

@@ -19,12 +19,15 @@ namespace fp8bs {
 
 namespace {
 
-constexpr int kBM = 256, kBN = 256, kThreads = 512;
-constexpr int kSlabBytes  = (kBM + kBN) * 128; // 64 KiB: 256 weight rows then 256 activation rows
-constexpr int kStageBytes = kSlabBytes + kBM * 4; // + this K block's x_scale for the 256 rows
+constexpr int kBM = 256, kThreads = 512;
 constexpr int kStages = 2;
-constexpr uint32_t kEpiPitch = 272; // bytes per row of a wave's 64 x 128 16-bit output block in LDS
 constexpr int kGroupN = 4; // n tiles swept together by consecutive workgroups
+// The tile is 256 (m) x NW * 32 (n): NW = 8 weight fragments per wave for the 256 x 256 tile, 4 for the
+// 256 x 128 one (twice the workgroups where the wide tiles leave compute units idle).
+constexpr int tile_n(int nw) { return nw * 32; }
+constexpr int slab_bytes(int nw) { return (kBM + tile_n(nw)) * 128; } // weight rows, then 256 activation rows
+constexpr int stage_bytes(int nw) { return slab_bytes(nw) + kBM * 4; } // + this K block's x_scale for the 256 rows
+constexpr uint32_t epi_pitch(int nw) { return (uint32_t)nw * 32u + 16u; } // bytes per row of a wave's 64 x NW*16 output block in LDS
 
 // 16-byte chunk c of stage row r is stored at chunk c ^ lds_swizzle(r): every group of 16 lanes
 // that the LDS serves together in a fragment read then falls on 16 different 16-byte bank groups.
@@ -40,7 +43,7 @@ __device__ __forceinline__ i32x8 read_frag(const uint8_t* base, uint32_t row, ui
 // SHUF: weights pre-shuffled (16,16).  A 16-row tile's K block is then 2 KiB of contiguous global
 // memory already in fragment order; the weight slab in LDS is a straight copy of it (tile after
 // tile), and a lane's fragment halves sit at kg*512 + l16*16 and 256 bytes further.
-template <In16 DT, bool SHUF>
+template <In16 DT, bool SHUF, int NW>
 __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams p, int tiles_m,
                                                                 int tiles_n, int splits,
                                                                 int kb_per_split, float* partial,
@@ -48,6 +51,10 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
                                                                 uint32_t* tickets)
 {
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    constexpr int      kBN = tile_n(NW), kSlabBytes = slab_bytes(NW), kStageBytes = stage_bytes(NW);
+    constexpr uint32_t kEpiPitch = epi_pitch(NW);
+    constexpr int      kLoads    = (kBM + kBN) / 64; // slab loads per wave and stage: 8 rows each, weights first
+    constexpr int      kWLoads   = kBN / 64;
 
     typedef const volatile i32x4 __attribute__((address_space(3)))* lds_vec_ptr;
     typedef uint8_t __attribute__((address_space(3)))*              lds_byte_ptr;
@@ -70,7 +77,7 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     asm volatile("" : "+v"(t));
     const int lane = t & 63, wave = t >> 6;
     const int l16 = lane & 15, kg = lane >> 4;
-    const int wn = wave & 1, wm = wave >> 1; // n half (128 rows), m quarter (64 rows)
+    const int wn = wave & 1, wm = wave >> 1; // n half (NW * 16 rows), m quarter (64 rows)
 
     // ---- tile choice: XCD-aware renumbering, then n-groups swept m-fastest
     int       v     = tile;
@@ -83,16 +90,16 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     const int tn     = group * kGroupN + (within - tm * gn);
     const int m0 = tm * kBM, n0 = tn * kBN;
 
-    // ---- global -> LDS plan: per stage 64 units of 8 rows (1 KiB); wave w moves units i*8+w.
+    // ---- global -> LDS plan: per stage 8 * kLoads units of 8 rows (1 KiB); wave w moves units i*8+w.
     // Lane p of a unit fills LDS chunk p, i.e. stage row 8u + p/8, stored chunk p%8, which must
     // hold the row's logical chunk (p%8) ^ lds_swizzle(row).
-    uint32_t goff[8];
+    uint32_t goff[kLoads];
 #pragma unroll
-    for(int i = 0; i < 8; ++i)
+    for(int i = 0; i < kLoads; ++i)
     {
         const uint32_t r = 64u * i + 8u * wave + (lane >> 3);
         const uint32_t c = (lane & 7u) ^ lds_swizzle(r);
-        if(i < 4 && SHUF)
+        if(i < kWLoads && SHUF)
         {
             // unit U = 8 i + wave is half of tile U/2's K block: 1 KiB, copied as it lies
             const uint32_t U    = 8u * i + wave;
@@ -100,7 +107,7 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
             tile                = min(tile, ((uint32_t)p.N >> 4) - 1u);
             goff[i]             = tile * 16u * (uint32_t)p.K + (U & 1u) * 1024u + (uint32_t)lane * 16u;
         }
-        else if(i < 4)
+        else if(i < kWLoads)
         {
             uint32_t n = n0 + r;
             n          = n < (uint32_t)p.N ? n : (uint32_t)p.N - 1;
@@ -108,7 +115,7 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         }
         else
         {
-            uint32_t m = m0 + (r - 256u);
+            uint32_t m = m0 + (r - (uint32_t)kBN);
             m          = m < (uint32_t)p.M ? m : (uint32_t)p.M - 1;
             goff[i]    = m * (uint32_t)p.lda + c * 16u;
         }
@@ -141,7 +148,7 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     }
 
     // ---- scales: x_scale comes through LDS with each stage, w_scale: one block per wave
-    uint32_t nb = (uint32_t)(n0 + wn * 128) >> 7;
+    uint32_t nb = (uint32_t)(n0 + wn * (NW * 16)) >> 7;
     nb          = min(nb, (uint32_t)((p.N + 127) / 128 - 1));
     const float* ws_row = p.ws + (size_t)nb * p.kblocks;
 
@@ -153,12 +160,12 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     const uint32_t hi_off = (uint32_t)l16 * 128u + (((2u * kg + 1u) ^ sw) << 4);
     const uint32_t wlo_off = SHUF ? (uint32_t)kg * 512u + (uint32_t)l16 * 16u : lo_off;
     const uint32_t whi_off = SHUF ? wlo_off + 256u : hi_off;
-    const uint32_t w_base = (uint32_t)wn * (128u * 128u);
+    const uint32_t w_base = (uint32_t)wn * ((uint32_t)(NW * 16) * 128u);
     const uint32_t x_base = (uint32_t)kBN * 128u + (uint32_t)wm * (64u * 128u);
 
-    float acc[8][4][4];
+    float acc[NW][4][4];
 #pragma unroll
-    for(int i = 0; i < 8; ++i)
+    for(int i = 0; i < NW; ++i)
 #pragma unroll
         for(int j = 0; j < 4; ++j)
 #pragma unroll
@@ -211,9 +218,9 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     {
         const uint32_t dst0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(smem3 + wave * 1024));
 #pragma unroll
-        for(int i = 0; i < 8; ++i)
+        for(int i = 0; i < kLoads; ++i)
             dma16(dst0 + i * 8192, goff[i],
-                  i < 4 ? p.wq + (size_t)kb_lo * (SHUF ? 2048 : 128) : p.xq + (size_t)kb_lo * 128);
+                  i < kWLoads ? p.wq + (size_t)kb_lo * (SHUF ? 2048 : 128) : p.xq + (size_t)kb_lo * 128);
         if(wave < 4)
             dma4(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(smem3 + kSlabBytes + wave * 256)),
                  xs_goff + (uint32_t)kb_lo * (uint32_t)p.xs_k * 4u, p.xs);
@@ -224,8 +231,8 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     const uint32_t xs_lds = (uint32_t)kSlabBytes + ((uint32_t)wm * 64u + (uint32_t)l16) * 4u;
 
     // ---- the K loop, skewed by a quarter of a K block.
-    // Issue order of one iteration (32 MFMA slots):
-    //   slots 0..7   the last 8 tiles (weight fragments 6 and 7) of the PREVIOUS K block, whose
+    // Issue order of one iteration (4 NW MFMA slots; the numbers are those of NW = 8):
+    //   slots 0..7   the last 8 tiles (weight fragments NW - 2 and NW - 1) of the PREVIOUS K block, whose
     //                operands are already in registers.  They keep the matrix pipe busy while
     //                the first fragments of this K block travel from LDS, which would otherwise
     //                be dead time right after the barrier (every wave reads at once).
@@ -248,6 +255,15 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         aw[q] = i32x8{0, 0, 0, 0, 0, 0, 0, 0};
     }
     float scp[4] = {0.f, 0.f, 0.f, 0.f}; // x_scale * w_scale of the previous K block, per m tile
+    // The zero fragments must sit in their registers before the first MFMA reads them: a vector
+    // move followed at once by a matrix instruction that reads its result needs wait states, and
+    // nothing inserts them around inline asm (a stale register read as fp8 codes can hold NaN
+    // codes, and NaN x the zero scale stays NaN).  Opaque to the compiler, so that it cannot
+    // re-create the zeros right in front of the first MFMA.
+#pragma unroll
+    for(int q = 0; q < 4; ++q)
+        asm volatile("" : "+v"(bx[q]), "+v"(aw[q]));
+    asm volatile("s_nop 7" ::: "memory");
 
     typedef const volatile float __attribute__((address_space(3)))* lds_f32_ptr;
 
@@ -272,12 +288,12 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
             sc[j] = *(lds_f32_ptr)(smem3 + stage + xs_lds + j * 64) * wsc;
 
 #pragma unroll
-        for(int q = 0; q < 32; ++q)
+        for(int q = 0; q < 4 * NW; ++q)
         {
             if(q == 2)
                 aw[1] = read_frag_w(stage, w_base + 1 * 2048);
 
-            if(q < 8) // deferred tile (6 + (q & 1), q >> 1) of the previous K block
+            if(q < 8) // deferred tile (NW - 2 + (q & 1), q >> 1) of the previous K block
                 FP8BS_MFMA(P[q & 3], aw[2 + (q & 1)], bx[q >> 1]);
             else      // tile ((q - 8) >> 2, (q - 8) & 3) of this K block
                 FP8BS_MFMA(P[q & 3], aw[((q - 8) >> 2) & 3], bx[(q - 8) & 3]);
@@ -289,32 +305,26 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
                 aw[2] = read_frag_w(stage, w_base + 2 * 2048);
             if(q == 7)
                 aw[3] = read_frag_w(stage, w_base + 3 * 2048);
-            if(q == 11)
-                aw[0] = read_frag_w(stage, w_base + 4 * 2048);
-            if(q == 15)
-                aw[1] = read_frag_w(stage, w_base + 5 * 2048);
-            if(q == 19)
-                aw[2] = read_frag_w(stage, w_base + 6 * 2048);
-            if(q == 23)
-                aw[3] = read_frag_w(stage, w_base + 7 * 2048);
+            if(q >= 11 && ((q - 11) & 3) == 0 && 4 + ((q - 11) >> 2) < NW) // fragments 4 .. NW - 1 at slots 11, 15, 19, 23
+                aw[((q - 11) >> 2) & 3] = read_frag_w(stage, w_base + (4 + ((q - 11) >> 2)) * 2048);
 
-            // next stage: 8 slab loads and the x_scale column, behind the first 17 slots
-            if((q & 1) == 1 && q < 16)
+            // next stage: the slab loads and the x_scale column, in the first half of the slots
+            if((q & 1) == 1 && q < 2 * kLoads)
             {
                 const int u = q >> 1;
-                dma16(dma_dst + u * 8192, goff[u], u < 4 ? p.wq + dma_koff_w : p.xq + dma_koff);
+                dma16(dma_dst + u * 8192, goff[u], u < kWLoads ? p.wq + dma_koff_w : p.xq + dma_koff);
             }
-            if(q == 16 && wave < 4)
+            if(q == 2 * kLoads && wave < 4)
                 dma4(__builtin_amdgcn_readfirstlane(dma_dst - wave * 1024 + kSlabBytes + wave * 256),
                      xs_goff + (uint32_t)kn * (uint32_t)p.xs_k * 4u, p.xs);
 
             // fold in the product issued two slots ago
             if(q == 0)
-                FP8BS_FMA4(acc[5][2], P[2], scp[2]);
+                FP8BS_FMA4(acc[NW - 3][2], P[2], scp[2]);
             else if(q == 1)
-                FP8BS_FMA4(acc[5][3], P[3], scp[3]);
+                FP8BS_FMA4(acc[NW - 3][3], P[3], scp[3]);
             else if(q < 10)
-                FP8BS_FMA4(acc[6 + ((q - 2) & 1)][(q - 2) >> 1], P[(q - 2) & 3], scp[(q - 2) >> 1]);
+                FP8BS_FMA4(acc[NW - 2 + ((q - 2) & 1)][(q - 2) >> 1], P[(q - 2) & 3], scp[(q - 2) >> 1]);
             else
                 FP8BS_FMA4(acc[(q - 10) >> 2][(q - 10) & 3], P[(q - 2) & 3], sc[(q - 10) & 3]);
         }
@@ -333,20 +343,20 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     {
         FP8BS_MFMA(P[q & 3], aw[2 + (q & 1)], bx[q >> 1]);
         if(q == 0)
-            FP8BS_FMA4(acc[5][2], P[2], scp[2]);
+            FP8BS_FMA4(acc[NW - 3][2], P[2], scp[2]);
         else if(q == 1)
-            FP8BS_FMA4(acc[5][3], P[3], scp[3]);
+            FP8BS_FMA4(acc[NW - 3][3], P[3], scp[3]);
         else
-            FP8BS_FMA4(acc[6 + ((q - 2) & 1)][(q - 2) >> 1], P[(q - 2) & 3], scp[(q - 2) >> 1]);
+            FP8BS_FMA4(acc[NW - 2 + ((q - 2) & 1)][(q - 2) >> 1], P[(q - 2) & 3], scp[(q - 2) >> 1]);
     }
     asm volatile("s_nop 15\n s_nop 15\n s_nop 15" ::: "memory"); // >= 11 wait states after the last MFMA
-    FP8BS_FMA4(acc[6][3], P[2], scp[3]);
-    FP8BS_FMA4(acc[7][3], P[3], scp[3]);
+    FP8BS_FMA4(acc[NW - 2][3], P[2], scp[3]);
+    FP8BS_FMA4(acc[NW - 1][3], P[3], scp[3]);
 #undef FP8BS_MFMA
 #undef FP8BS_FMA4
 
     // ---- K shared out over workgroups: every workgroup parks its fp32 accumulators in the
-    // workspace exactly as its lanes hold them (item slot x 32 MFMA tiles x 512 lanes x 16 bytes:
+    // workspace exactly as its lanes hold them (item slot x 4 NW MFMA tiles x 512 lanes x 16 bytes:
     // every store and load is 1 KiB contiguous per wave), takes a ticket, and the one that draws
     // the last ticket of the tile adds the slots in split order (so the result does not depend on
     // who came last) and carries on into the ordinary epilogue.  The workgroups of a tile run on
@@ -358,9 +368,10 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         const __amdgpu_buffer_rsrc_t rsrc =
             __builtin_amdgcn_make_buffer_rsrc(partial, 0, (int)partial_bytes, 0x00020000);
         constexpr int kCoherent = 16;
-        const uint32_t mine     = ((uint32_t)(tile * splits + split) * 32u * 512u + (uint32_t)t) * 16u;
+        constexpr uint32_t kTilesPerWave = 4u * NW;
+        const uint32_t mine     = ((uint32_t)(tile * splits + split) * kTilesPerWave * 512u + (uint32_t)t) * 16u;
 #pragma unroll
-        for(int i = 0; i < 8; ++i)
+        for(int i = 0; i < NW; ++i)
 #pragma unroll
             for(int j = 0; j < 4; ++j)
                 __builtin_amdgcn_raw_buffer_store_b128(
@@ -377,7 +388,7 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
             if(t == 0) // leave the ticket ready for the next launch
                 __hip_atomic_store(tickets + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-            for(int i = 0; i < 8; ++i)
+            for(int i = 0; i < NW; ++i)
 #pragma unroll
                 for(int j = 0; j < 4; ++j)
                 {
@@ -388,7 +399,7 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
                     for(int sp = 0; sp < splits; ++sp)
                     {
                         const uint32_t off =
-                            ((uint32_t)(tile * splits + sp) * 32u * 512u + (uint32_t)t) * 16u +
+                            ((uint32_t)(tile * splits + sp) * kTilesPerWave * 512u + (uint32_t)t) * 16u +
                             (uint32_t)(i * 4 + j) * (512u * 16u);
                         if(sp == split) // uniform
                             sum += own;
@@ -402,12 +413,13 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         }
     }
 
-    // ---- epilogue.  A lane owns out[m][n .. n+3] for each of its 8 x 4 tiles: stored from there,
-    // one instruction would touch 16 rows with 32 bytes each.  The wave's 64 x 128 block goes
+    // ---- epilogue.  A lane owns out[m][n .. n+3] for each of its NW x 4 tiles: stored from there,
+    // one instruction would touch 16 rows with 32 bytes each.  The wave's 64 x NW*16 block goes
     // through its own LDS region instead (the stage buffers are free after the loop's last
-    // barrier; rows padded to 272 bytes so the 16 rows of one write fall on different banks) and
-    // leaves as 16-byte stores, 16 lanes per 256-byte row piece, 4 rows per instruction.  LDS
-    // operations of one wave complete in order, so no barrier stands between write and read.
+    // barrier; rows padded by 16 bytes so the 16 rows of one write fall on different banks) and
+    // leaves as 16-byte stores, 2 NW lanes per row piece (256 or 128 bytes), 4 or 8 rows per
+    // instruction.  LDS operations of one wave complete in order, so no barrier stands between
+    // write and read.
     if(writes_out) // uniform
     {
         const uint32_t ebase = (uint32_t)wave * (64u * kEpiPitch);
@@ -416,18 +428,20 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
 #pragma unroll
         for(int j = 0; j < 4; ++j)
 #pragma unroll
-            for(int i = 0; i < 8; ++i)
+            for(int i = 0; i < NW; ++i)
                 *(lds_u2_ptr)(smem3 + ebase + (uint32_t)(j * 16 + l16) * kEpiPitch +
                               (uint32_t)(i * 16 + kg * 4) * 2u) =
                     u32x2{pack2<DT>(acc[i][j][0], acc[i][j][1]), pack2<DT>(acc[i][j][2], acc[i][j][3])};
 
-        const int  col    = (lane & 15) * 8;
-        const int  n      = n0 + wn * 128 + col;
+        constexpr int kRowLanes = 2 * NW;          // lanes that store one row piece
+        constexpr int kRowsPer  = 64 / kRowLanes;  // rows per store instruction
+        const int  col    = (lane & (kRowLanes - 1)) * 8;
+        const int  n      = n0 + wn * (NW * 16) + col;
         const bool vec_ok = (p.N & 7) == 0 && ((uintptr_t)p.out & 15) == 0 && n + 8 <= p.N;
 #pragma unroll
-        for(int c = 0; c < 16; ++c)
+        for(int c = 0; c < 64 / kRowsPer; ++c)
         {
-            const int   row = c * 4 + (lane >> 4);
+            const int   row = c * kRowsPer + lane / kRowLanes;
             const int   m   = m0 + wm * 64 + row;
             const u32x4 vv  = *(lds_u4_ptr)(smem3 + ebase + (uint32_t)row * kEpiPitch + (uint32_t)col * 2u);
             if(m >= p.M)
@@ -467,71 +481,81 @@ bool gemm_prefill_supports(const GemmKernelParams& p)
 // cover all (8192 x 36864 x 7168: 18 rounds x (8 + 56 x 1.79) = 1948 us, measured 1950).  K
 // ranges over s workgroups per tile cost 4 us plus the parked tiles' traffic, (2 s - 1) x 256 KiB
 // per tile at about 5 TB/s (2048 x 4096 x 7168: 89.8 us as one range, 77-80 us as two).
+// 256 x 128 tiles: 6 us per round and 1.2 us per K block, rising to 1.4 us when the workgroups of a round
+// cover all compute units (a compute unit takes in its 48 KiB per K block no faster than the wide
+// tile's 64 KiB: what the narrow tile buys is workgroups, not speed; 1024 x 7168 x 2048: 26.4 us
+// against 34.4, 256 x 24576 x 1536: 22.5 against 30.9, 2048 x 4096 x 7168: 84.0 against 78.8 with
+// the wide tile's K ranges).
+constexpr float kFixed128 = 6.f, kIter128 = 1.2f;
+
+static float plan_cost(const GemmKernelParams& p, int cus, int bn, int s)
+{
+    const int   tiles  = ((p.M + kBM - 1) / kBM) * ((p.N + bn - 1) / bn);
+    const int   items  = tiles * s;
+    const int   rounds = (items + cus - 1) / cus;
+    const float share  = (float)items / (float)(rounds * cus);
+    const int   kb     = (p.kblocks + s - 1) / s;
+    if(bn == 128)
+        return (float)rounds * (kFixed128 + (float)kb * (kIter128 + (share > 0.44f ? (share - 0.44f) * 0.35f : 0.f)));
+    const float iter = 1.36f + (share > 0.44f ? (share - 0.44f) * 0.77f : 0.f);
+    return (float)rounds * (8.f + (float)kb * iter) +
+           (s > 1 ? 4.f + (float)tiles * (float)(2 * s - 1) * 0.05f : 0.f);
+}
+
 PrefillPlan gemm_prefill_plan(const GemmKernelParams& p, int cus)
 {
-    const int tiles = ((p.M + kBM - 1) / kBM) * ((p.N + kBN - 1) / kBN);
+    const int tiles = ((p.M + kBM - 1) / kBM) * ((p.N + 255) / 256);
     cus             = std::max(cus, 1);
-    auto cost = [&](int s) {
-        const int   items  = tiles * s;
-        const int   rounds = (items + cus - 1) / cus;
-        const float share  = (float)items / (float)(rounds * cus);
-        const float iter   = 1.36f + (share > 0.44f ? (share - 0.44f) * 0.77f : 0.f);
-        const int   kb     = (p.kblocks + s - 1) / s;
-        return (float)rounds * (8.f + (float)kb * iter) +
-               (s > 1 ? 4.f + (float)tiles * (float)(2 * s - 1) * 0.05f : 0.f);
-    };
-    PrefillPlan best{1, cost(1)};
+    PrefillPlan best{1, plan_cost(p, cus, 256, 1), 256};
     for(int s = 2; s <= 3; ++s)
     {
         // (below 64 tiles the model is off: 1024 x 2112 x 7168, 36 tiles x 3, takes 67 us where it
         // says 47, and the mid_* kernels need 51)
         if(tiles < 64 || tiles * s > cus || p.kblocks / s < 8 || (p.N & 3) != 0)
             break;
-        const float c = cost(s);
+        const float c = plan_cost(p, cus, 256, s);
         if(c < best.us * 0.97f)
-            best = PrefillPlan{s, c};
+            best = PrefillPlan{s, c, 256};
+    }
+    // half-width tiles where the wide ones leave at least half of the compute units without a workgroup
+    if(tiles * 2 <= cus)
+    {
+        const float c = plan_cost(p, cus, 128, 1);
+        if(c < best.us * 0.97f)
+            best = PrefillPlan{1, c, 128};
     }
     return best;
 }
 
-hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, const LaunchCtx& ctx, int want_splits)
+template <int NW>
+static hipError_t launch_prefill_nw(const GemmKernelParams& p, In16 out_dtype, const LaunchCtx& ctx, int splits,
+                                    int device, int cus)
 {
+    constexpr int     kBN    = tile_n(NW);
     const hipStream_t stream = ctx.stream;
     const int    tiles_m = (p.M + kBM - 1) / kBM, tiles_n = (p.N + kBN - 1) / kBN;
     // the two stages, or the eight waves' output blocks of the epilogue, whichever is larger
-    const size_t smem    = std::max((size_t)kStages * kStageBytes, (size_t)8 * 64 * kEpiPitch);
+    const size_t smem    = std::max((size_t)kStages * stage_bytes(NW), (size_t)8 * 64 * epi_pitch(NW));
     const bool   bf      = out_dtype == In16::bf16;
-    auto         kernel  = p.w_shuffled ? (bf ? gemm_prefill_kernel<In16::bf16, true> : gemm_prefill_kernel<In16::fp16, true>)
-                                        : (bf ? gemm_prefill_kernel<In16::bf16, false> : gemm_prefill_kernel<In16::fp16, false>);
-    // Per device and instantiation, once: the opt-in to more than 64 KiB of LDS, and the number of
-    // compute units.  (Racing first calls repeat the same idempotent set-up.)
+    auto         kernel  = p.w_shuffled ? (bf ? gemm_prefill_kernel<In16::bf16, true, NW> : gemm_prefill_kernel<In16::fp16, true, NW>)
+                                        : (bf ? gemm_prefill_kernel<In16::bf16, false, NW> : gemm_prefill_kernel<In16::fp16, false, NW>);
+    // Per device and instantiation, once: the opt-in to more than 64 KiB of LDS.  (Racing first
+    // calls repeat the same idempotent set-up.)
     constexpr int kMaxDevices = 64;
-    static std::atomic<int>  cus_of[kMaxDevices];
     static std::atomic<bool> ready[kMaxDevices][4];
-    int           device = 0, cus = 0;
-    hipError_t    e = hipGetDevice(&device);
-    if(e != hipSuccess)
-        return e;
     const int inst = (p.w_shuffled ? 2 : 0) + (bf ? 0 : 1);
+    hipError_t e;
     if(device < 0 || device >= kMaxDevices || !ready[device][inst])
     {
         if((e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem)) != hipSuccess ||
-           (e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device)) != hipSuccess)
+                                    (int)smem)) != hipSuccess)
             return e;
         if(device >= 0 && device < kMaxDevices)
-        {
-            cus_of[device]      = cus;
             ready[device][inst] = true;
-        }
     }
-    else
-        cus = cus_of[device];
     // one workgroup fills a compute unit (LDS, registers); with more tiles than compute units the
     // workgroups walk the tiles.  A multiple of 8 keeps a workgroup's tiles on one XCD's patch order.
     const int total = tiles_m * tiles_n;
-    // want_splits: 0 = the plan's choice, otherwise as told
-    int splits = want_splits > 0 ? want_splits : gemm_prefill_plan(p, cus).splits;
     if(total * splits > 4096) // 32-bit byte offsets into the parked tiles
         splits = 1;
     splits                 = std::max(1, std::min(splits, (int)p.kblocks));
@@ -543,7 +567,7 @@ hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, const 
     WorkspaceLock lock(splits > 1);
     if(splits > 1)
     {
-        bytes = (size_t)total * splits * 32 * 512 * 16;
+        bytes = (size_t)total * splits * (4 * NW) * 512 * 16;
         if((e = split_workspace(ctx, lock, bytes, (size_t)total, &partial, &tickets)) != hipSuccess)
             return e;
     }
@@ -552,6 +576,33 @@ hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, const 
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), smem, stream, p, tiles_m, tiles_n, splits,
                        kb_per_split, partial, (uint32_t)bytes, tickets);
     return hipGetLastError();
+}
+
+hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, const LaunchCtx& ctx, int want_splits,
+                               int want_tile_n)
+{
+    // the number of compute units, per device, once
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> cus_of[kMaxDevices];
+    int           device = 0, cus = 0;
+    hipError_t    e = hipGetDevice(&device);
+    if(e != hipSuccess)
+        return e;
+    if(device >= 0 && device < kMaxDevices)
+        cus = cus_of[device];
+    if(cus == 0)
+    {
+        if((e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device)) != hipSuccess)
+            return e;
+        if(device >= 0 && device < kMaxDevices)
+            cus_of[device] = cus;
+    }
+    // want_splits / want_tile_n: 0 = the plan's choice, otherwise as told
+    const PrefillPlan plan = gemm_prefill_plan(p, cus);
+    const int bn     = want_tile_n == 128 || want_tile_n == 256 ? want_tile_n : (want_splits > 0 ? 256 : plan.tile_n);
+    const int splits = want_splits > 0 ? want_splits : (bn == plan.tile_n ? plan.splits : 1);
+    return bn == 128 ? launch_prefill_nw<4>(p, out_dtype, ctx, splits, device, cus)
+                     : launch_prefill_nw<8>(p, out_dtype, ctx, splits, device, cus);
 }
 
 } // namespace fp8bs
