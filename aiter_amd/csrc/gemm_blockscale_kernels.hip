@@ -161,7 +161,7 @@ static hipError_t launch_tile(const GemmKernelParams& p, hipStream_t stream)
 }
 
 static const char* const kKernelNames =
-    "tile_16x256,tile_64x128,tile_128x128,mid_64x64,mid_64x128,mid_128x128,prefill_256x256,prefill_256x128,"
+    "tile_16x256,tile_64x128,tile_128x128,mid_64x64,mid_64x128,mid_128x128,prefill_256x256,prefill_256x192,prefill_256x128,"
     "decode_stream";
 
 const char* gemm_kernel_names() { return kKernelNames; }
@@ -181,7 +181,10 @@ static const char* automatic_choice(const GemmKernelParams& p)
     if(gemm_mid_supports(p) && (!gemm_prefill_supports(p) || gemm_mid_estimate_us(p) * 1.03f < prefill_us))
         return "mid_auto";
     if(gemm_prefill_supports(p))
-        return gemm_prefill_plan(p, 256).tile_n == 128 ? "prefill_256x128" : "prefill_256x256";
+    {
+        const int bn = gemm_prefill_plan(p, 256).tile_n;
+        return bn == 128 ? "prefill_256x128" : bn == 192 ? "prefill_256x192" : "prefill_256x256";
+    }
     return "tile_128x128";
 }
 
@@ -255,11 +258,11 @@ static bool parse_kernel_name(const char* name, ParsedKernel* out)
             return false;
         return out->tile >= 0;
     }
-    // "prefill_256x256" / "prefill_256x128", or "prefill_256x256:s=2" to pin the number of K ranges per tile
-    if(is("prefill_256x256") || is("prefill_256x128"))
+    // "prefill_256x256" / "prefill_256x192" / "prefill_256x128", or "prefill_256x256:s=2" to pin the number of K ranges per tile
+    if(is("prefill_256x256") || is("prefill_256x192") || is("prefill_256x128"))
     {
         out->family = Family::prefill;
-        out->tile   = is("prefill_256x128") ? 128 : 256;
+        out->tile   = is("prefill_256x128") ? 128 : is("prefill_256x192") ? 192 : 256;
         if(colon && (sscanf(colon, ":s=%d", &out->splits) != 1 || out->splits < 1 || out->splits > 16))
             return false;
         return true;

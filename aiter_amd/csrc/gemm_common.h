@@ -88,11 +88,11 @@ struct PrefillPlan
 {
     int   splits;
     float us;
-    int   tile_n; // 256 or 128 columns per tile
+    int   tile_n; // 256, 192 or 128 columns per tile
 };
 PrefillPlan gemm_prefill_plan(const GemmKernelParams& p, int cus);
 // want_splits: K ranges per tile; 0 lets the launcher choose, 1 keeps a tile in one workgroup.
-// want_tile_n: 256 or 128 columns per tile; 0 lets the launcher choose (together with the K ranges).
+// want_tile_n: 256, 192 or 128 columns per tile; 0 lets the launcher choose (together with the K ranges).
 hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, const LaunchCtx& ctx, int want_splits,
                                int want_tile_n = 0);
 bool       gemm_prefill_supports(const GemmKernelParams& p);

@@ -23,7 +23,8 @@ constexpr int kBM = 256, kThreads = 512;
 constexpr int kStages = 2;
 constexpr int kGroupN = 4; // n tiles swept together by consecutive workgroups
 // The tile is 256 (m) x NW * 32 (n): NW = 8 weight fragments per wave for the 256 x 256 tile, 4 for the
-// 256 x 128 one (twice the workgroups where the wide tiles leave compute units idle).
+// 256 x 128 one (twice the workgroups where the wide tiles leave compute units idle), 6 for the
+// 256 x 192 one (N = 2112 = 11 x 192: no ragged last column of tiles).
 constexpr int tile_n(int nw) { return nw * 32; }
 constexpr int slab_bytes(int nw) { return (kBM + tile_n(nw)) * 128; } // weight rows, then 256 activation rows
 constexpr int stage_bytes(int nw) { return slab_bytes(nw) + kBM * 4; } // + this K block's x_scale for the 256 rows
@@ -147,10 +148,16 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         xs_goff    = m * (uint32_t)p.xs_m * 4u;
     }
 
-    // ---- scales: x_scale comes through LDS with each stage, w_scale: one block per wave
-    uint32_t nb = (uint32_t)(n0 + wn * (NW * 16)) >> 7;
-    nb          = min(nb, (uint32_t)((p.N + 127) / 128 - 1));
-    const float* ws_row = p.ws + (size_t)nb * p.kblocks;
+    // ---- scales: x_scale comes through LDS with each stage, w_scale: one block per wave, or (six
+    // fragments: a wave's 96 columns can straddle a block boundary) two, the second from fragment
+    // `ws_split` on.  Fragments share a scale in pairs: group g = fragment / 2.
+    constexpr int  kScaleGroups = NW == 6 ? 3 : 1;
+    const uint32_t n_wave  = (uint32_t)(n0 + wn * (NW * 16));
+    const uint32_t nb_last = (uint32_t)((p.N + 127) / 128 - 1);
+    const uint32_t nb      = min(n_wave >> 7, nb_last);
+    const float* ws_row  = p.ws + (size_t)nb * p.kblocks;
+    const float* ws_row2 = p.ws + (size_t)min(nb + 1u, nb_last) * p.kblocks;
+    const int    ws_split = __builtin_amdgcn_readfirstlane((int)((128u - (n_wave & 127u)) >> 4)); // 8, 6, 4 or 2
 
     // ---- LDS read addresses.  A fragment is 32 bytes of one row: logical chunks 2kg and 2kg+1.
     // Tile rows start at multiples of 16, so the swizzle term depends on l16 only and every
@@ -206,13 +213,14 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     // w_scale of this wave's n block for 64 consecutive K blocks lives in one VGPR (lane = K
     // block) and is picked with v_readlane: a scalar load inside the loop would share the LGKM
     // counter with the LDS reads and force them to be waited for in full.
-    auto load_ws_window = [&](int kb0) -> float {
+    auto load_ws_window = [&](const float* row, int kb0) -> float {
         const int k = kb0 + lane;
-        return ws_row[k < p.kblocks ? k : p.kblocks - 1];
+        return row[k < p.kblocks ? k : p.kblocks - 1];
     };
-    float ws_vec = load_ws_window(kb_lo & ~63);
-    auto  ws_at  = [&](int kb) -> float {
-        return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(ws_vec), kb & 63));
+    float ws_vec  = load_ws_window(ws_row, kb_lo & ~63);
+    float ws_vec2 = kScaleGroups > 1 ? load_ws_window(ws_row2, kb_lo & ~63) : 0.f;
+    auto  ws_at   = [&](float vec, int kb) -> float {
+        return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(vec), kb & 63));
     };
 
     {
@@ -246,15 +254,24 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
 #pragma unroll
     for(int q = 0; q < 4; ++q)
         P[q] = f32x4{0.f, 0.f, 0.f, 0.f};
-    i32x8 bx[4], aw[4];
+    // weight fragment i lives in buffer BUF(i): four buffers in rotation, or one per fragment
+    constexpr int kBufs = NW == 6 ? 6 : 4;
+#define FP8BS_BUF(i) (NW == 6 ? (i) : ((i)&3))
+    i32x8 bx[4], aw[kBufs];
 #pragma unroll
-    for(int q = 0; q < 4; ++q)
-    {
-        // first iteration: the "previous K block" is all zero codes with zero scales
+    for(int q = 0; q < 4; ++q) // first iteration: the "previous K block" is all zero codes with zero scales
         bx[q] = i32x8{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for(int q = 0; q < kBufs; ++q)
         aw[q] = i32x8{0, 0, 0, 0, 0, 0, 0, 0};
-    }
-    float scp[4] = {0.f, 0.f, 0.f, 0.f}; // x_scale * w_scale of the previous K block, per m tile
+    // x_scale * w_scale of the previous K block, per scale group and m tile
+    float scp[kScaleGroups][4];
+#pragma unroll
+    for(int g = 0; g < kScaleGroups; ++g)
+#pragma unroll
+        for(int j = 0; j < 4; ++j)
+            scp[g][j] = 0.f;
+#define FP8BS_GROUP(i) (NW == 6 ? (i) >> 1 : 0)
     // The zero fragments must sit in their registers before the first MFMA reads them: a vector
     // move followed at once by a matrix instruction that reads its result needs wait states, and
     // nothing inserts them around inline asm (a stale register read as fp8 codes can hold NaN
@@ -262,7 +279,10 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     // re-create the zeros right in front of the first MFMA.
 #pragma unroll
     for(int q = 0; q < 4; ++q)
-        asm volatile("" : "+v"(bx[q]), "+v"(aw[q]));
+        asm volatile("" : "+v"(bx[q]));
+#pragma unroll
+    for(int q = 0; q < kBufs; ++q)
+        asm volatile("" : "+v"(aw[q]));
     asm volatile("s_nop 7" ::: "memory");
 
     typedef const volatile float __attribute__((address_space(3)))* lds_f32_ptr;
@@ -278,14 +298,30 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         const size_t   dma_koff_w = SHUF ? (size_t)kn * 2048 : dma_koff;
 
         if((kb & 63) == 0 && kb != kb_lo)
-            ws_vec = load_ws_window(kb);
-        const float wsc = ws_at(kb);
+        {
+            ws_vec = load_ws_window(ws_row, kb);
+            if(kScaleGroups > 1)
+                ws_vec2 = load_ws_window(ws_row2, kb);
+        }
+        float wsc[kScaleGroups];
+        wsc[0] = ws_at(ws_vec, kb);
+        if constexpr(kScaleGroups > 1)
+        {
+            const float second = ws_at(ws_vec2, kb);
+            wsc[1]             = ws_split <= 2 ? second : wsc[0]; // fragments 2, 3
+            wsc[2]             = ws_split <= 4 ? second : wsc[0]; // fragments 4, 5
+        }
 
         aw[0] = read_frag_w(stage, w_base); // weight fragment 0 of this K block
-        float sc[4];
+        float sc[kScaleGroups][4];
 #pragma unroll
         for(int j = 0; j < 4; ++j)
-            sc[j] = *(lds_f32_ptr)(smem3 + stage + xs_lds + j * 64) * wsc;
+        {
+            const float xsv = *(lds_f32_ptr)(smem3 + stage + xs_lds + j * 64);
+#pragma unroll
+            for(int g = 0; g < kScaleGroups; ++g)
+                sc[g][j] = xsv * wsc[g];
+        }
 
 #pragma unroll
         for(int q = 0; q < 4 * NW; ++q)
@@ -294,9 +330,9 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
                 aw[1] = read_frag_w(stage, w_base + 1 * 2048);
 
             if(q < 8) // deferred tile (NW - 2 + (q & 1), q >> 1) of the previous K block
-                FP8BS_MFMA(P[q & 3], aw[2 + (q & 1)], bx[q >> 1]);
+                FP8BS_MFMA(P[q & 3], aw[FP8BS_BUF(NW - 2 + (q & 1))], bx[q >> 1]);
             else      // tile ((q - 8) >> 2, (q - 8) & 3) of this K block
-                FP8BS_MFMA(P[q & 3], aw[((q - 8) >> 2) & 3], bx[(q - 8) & 3]);
+                FP8BS_MFMA(P[q & 3], aw[FP8BS_BUF((q - 8) >> 2)], bx[(q - 8) & 3]);
 
             // LDS reads that the slot just issued has made room for
             if(q < 8 && (q & 1))
@@ -306,7 +342,7 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
             if(q == 7)
                 aw[3] = read_frag_w(stage, w_base + 3 * 2048);
             if(q >= 11 && ((q - 11) & 3) == 0 && 4 + ((q - 11) >> 2) < NW) // fragments 4 .. NW - 1 at slots 11, 15, 19, 23
-                aw[((q - 11) >> 2) & 3] = read_frag_w(stage, w_base + (4 + ((q - 11) >> 2)) * 2048);
+                aw[FP8BS_BUF(4 + ((q - 11) >> 2))] = read_frag_w(stage, w_base + (4 + ((q - 11) >> 2)) * 2048);
 
             // next stage: the slab loads and the x_scale column, in the first half of the slots
             if((q & 1) == 1 && q < 2 * kLoads)
@@ -320,17 +356,21 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
 
             // fold in the product issued two slots ago
             if(q == 0)
-                FP8BS_FMA4(acc[NW - 3][2], P[2], scp[2]);
+                FP8BS_FMA4(acc[NW - 3][2], P[2], scp[FP8BS_GROUP(NW - 3)][2]);
             else if(q == 1)
-                FP8BS_FMA4(acc[NW - 3][3], P[3], scp[3]);
+                FP8BS_FMA4(acc[NW - 3][3], P[3], scp[FP8BS_GROUP(NW - 3)][3]);
             else if(q < 10)
-                FP8BS_FMA4(acc[NW - 2 + ((q - 2) & 1)][(q - 2) >> 1], P[(q - 2) & 3], scp[(q - 2) >> 1]);
+                FP8BS_FMA4(acc[NW - 2 + ((q - 2) & 1)][(q - 2) >> 1], P[(q - 2) & 3],
+                           scp[FP8BS_GROUP(NW - 2)][(q - 2) >> 1]);
             else
-                FP8BS_FMA4(acc[(q - 10) >> 2][(q - 10) & 3], P[(q - 2) & 3], sc[(q - 10) & 3]);
+                FP8BS_FMA4(acc[(q - 10) >> 2][(q - 10) & 3], P[(q - 2) & 3],
+                           sc[FP8BS_GROUP((q - 10) >> 2)][(q - 10) & 3]);
         }
 #pragma unroll
-        for(int j = 0; j < 4; ++j)
-            scp[j] = sc[j];
+        for(int g = 0; g < kScaleGroups; ++g)
+#pragma unroll
+            for(int j = 0; j < 4; ++j)
+                scp[g][j] = sc[g][j];
 
         // vmcnt(0): this wave's share of the next stage is in LDS; the barrier (which also
         // waits for this wave's outstanding LDS reads) publishes it and retires the stage just read
@@ -341,19 +381,22 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
 #pragma unroll
     for(int q = 0; q < 8; ++q)
     {
-        FP8BS_MFMA(P[q & 3], aw[2 + (q & 1)], bx[q >> 1]);
+        FP8BS_MFMA(P[q & 3], aw[FP8BS_BUF(NW - 2 + (q & 1))], bx[q >> 1]);
         if(q == 0)
-            FP8BS_FMA4(acc[NW - 3][2], P[2], scp[2]);
+            FP8BS_FMA4(acc[NW - 3][2], P[2], scp[FP8BS_GROUP(NW - 3)][2]);
         else if(q == 1)
-            FP8BS_FMA4(acc[NW - 3][3], P[3], scp[3]);
+            FP8BS_FMA4(acc[NW - 3][3], P[3], scp[FP8BS_GROUP(NW - 3)][3]);
         else
-            FP8BS_FMA4(acc[NW - 2 + ((q - 2) & 1)][(q - 2) >> 1], P[(q - 2) & 3], scp[(q - 2) >> 1]);
+            FP8BS_FMA4(acc[NW - 2 + ((q - 2) & 1)][(q - 2) >> 1], P[(q - 2) & 3],
+                       scp[FP8BS_GROUP(NW - 2)][(q - 2) >> 1]);
     }
     asm volatile("s_nop 15\n s_nop 15\n s_nop 15" ::: "memory"); // >= 11 wait states after the last MFMA
-    FP8BS_FMA4(acc[NW - 2][3], P[2], scp[3]);
-    FP8BS_FMA4(acc[NW - 1][3], P[3], scp[3]);
+    FP8BS_FMA4(acc[NW - 2][3], P[2], scp[FP8BS_GROUP(NW - 2)][3]);
+    FP8BS_FMA4(acc[NW - 1][3], P[3], scp[FP8BS_GROUP(NW - 1)][3]);
 #undef FP8BS_MFMA
 #undef FP8BS_FMA4
+#undef FP8BS_BUF
+#undef FP8BS_GROUP
 
     // ---- K shared out over workgroups: every workgroup parks its fp32 accumulators in the
     // workspace exactly as its lanes hold them (item slot x 4 NW MFMA tiles x 512 lanes x 16 bytes:
@@ -434,14 +477,17 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
                     u32x2{pack2<DT>(acc[i][j][0], acc[i][j][1]), pack2<DT>(acc[i][j][2], acc[i][j][3])};
 
         constexpr int kRowLanes = 2 * NW;          // lanes that store one row piece
-        constexpr int kRowsPer  = 64 / kRowLanes;  // rows per store instruction
-        const int  col    = (lane & (kRowLanes - 1)) * 8;
+        constexpr int kRowsPer  = 64 / kRowLanes;  // rows per store instruction (lanes beyond them idle)
+        const int  rl     = lane / kRowLanes;
+        const int  col    = (lane - rl * kRowLanes) * 8;
         const int  n      = n0 + wn * (NW * 16) + col;
         const bool vec_ok = (p.N & 7) == 0 && ((uintptr_t)p.out & 15) == 0 && n + 8 <= p.N;
 #pragma unroll
-        for(int c = 0; c < 64 / kRowsPer; ++c)
+        for(int c = 0; c < (64 + kRowsPer - 1) / kRowsPer; ++c)
         {
-            const int   row = c * kRowsPer + lane / kRowLanes;
+            const int row = c * kRowsPer + rl;
+            if(rl >= kRowsPer || row >= 64)
+                continue;
             const int   m   = m0 + wm * 64 + row;
             const u32x4 vv  = *(lds_u4_ptr)(smem3 + ebase + (uint32_t)row * kEpiPitch + (uint32_t)col * 2u);
             if(m >= p.M)
@@ -497,6 +543,10 @@ static float plan_cost(const GemmKernelParams& p, int cus, int bn, int s)
     const int   kb     = (p.kblocks + s - 1) / s;
     if(bn == 128)
         return (float)rounds * (kFixed128 + (float)kb * (kIter128 + (share > 0.44f ? (share - 0.44f) * 0.35f : 0.f)));
+    if(bn == 192) // 56 KiB and 24 MFMA slots per K block: 1.4 us (4096 x 2112 x 7168, 176 workgroups: 86.9 us;
+                  // 2048 x 2112 x 7168 as 88 tiles x 2 K ranges: 60.3 us against 73.1 with the wide tile)
+        return (float)rounds * (7.f + (float)kb * 1.4f) +
+               (s > 1 ? 4.f + (float)tiles * (float)(2 * s - 1) * 0.0375f : 0.f);
     const float iter = 1.36f + (share > 0.44f ? (share - 0.44f) * 0.77f : 0.f);
     return (float)rounds * (8.f + (float)kb * iter) +
            (s > 1 ? 4.f + (float)tiles * (float)(2 * s - 1) * 0.05f : 0.f);
@@ -523,6 +573,20 @@ PrefillPlan gemm_prefill_plan(const GemmKernelParams& p, int cus)
         const float c = plan_cost(p, cus, 128, 1);
         if(c < best.us * 0.97f)
             best = PrefillPlan{1, c, 128};
+    }
+    // 192-wide tiles where they divide N and 256-wide ones do not (N = 2112: a ninth column of tiles
+    // that is three quarters empty against eleven full ones)
+    if(p.N % 192 == 0 && p.N % 256 != 0)
+    {
+        const int t192 = ((p.M + kBM - 1) / kBM) * (p.N / 192);
+        for(int s = 1; s <= 3; ++s)
+        {
+            if(s > 1 && (t192 < 64 || t192 * s > cus || p.kblocks / s < 8)) // (as above: few tiles, model off)
+                break;
+            const float c = plan_cost(p, cus, 192, s);
+            if(c < best.us * 0.97f)
+                best = PrefillPlan{s, c, 192};
+        }
     }
     return best;
 }
@@ -599,10 +663,13 @@ hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, const 
     }
     // want_splits / want_tile_n: 0 = the plan's choice, otherwise as told
     const PrefillPlan plan = gemm_prefill_plan(p, cus);
-    const int bn     = want_tile_n == 128 || want_tile_n == 256 ? want_tile_n : (want_splits > 0 ? 256 : plan.tile_n);
+    const int bn     = want_tile_n == 128 || want_tile_n == 192 || want_tile_n == 256
+                           ? want_tile_n
+                           : (want_splits > 0 ? 256 : plan.tile_n);
     const int splits = want_splits > 0 ? want_splits : (bn == plan.tile_n ? plan.splits : 1);
-    return bn == 128 ? launch_prefill_nw<4>(p, out_dtype, ctx, splits, device, cus)
-                     : launch_prefill_nw<8>(p, out_dtype, ctx, splits, device, cus);
+    return bn == 128   ? launch_prefill_nw<4>(p, out_dtype, ctx, splits, device, cus)
+           : bn == 192 ? launch_prefill_nw<6>(p, out_dtype, ctx, splits, device, cus)
+                       : launch_prefill_nw<8>(p, out_dtype, ctx, splits, device, cus);
 }
 
 } // namespace fp8bs

@@ -63,7 +63,7 @@ def test_config1_plumbing():
 
 
 @pytest.mark.parametrize("kernel", [None, "tile_16x256", "tile_64x128", "tile_128x128", "mid_64x64", "mid_64x128",
-                                    "mid_128x128", "prefill_256x256", "prefill_256x128", "decode_stream"])
+                                    "mid_128x128", "prefill_256x256", "prefill_256x192", "prefill_256x128", "decode_stream"])
 @pytest.mark.parametrize(
     "m,n,k",
     [(1, 128, 128), (1, 2112, 512), (16, 256, 1024), (17, 384, 256), (64, 2112, 1024), (130, 520, 384), (257, 1000, 256)],
@@ -74,7 +74,7 @@ def test_shapes_and_tiles(kernel, m, n, k):
     assert_close_to_f64(out, xq, wq, xs, ws, f"{kernel} {m}x{n}x{k}")
 
 
-@pytest.mark.parametrize("name", ["prefill_256x256", "prefill_256x128"])
+@pytest.mark.parametrize("name", ["prefill_256x256", "prefill_256x192", "prefill_256x128"])
 @pytest.mark.parametrize("m,n,k", [(256, 256, 128), (512, 768, 1024), (300, 1000, 384), (1024, 2112, 512), (257, 260, 256)])
 def test_prefill_kernel_shapes(m, n, k, name):
     xq, wq, xs, ws = make_problem(m, n, k, seed=m + n + k, outliers=0.01)
@@ -410,6 +410,8 @@ def test_config4_full_size(layout):
     (256, 256, 4096, "prefill_256x256:s=4"),   # one tile, four workgroups
     (512, 768, 2048, "prefill_256x128:s=2"),   # half-width tiles: 12 tiles x 2 ranges
     (300, 1000, 1408, "prefill_256x128:s=3"),
+    (512, 2112, 2048, "prefill_256x192:s=2"),  # eleven full 192-wide tiles per row of tiles, two scale blocks per wave
+    (300, 1000, 1408, "prefill_256x192:s=3"),
     (2048, 4096, 7168, ""),                    # BASELINE config 5's GEMM: the library's own choice (2 ranges)
 ])
 def test_prefill_kernel_k_ranges_across_workgroups(m, n, k, name):

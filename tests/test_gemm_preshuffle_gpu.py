@@ -49,7 +49,7 @@ def test_matches_oracle_and_plain_layout(m, n, k, form):
 
 
 @pytest.mark.parametrize("kernel", ["tile_16x256", "tile_64x128", "tile_128x128", "mid_64x64", "mid_64x128", "mid_128x128", "prefill_256x256",
-                                    "prefill_256x128", "decode_stream", "mid_128x128:s=2", "mid_64x64:s=2"])
+                                    "prefill_256x192", "prefill_256x128", "decode_stream", "mid_128x128:s=2", "mid_64x64:s=2"])
 @pytest.mark.parametrize("m", [48, 272])
 def test_named_kernels(kernel, m):
     n, k = 1008, 1024
