@@ -24,6 +24,8 @@
 #include "gemm_common.h"
 #include "moe_launch.h"
 
+#include <atomic>
+
 namespace fp8bs {
 
 namespace {
@@ -879,6 +881,7 @@ struct DownColsParams
 constexpr int kColsDepth     = 8;
 constexpr int kColsTiles     = 2;    // 16-column tiles per workgroup
 constexpr int kColsMaxBlocks = 1024; // blocks the unit scan takes (16 per lane)
+constexpr size_t kColsTableBytes = (size_t)140 << 10; // LDS for the per-token tables; the unit list (16 KiB at most) comes on top
 
 struct ColsStage
 {
@@ -1180,18 +1183,19 @@ size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 bool rows_in_f32(const MoeArgs& a) { return (size_t)a.M * a.topk * a.dim * 4 <= ((size_t)32 << 20); }
 
 // Decode-size batches take the second GEMM that owns output columns and sums per token in LDS
-// (moe_down_cols_kernel): its tables, [2 * inter/128][tokens + 16][16] fp32 (at most 44 KiB), and its unit list
-// (16 bytes per block, at most 16 KiB) have to fit 64 KiB of LDS.  Beyond, rows go through memory and moe_combine_kernel adds them.  down_mode 1 / 2
+// (moe_down_cols_kernel): its tables, [2 * inter/128][tokens + 16][16] fp32 (at most 140 KiB: 544 tokens at
+// inter = 256), and its unit list (16 bytes per block, at most 16 KiB) have to fit the 160 KiB of LDS.  Beyond, rows go through memory and moe_combine_kernel adds them.  down_mode 1 / 2
 // force the one / the other (2 only where it fits).
 bool down_by_columns(const MoeArgs& a)
 {
     const int  kblocks = a.inter / 128;
-    const bool fits    = kblocks <= 4 && (size_t)kColsTiles * kblocks * (a.M + 16) * 64 <= ((size_t)44 << 10) &&
+    const bool fits    = kblocks <= 4 && (size_t)kColsTiles * kblocks * (a.M + 16) * 64 <= kColsTableBytes &&
                       a.max_blocks <= kColsMaxBlocks && a.dim % (16 * kColsTiles) == 0;
     if(a.down_mode == 1 || !fits)
         return false;
-    // measured on the DeepSeek-V3 layer: 12 % faster at 1 token, 1-2 % up to 128, slower from 256
-    return a.down_mode == 2 || a.M <= 128;
+    // measured on the DeepSeek-V3 layer against rows through memory: 12 % faster at 1 token, 3 % at 128 and
+    // 192, 2 % at 256, even at 384, 8 % slower at 512 (the tables' clearing and final sum grow with the tokens)
+    return a.down_mode == 2 || a.M <= 320;
 }
 
 } // namespace
@@ -1442,10 +1446,21 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
         c.experts           = a.experts;
         const size_t lds    = (size_t)a.max_blocks * 16 + (size_t)kColsTiles * c.kblocks * (a.M + 16) * 64;
         const dim3   grid((unsigned)(a.dim / (16 * kColsTiles))), block((unsigned)(64 * c.kblocks * kColsTiles));
-        if(a.out_dtype == In16::bf16)
-            hipLaunchKernelGGL(moe_down_cols_kernel<In16::bf16>, grid, block, lds, stream, c);
-        else
-            hipLaunchKernelGGL(moe_down_cols_kernel<In16::fp16>, grid, block, lds, stream, c);
+        auto kernel = a.out_dtype == In16::bf16 ? moe_down_cols_kernel<In16::bf16> : moe_down_cols_kernel<In16::fp16>;
+        constexpr int            kMaxDevices = 64;
+        static std::atomic<bool> raised[kMaxDevices][2]; // dynamic LDS above the default limit needs opting in, once
+        const int                inst = a.out_dtype == In16::bf16 ? 0 : 1;
+        if(a.device_id < 0 || a.device_id >= kMaxDevices)
+            return hipErrorInvalidDevice;
+        if(!raised[a.device_id][inst])
+        {
+            e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)(kColsTableBytes + kColsMaxBlocks * 16));
+            if(e != hipSuccess)
+                return e;
+            raised[a.device_id][inst] = true;
+        }
+        hipLaunchKernelGGL(kernel, grid, block, lds, stream, c);
         return hipGetLastError();
     }
 
