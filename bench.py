@@ -8,7 +8,7 @@ A step is one pass of the hot path over one batch of synthetic input that is alr
 in HBM.  The primary workload (default ``quant``) fills ``value``; the other workloads of the
 path are timed briefly as well and reported under ``also`` in the same JSON line.
 
-Workloads (BASELINE.json configs):
+Workloads (the benchmark configurations):
   quant    config 2  x bf16 [16384,7168] (1 % channels x50) -> fp8 + fp32 scales, HBM-bound
   prefill  config 4  blockscale GEMM M=8192 N=36864 K=7168, MFMA-bound
   decode   config 3  blockscale GEMM M=64 N=24576 K=1536 (the largest decode shape)

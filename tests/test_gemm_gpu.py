@@ -47,7 +47,7 @@ def assert_close_to_f64(out, xq, wq, xs, ws, what=""):
 
 
 def test_config1_plumbing():
-    # BASELINE config 1: [32,1024] x [512,1024]^T, seed 0
+    # benchmark config 1: [32,1024] x [512,1024]^T, seed 0
     xq, wq, xs, ws = make_problem(32, 512, 1024, seed=0)
     out = run_gpu(xq, wq, xs, ws)
     assert out.shape == (32, 512) and out.dtype == torch.bfloat16
@@ -306,7 +306,7 @@ def test_decode_split_k_repeated_calls_leave_tickets_clean():
 @pytest.mark.parametrize("m", [1, 16, 64])
 @pytest.mark.parametrize("n,k", [(7168, 2048), (24576, 1536), (2112, 7168)])
 def test_decode_shapes(m, n, k):
-    # BASELINE config 3
+    # benchmark config 3
     xq, wq, xs, ws = make_problem(m, n, k, seed=m + n)
     out = run_gpu(xq, wq, xs, ws)
     ref32 = tr.gemm_a8w8_blockscale_ref(xq, wq, xs, ws)
@@ -315,7 +315,7 @@ def test_decode_shapes(m, n, k):
 
 
 def test_fused_config_shape_sampled_rows():
-    # BASELINE config 5 GEMM: [2048,7168] x [4096,7168]^T; 64 sampled rows vs fp32 torch
+    # benchmark config 5 GEMM: [2048,7168] x [4096,7168]^T; 64 sampled rows vs fp32 torch
     m, n, k = 2048, 4096, 7168
     xq, wq, xs, ws = make_problem(m, n, k, seed=0)
     out = run_gpu(xq, wq, xs, ws)
@@ -375,7 +375,7 @@ def test_prefill_kernel_more_tiles_than_compute_units(m, n, k):
 
 @pytest.mark.parametrize("layout", ["plain", "preshuffled"])
 def test_config4_full_size(layout):
-    # BASELINE config 4: M=8192, N=36864, K=7168 through the library's own kernel choice.  Every
+    # benchmark config 4: M=8192, N=36864, K=7168 through the library's own kernel choice.  Every
     # output is compared bit for bit with the generic tile kernel (same products, same order of
     # additions), and 72 rows x all N with the fp64 reference on the CPU: two rows out of each of the
     # 32 tiles of 256 rows, 96 rows apart (another 64-row wave quarter and the other 32-row half of
@@ -412,7 +412,7 @@ def test_config4_full_size(layout):
     (300, 1000, 1408, "prefill_256x128:s=3"),
     (512, 2112, 2048, "prefill_256x192:s=2"),  # eleven full 192-wide tiles per row of tiles, two scale blocks per wave
     (300, 1000, 1408, "prefill_256x192:s=3"),
-    (2048, 4096, 7168, ""),                    # BASELINE config 5's GEMM: the library's own choice (2 ranges)
+    (2048, 4096, 7168, ""),                    # benchmark config 5's GEMM: the library's own choice (2 ranges)
 ])
 def test_prefill_kernel_k_ranges_across_workgroups(m, n, k, name):
     xq, wq, xs, ws = _gpu_problem(m, n, k, seed=m + n + k, outliers=True)

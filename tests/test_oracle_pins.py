@@ -90,7 +90,7 @@ def _check_quant(x, in_dtype="bf16", group=128):
 
 
 def test_quant_config1_matches_torch_restatement():
-    # BASELINE config 1
+    # benchmark config 1
     _check_quant(tr.make_activation(32, 1024, seed=0))
 
 
@@ -186,7 +186,7 @@ def _problem(m, n, k, seed=0):
 
 
 def test_gemm_matches_textbook_fp64_and_torch_linear():
-    xq, wq, xs, ws = _problem(32, 512, 1024)  # BASELINE config 1
+    xq, wq, xs, ws = _problem(32, 512, 1024)  # benchmark config 1
     o, ob = co.gemm_blockscale(co.codes8(xq), co.codes8(wq), xs.numpy(), ws.numpy())
     ref64 = tr.gemm_a8w8_blockscale_ref_f64(xq, wq, xs, ws)
     assert np.array_equal(o, ref64.float().numpy())

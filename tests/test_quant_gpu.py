@@ -19,7 +19,7 @@ def hip_quant(x, **kw):
 
 
 def test_config1_plumbing_matches_torch_reference():
-    # BASELINE config 1: x [32,1024] ~ N(0,1), seed 0
+    # benchmark config 1: x [32,1024] ~ N(0,1), seed 0
     x = tr.make_activation(32, 1024, seed=0)
     y, s = hip_quant(x.to(DEV))
     torch.cuda.synchronize()
@@ -193,7 +193,7 @@ def test_guard_bands_untouched():
 
 
 def test_full_size_properties():
-    # BASELINE config 2 at full size: [16384, 7168] with 1 % outlier channels.  Too big for the
+    # benchmark config 2 at full size: [16384, 7168] with 1 % outlier channels.  Too big for the
     # scalar oracle in seconds, so check 64 sampled rows bit-exactly plus size-independent
     # properties on everything: scale == amax/448 and the amax element encodes +-448.
     x = tr.make_activation(16384, 7168, seed=0, outlier_frac=0.01)

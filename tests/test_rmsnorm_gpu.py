@@ -17,7 +17,7 @@ DEV = "cuda:0"
 def make_norm_inputs(m, k, seed):
     x = tr.make_activation(m, k, seed=seed)
     g = torch.Generator().manual_seed(seed + 100)
-    w = (torch.rand(k, generator=g) + 0.5).bfloat16()  # U(0.5, 1.5), BASELINE config 5
+    w = (torch.rand(k, generator=g) + 0.5).bfloat16()  # U(0.5, 1.5), benchmark config 5
     return x, w
 
 
@@ -76,7 +76,7 @@ def test_gemma_norm_uses_one_plus_weight():
 
 @pytest.mark.parametrize("m,k,group", [(2048, 7168, 128), (3, 256, 128), (40, 8192, 128), (12, 1024, 64), (12, 1024, 32)])
 def test_fused_equals_unfused_bitwise(m, k, group):
-    # BASELINE config 5: fused norm+quant must equal norm -> bf16 -> quant exactly
+    # benchmark config 5: fused norm+quant must equal norm -> bf16 -> quant exactly
     x, w = make_norm_inputs(m, k, seed=7)
     xd, wd = x.to(DEV), w.to(DEV)
     yf, sf = gpu_rmsnorm_quant(xd, wd, 1e-6, group)
