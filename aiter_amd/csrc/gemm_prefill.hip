@@ -593,7 +593,7 @@ PrefillPlan gemm_prefill_plan(const GemmKernelParams& p, int cus)
 
 template <int NW>
 static hipError_t launch_prefill_nw(const GemmKernelParams& p, In16 out_dtype, const LaunchCtx& ctx, int splits,
-                                    int device, int cus)
+                                    bool splits_chosen_here, int device, int cus)
 {
     constexpr int     kBN    = tile_n(NW);
     const hipStream_t stream = ctx.stream;
@@ -621,6 +621,10 @@ static hipError_t launch_prefill_nw(const GemmKernelParams& p, In16 out_dtype, c
     // workgroups walk the tiles.  A multiple of 8 keeps a workgroup's tiles on one XCD's patch order.
     const int total = tiles_m * tiles_n;
     if(total * splits > 4096) // 32-bit byte offsets into the parked tiles
+        splits = 1;
+    // a caller that may not allocate gets one K range per tile where the library's own choice of more
+    // would not fit the fixed buffer (a count asked for by name is an error there instead)
+    if(ctx.static_only && splits_chosen_here && (size_t)total * splits * (4 * NW) * 512 * 16 > kStaticPartialBytes)
         splits = 1;
     splits                 = std::max(1, std::min(splits, (int)p.kblocks));
     const int kb_per_split = (p.kblocks + splits - 1) / splits;
@@ -667,9 +671,10 @@ hipError_t launch_gemm_prefill(const GemmKernelParams& p, In16 out_dtype, const 
                            ? want_tile_n
                            : (want_splits > 0 ? 256 : plan.tile_n);
     const int splits = want_splits > 0 ? want_splits : (bn == plan.tile_n ? plan.splits : 1);
-    return bn == 128   ? launch_prefill_nw<4>(p, out_dtype, ctx, splits, device, cus)
-           : bn == 192 ? launch_prefill_nw<6>(p, out_dtype, ctx, splits, device, cus)
-                       : launch_prefill_nw<8>(p, out_dtype, ctx, splits, device, cus);
+    const bool chosen = want_splits <= 0;
+    return bn == 128   ? launch_prefill_nw<4>(p, out_dtype, ctx, splits, chosen, device, cus)
+           : bn == 192 ? launch_prefill_nw<6>(p, out_dtype, ctx, splits, chosen, device, cus)
+                       : launch_prefill_nw<8>(p, out_dtype, ctx, splits, chosen, device, cus);
 }
 
 } // namespace fp8bs
