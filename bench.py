@@ -790,7 +790,7 @@ def main():
             del w3
         also["decode"] = dec
         mid = []
-        for (m, n, k) in [(256, 4096, 7168), (512, 7168, 2048), (1024, 4096, 7168)]:
+        for (m, n, k) in [(256, 4096, 7168), (512, 7168, 2048), (1024, 7168, 2048), (1024, 4096, 7168), (4096, 2112, 7168)]:
             w4 = GemmWorkload("sweep", m, n, k, "sweep")
             w4.rotate_always = True
             w4.setup(torch, dev)
