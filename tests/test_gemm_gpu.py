@@ -5,6 +5,7 @@ import pytest
 import torch
 
 import aiter_amd
+from aiter_amd import _ffi
 from aiter_amd import dtypes
 from oracle import c_oracle as co
 from oracle import torch_ref as tr
@@ -356,6 +357,38 @@ def _check_rows_against_f64(out, xq, wq, xs, ws, rows, what):
     err = (o - ref).abs()
     bad = (err > ATOL + RTOL * ref.abs()).sum().item()
     assert bad == 0, f"{what}: {bad} of {o.numel()} outside rtol=atol=1e-2, max abs err {err.max().item():.4g}"
+
+
+@pytest.mark.parametrize("m,n,k,expect", [
+    (4096, 2112, 1024, "prefill_256x192"),       # eleven full 192-wide tiles per row of tiles, one round
+    (2048, 2112, 7168, "prefill_256x192:s=2"),   # the same tiles with two K ranges each
+    (8192, 2880, 512, "prefill_256x192"),        # 480 tiles on 256 workgroups: a second tile per workgroup
+    (1024, 7168, 2048, "prefill_256x128"),       # half-width tiles where the wide ones cover 112 compute units
+    (200, 24576, 1536, "prefill_256x128"),       # ... with a ragged row of tiles
+])
+def test_narrow_prefill_tiles_as_the_library_chooses_them(m, n, k, expect):
+    assert _ffi.gemm_choice(m, n, k) == expect
+    xq, wq, xs, ws = _gpu_problem(m, n, k, seed=m + n + k, outliers=True)
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, xs, ws, out, splitK=-1)
+    tile = torch.empty_like(out)
+    aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, xs, ws, tile, kernelName="tile_128x128")
+    torch.cuda.synchronize()
+    if ":s=" in expect:  # K ranges regroup the fp32 additions
+        assert (out.view(torch.int16) != tile.view(torch.int16)).float().mean().item() < 0.02
+    else:               # same products, same order over K blocks: same bits as the generic kernel
+        assert torch.equal(out.view(torch.int16), tile.view(torch.int16))
+    rows = torch.tensor(sorted({r for r in (0, 15, 16, 63, 64, 255, 256, m // 2, m - 1) if r < m}), device=DEV)
+    _check_rows_against_f64(out, xq, wq, xs, ws, rows, f"{expect} {m}x{n}x{k}")
+    # pre-shuffled weights: the same kernel on the other layout gives the same bits
+    wsh = aiter_amd.shuffle_weight(wq.view(torch.uint8)).view(wq.dtype)
+    pre = torch.empty_like(out)
+    aiter_amd.gemm_a8w8_blockscale_bpreshuffle_ck(xq, wsh, xs.t().contiguous().view(*xs.shape), ws, pre,
+                                                  kernelName=expect)
+    named = torch.empty_like(out)
+    aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, xs, ws, named, splitK=-1, kernelName=expect)
+    torch.cuda.synchronize()
+    assert torch.equal(pre.view(torch.int16), named.view(torch.int16))
 
 
 @pytest.mark.parametrize("m,n,k", [(4352, 4096, 256), (4352, 4352, 128), (4100, 4360, 256)])
