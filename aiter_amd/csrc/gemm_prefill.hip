@@ -544,8 +544,9 @@ static float plan_cost(const GemmKernelParams& p, int cus, int bn, int s)
     if(bn == 128)
         return (float)rounds * (kFixed128 + (float)kb * (kIter128 + (share > 0.44f ? (share - 0.44f) * 0.35f : 0.f)));
     if(bn == 192) // 56 KiB and 24 MFMA slots per K block: 1.4 us (4096 x 2112 x 7168, 176 workgroups: 86.9 us;
-                  // 2048 x 2112 x 7168 as 88 tiles x 2 K ranges: 60.3 us against 73.1 with the wide tile)
-        return (float)rounds * (7.f + (float)kb * 1.4f) +
+                  // 2048 x 2112 x 7168 as 88 tiles x 2 K ranges: 60.3 us against 73.1 with the wide tile),
+                  // 1.5 us with a workgroup on every compute unit (8192 x 1536 x 7168, 256 tiles: 93 us)
+        return (float)rounds * (7.f + (float)kb * (1.4f + (share > 0.75f ? (share - 0.75f) * 0.4f : 0.f))) +
                (s > 1 ? 4.f + (float)tiles * (float)(2 * s - 1) * 0.0375f : 0.f);
     const float iter = 1.36f + (share > 0.44f ? (share - 0.44f) * 0.77f : 0.f);
     return (float)rounds * (8.f + (float)kb * iter) +
@@ -574,12 +575,16 @@ PrefillPlan gemm_prefill_plan(const GemmKernelParams& p, int cus)
         if(c < best.us * 0.97f)
             best = PrefillPlan{1, c, 128};
     }
-    // 192-wide tiles where they divide N and 256-wide ones do not (N = 2112: a ninth column of tiles
-    // that is three quarters empty against eleven full ones)
-    if(p.N % 192 == 0 && p.N % 256 != 0)
+    // 192-wide tiles where they divide N: no ragged last column where 256 does not divide it (N = 2112: a
+    // ninth column of tiles that is three quarters empty against eleven full ones), and a better
+    // fit of whole rounds where both do (1024 x 24576 x 1536: 512 tiles in two full rounds, 48 us,
+    // against 384 wide ones in one and a half, 59 us; 512 x 24576 x 1536: 26 us against 32;
+    // 2048 x 4608 x 7168: 192 tiles, 88 us, against 144 wide ones, 100 us).  At most two K ranges:
+    // three (2048 x 1536 x 7168, 64 tiles) take 53 us where the model says 50 and mid_128x128 needs 49.
+    if(p.N % 192 == 0)
     {
         const int t192 = ((p.M + kBM - 1) / kBM) * (p.N / 192);
-        for(int s = 1; s <= 3; ++s)
+        for(int s = 1; s <= 2; ++s)
         {
             if(s > 1 && (t192 < 64 || t192 * s > cus || p.kblocks / s < 8)) // (as above: few tiles, model off)
                 break;

@@ -53,23 +53,23 @@ def test_two_launch_kernel_family_and_named_splits():
 
 
 def test_own_choice_of_k_ranges_fits_the_buffer():
-    # the library's own choice for this shape is two K ranges per 256 x 256 tile: 72 tiles x 2 x 256 KiB of
+    # the library's own choice for this shape is two K ranges per 256 x 192 tile: 96 tiles x 2 x 192 KiB of
     # parked accumulators, more than the fixed buffer's 32 MiB; the entry point that may not allocate then
     # keeps a tile in one workgroup (the named kernel's result, bit for bit) instead of failing
     m, n, k = 2048, 2304, 7168
-    assert _ffi.gemm_choice(m, n, k) == "prefill_256x256:s=2"
+    assert _ffi.gemm_choice(m, n, k) == "prefill_256x192:s=2"
     a = [t.to(DEV) for t in make_problem(m, n, k, seed=74)]
     got = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
     one = torch.empty_like(got)
     two = torch.empty_like(got)
     _ffi.call("gemm_a8w8_blockscale_noalloc", *a, got, -1, "")
-    _ffi.call("gemm_a8w8_blockscale", *a, one, -1, "prefill_256x256")
+    _ffi.call("gemm_a8w8_blockscale", *a, one, -1, "prefill_256x192")
     _ffi.call("gemm_a8w8_blockscale", *a, two, -1, "")
     torch.cuda.synchronize()
     assert torch.equal(got.view(torch.int16), one.view(torch.int16))
     assert (got.view(torch.int16) != two.view(torch.int16)).float().mean().item() < 0.02
     with pytest.raises(RuntimeError, match="32 MiB"):  # asked for by name it is an error
-        _ffi.call("gemm_a8w8_blockscale_noalloc", *a, got, -1, "prefill_256x256:s=2")
+        _ffi.call("gemm_a8w8_blockscale_noalloc", *a, got, -1, "prefill_256x192:s=2")
 
 
 def test_rejects_what_the_buffer_cannot_hold():
