@@ -3,9 +3,9 @@
 //
 // BM (m) x BN (n) output tile per workgroup, 128x128, 64x128 or 64x64, and a number of K ranges,
 // picked together at launch from a small cost model so that every compute unit has work.
-// 4 waves laid out 2 (n) x 2 (m).  Both operand slabs of a K block and
-// the block's x_scale column come in with direct global->LDS loads into a four-stage ring: three
-// K blocks are in flight while one is multiplied.  The 64x64 tile leaves room for two workgroups
+// 4 waves laid out 2 (n) x 2 (m) multiply; 4 more issue the loads.  Both operand slabs of a K
+// block and the block's x_scale column come in with direct global->LDS loads into a four-stage
+// ring: three K blocks are in flight while one is multiplied.  The 64x64 tile leaves room for two workgroups
 // per compute unit; when there are no more workgroups than compute units it runs a six-stage ring
 // instead, filled two K blocks at a time.
 //
@@ -26,7 +26,7 @@ namespace fp8bs {
 
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 512; // four waves that multiply, four that fetch
 constexpr size_t kMaxPartialBytes = (size_t)2 << 30; // what the arenas serve for partial tiles
 
 // s_waitcnt immediate for vmcnt(n) alone (expcnt and lgkmcnt left at their maxima)
@@ -103,9 +103,15 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     const GemmKernelParams& g = p.g;
 
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int l16 = lane & 15, kg = lane >> 4;
-    const int wn = wave & 1, wm = wave >> 1;
+    // Waves 0-3 multiply, waves 4-7 issue the ring's loads.  A wave that issues loads is held at
+    // the issue while the memory pipeline's queue is full (a compute unit takes in about 40 KB/us
+    // from HBM), so a wave that did both would start its LDS reads and MFMAs only after its share
+    // of the next stage had been accepted: fetch and arithmetic of a K block would add up instead
+    // of overlapping (0.19 us of 0.5 us per K block in the 64x64 tile).
+    const int  t = threadIdx.x, lane = t & 63, wave = (t >> 6) & 3;
+    const bool fetches = __builtin_amdgcn_readfirstlane(t >> 8) != 0;
+    const int  l16 = lane & 15, kg = lane >> 4;
+    const int  wn = wave & 1, wm = wave >> 1;
 
     // ---- which tile and K range: workgroups go round-robin over the 8 XCDs, so give each XCD
     // a contiguous run of (split, tile) pairs, tiles m-fastest: neighbours share weight slabs
@@ -198,8 +204,8 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
 
     // ---- w_scale of this wave's BN/2 weight rows (one 128-row block): 64 consecutive K blocks
     // live in one VGPR (lane = K block) and are picked with v_readlane.  The window is a vector
-    // load the compiler waits for with vmcnt(0) at its first use, which also drains the ring of
-    // LDS-direct loads it cannot see: once at the first K block and once every 64 after that.
+    // load the compiler waits for with vmcnt(0) at its first use: in the waves that multiply,
+    // which have no LDS-direct loads of their own in flight.
     uint32_t nb = (uint32_t)(n0 + wn * (BN / 2)) >> 7;
     nb          = min(nb, (uint32_t)((g.N + 127) / 128 - 1));
     const float* ws_row = g.ws + (size_t)nb * g.kblocks;
@@ -248,38 +254,44 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
     // in the previous iteration), refill that previous stage, multiply.
     const int nkb = kb_hi - kb_lo;
     constexpr int kAhead = PAIR ? 4 : kStages - 2; // most stages in flight behind the one waited for
+    if(fetches)
+    {
 #pragma unroll
-    for(int s0 = 0; s0 < (PAIR ? 4 : kStages - 1); ++s0)
-        if(s0 < nkb)
-            fill_stage(s0, kb_lo + s0);
+        for(int s0 = 0; s0 < (PAIR ? 4 : kStages - 1); ++s0)
+            if(s0 < nkb)
+                fill_stage(s0, kb_lo + s0);
+    }
 
     for(int it = 0; it < nkb; ++it)
     {
         const int kb    = kb_lo + it;
         // younger stages already requested
         const int ahead = min(nkb - 1 - it, PAIR ? ((it & 1) ? 4 : 3) : kStages - 2);
-        wait_ahead<kAhead, kLoadsPerStage>(ahead);
+        if(fetches)
+            wait_ahead<kAhead, kLoadsPerStage>(ahead);
         __syncthreads();
-        // (the scale is picked before the refill is issued: where the compiler drains the ring
-        // for the window load, the stage requested below is not yet part of it)
+        if(fetches)
+        {
+            if constexpr(PAIR)
+            {
+                // two K blocks are requested together every other iteration: a weight row's 256
+                // consecutive bytes then reach the memory controller side by side
+                if((it & 1) == 0)
+                {
+                    if(it + 4 < nkb)
+                        fill_stage((it + 4) % kStages, kb + 4);
+                    if(it + 5 < nkb)
+                        fill_stage((it + 5) % kStages, kb + 5);
+                }
+            }
+            else if(it + kStages - 1 < nkb)
+                fill_stage((it + kStages - 1) % kStages, kb + kStages - 1);
+            continue;
+        }
         if((kb & 63) == 0 && it != 0)
             ws_vec = load_ws_window(kb);
         const float wsc = ws_at(kb);
         asm volatile("" ::"s"(wsc));
-        if constexpr(PAIR)
-        {
-            // two K blocks are requested together every other iteration: a weight row's 256
-            // consecutive bytes then reach the memory controller side by side
-            if((it & 1) == 0)
-            {
-                if(it + 4 < nkb)
-                    fill_stage((it + 4) % kStages, kb + 4);
-                if(it + 5 < nkb)
-                    fill_stage((it + 5) % kStages, kb + 5);
-            }
-        }
-        else if(it + kStages - 1 < nkb)
-            fill_stage((it + kStages - 1) % kStages, kb + kStages - 1);
 
         const uint32_t stage = (uint32_t)(it % kStages) * kStageBytes;
         // Fragment reads are volatile so that they stay where they are written: the activation
@@ -321,6 +333,8 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
         for(int j = 0; j < TJ; ++j)
             scp[j] = sc[j];
     }
+    if(fetches)
+        return;
     // drain the two products still in flight (>= 11 wait states after the last MFMA)
     asm volatile("s_nop 15\n s_nop 15\n s_nop 15" ::: "memory");
     fma4_asm(acc[(NQ - 2) / TJ][(NQ - 2) % TJ], P[(NQ - 2) & 3], scp[(NQ - 2) % TJ]);
