@@ -509,12 +509,12 @@ static MidPlan plan_cost(const GemmKernelParams& g, int tile, int splits)
 {
     const int   bm = tile == 128 ? 128 : 64, bn = tile == 64 ? 64 : 128;
     const int   occupancy = tile == 64 ? 2 : 1;
-    const float fixed     = tile == 64 ? 4.5f : tile == 64128 ? 5.7f : 6.9f;
-    const float iter1     = tile == 64 ? 0.07f : tile == 64128 ? 0.08f : 0.12f;
+    const float fixed     = tile == 64 ? 3.8f : tile == 64128 ? 4.7f : 5.5f;
+    const float iter1     = tile == 64 ? 0.f : tile == 64128 ? 0.13f : 0.16f;
     const int   tiles     = ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
     const int   wgs = tiles * splits, slots = 256 * occupancy;
     // (64x64 with a compute unit per workgroup runs the six-stage ring)
-    const float iter0 = tile == 64 ? (wgs <= 256 ? 0.50f : 0.56f) : tile == 64128 ? 0.70f : 0.74f;
+    const float iter0 = tile == 64 ? (wgs <= 256 ? 0.35f : 0.525f) : tile == 64128 ? 0.35f : 0.535f;
     const int   rounds    = (wgs + slots - 1) / slots;
     const float per_cu    = (float)(wgs < slots ? wgs : slots) / 256.f;
     const int   iters     = (g.kblocks + splits - 1) / splits;
@@ -523,7 +523,7 @@ static MidPlan plan_cost(const GemmKernelParams& g, int tile, int splits)
     if(splits > 1)
     {
         // partial tiles written and read back at about 6 TB/s, plus the second launch
-        cost += 3.2f + (float)splits * (float)g.M * (float)g.N * 4.f / 6.0e6f;
+        cost += (tile == 64 ? 3.8f : 3.05f) + (float)splits * (float)g.M * (float)g.N * 4.f / 6.0e6f;
     }
     return MidPlan{tile, splits, cost};
 }

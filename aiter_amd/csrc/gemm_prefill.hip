@@ -523,8 +523,9 @@ bool gemm_prefill_supports(const GemmKernelParams& p)
 
 // Duration model (us) on `cus` compute units, fitted to event timings with weights from HBM:
 // a round of workgroups costs 8 us (first slabs, output tile) plus, per K block, 1.36 us while
-// the workgroups of a round cover up to 44 % of the compute units, rising to 1.79 us when they
-// cover all (8192 x 36864 x 7168: 18 rounds x (8 + 56 x 1.79) = 1948 us, measured 1950).  K
+// the workgroups of a round cover up to 44 % of the compute units, rising to 1.79 us from 62 % on
+// (8192 x 36864 x 7168: 18 rounds x (8 + 56 x 1.79) = 1948 us, measured 1950; 2048 x 4608 x 7168,
+// 144 workgroups: 100 us; 1536 x 7168 x 2048, 168 workgroups: 36 us).  K
 // ranges over s workgroups per tile cost 4 us plus the parked tiles' traffic, (2 s - 1) x 256 KiB
 // per tile at about 5 TB/s (2048 x 4096 x 7168: 89.8 us as one range, 77-80 us as two).
 // 256 x 128 tiles: 6 us per round and 1.2 us per K block, rising to 1.4 us when the workgroups of a round
@@ -548,7 +549,7 @@ static float plan_cost(const GemmKernelParams& p, int cus, int bn, int s)
                   // 1.5 us with a workgroup on every compute unit (8192 x 1536 x 7168, 256 tiles: 93 us)
         return (float)rounds * (7.f + (float)kb * (1.4f + (share > 0.75f ? (share - 0.75f) * 0.4f : 0.f))) +
                (s > 1 ? 4.f + (float)tiles * (float)(2 * s - 1) * 0.0375f : 0.f);
-    const float iter = 1.36f + (share > 0.44f ? (share - 0.44f) * 0.77f : 0.f);
+    const float iter = std::min(1.79f, 1.36f + (share > 0.44f ? (share - 0.44f) * 2.4f : 0.f));
     return (float)rounds * (8.f + (float)kb * iter) +
            (s > 1 ? 4.f + (float)tiles * (float)(2 * s - 1) * 0.05f : 0.f);
 }
@@ -575,15 +576,15 @@ PrefillPlan gemm_prefill_plan(const GemmKernelParams& p, int cus)
         if(c < best.us * 0.97f)
             best = PrefillPlan{1, c, 128};
     }
-    // 192-wide tiles where they divide N: no ragged last column where 256 does not divide it (N = 2112: a
-    // ninth column of tiles that is three quarters empty against eleven full ones), and a better
-    // fit of whole rounds where both do (1024 x 24576 x 1536: 512 tiles in two full rounds, 48 us,
+    // 192-wide tiles: no ragged last column where they divide N and 256 does not (N = 2112: a
+    // ninth column of tiles that is three quarters empty against eleven full ones), and often a better
+    // fit of whole rounds (1024 x 24576 x 1536: 512 tiles in two full rounds, 48 us,
     // against 384 wide ones in one and a half, 59 us; 512 x 24576 x 1536: 26 us against 32;
-    // 2048 x 4608 x 7168: 192 tiles, 88 us, against 144 wide ones, 100 us).  At most two K ranges:
+    // 2048 x 4608 x 7168: 192 tiles, 88 us, against 144 wide ones, 100 us; 1536 x 7168 x 2048: 228
+    // tiles, the last column a third full, 30 us against 36).  At most two K ranges:
     // three (2048 x 1536 x 7168, 64 tiles) take 53 us where the model says 50 and mid_128x128 needs 49.
-    if(p.N % 192 == 0)
     {
-        const int t192 = ((p.M + kBM - 1) / kBM) * (p.N / 192);
+        const int t192 = ((p.M + kBM - 1) / kBM) * ((p.N + 191) / 192);
         for(int s = 1; s <= 2; ++s)
         {
             if(s > 1 && (t192 < 64 || t192 * s > cus || p.kblocks / s < 8)) // (as above: few tiles, model off)

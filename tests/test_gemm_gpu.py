@@ -363,6 +363,7 @@ def _check_rows_against_f64(out, xq, wq, xs, ws, rows, what):
     (4096, 2112, 1024, "prefill_256x192"),       # eleven full 192-wide tiles per row of tiles, one round
     (2048, 2112, 7168, "prefill_256x192:s=2"),   # the same tiles with two K ranges each
     (8192, 2880, 512, "prefill_256x192"),        # 480 tiles on 256 workgroups: a second tile per workgroup
+    (1536, 7168, 2048, "prefill_256x192"),       # 192 does not divide N: the last column of tiles is a third full
     (1024, 7168, 2048, "prefill_256x128"),       # half-width tiles where the wide ones cover 112 compute units
     (200, 24576, 1536, "prefill_256x128"),       # ... with a ragged row of tiles
 ])
