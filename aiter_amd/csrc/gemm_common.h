@@ -99,6 +99,7 @@ bool       gemm_prefill_supports(const GemmKernelParams& p);
 hipError_t launch_gemm_decode(const GemmKernelParams& p, In16 out_dtype, int split_k_log2, const LaunchCtx& ctx,
                               const char* tuning = nullptr);
 bool       gemm_decode_supports(const GemmKernelParams& p);
+float      gemm_decode_estimate_us(const GemmKernelParams& p);
 hipError_t launch_gemm_mid(const GemmKernelParams& p, In16 out_dtype, int split_k_log2, const LaunchCtx& ctx,
                            int tile = 0, int splits = 0);
 bool       gemm_mid_supports(const GemmKernelParams& p);

@@ -690,20 +690,27 @@ bool gemm_decode_supports(const GemmKernelParams& p)
     return p.M >= 1 && p.M <= kDecodeMaxM && p.kblocks >= 1;
 }
 
+// How a problem is split over workgroups and waves.
+struct DecodePlan
+{
+    int  mt;       // m tiles a wave holds at a time
+    int  rows;     // 16-row weight tiles per group
+    int  n_tiles, n_groups, steps;
+    int  splits, steps_per_split, waves;
+    bool single;   // one step per wave covers the workgroup's K range
+    bool full;
+    int  m_chunks, grid_x;
+};
+
 // split_k_log2 < 0: choose.  Otherwise 2^split_k_log2 K ranges (rounded to whole steps).
 // `tuning` may override the choices: "r=<row tiles per group>,s=<K ranges>,w=<waves>,g=<grid.x>".
-hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int split_k_log2, const LaunchCtx& ctx,
-                              const char* tuning)
+static DecodePlan plan_decode(const GemmKernelParams& g, int split_k_log2, const char* tuning)
 {
-    const hipStream_t stream = ctx.stream;
-    DecodeParams p{};
-    p.g           = g;
-    p.bf16_out    = out_dtype == In16::bf16 ? 1 : 0;
-    p.n_tiles     = (g.N + 15) / 16;
-    p.xs_vec4     = (g.xs_k == 1 && (g.xs_m & 3) == 0 && ((uintptr_t)g.xs & 15) == 0) ? 1 : 0;
-    int       mt        = g.M > 64 ? 4 : (g.M + 15) / 16; // m tiles a wave holds at a time
+    DecodePlan d{};
+    d.n_tiles           = (g.N + 15) / 16;
+    d.mt                = g.M > 64 ? 4 : (g.M + 15) / 16;
     const int max_waves = 4;
-    const int steps     = (g.kblocks + kStepKb - 1) / kStepKb;
+    d.steps             = (g.kblocks + kStepKb - 1) / kStepKb;
     const int kChipCus  = 256;
 
     // Two row tiles per group halve the activation traffic and double what a wave keeps in
@@ -711,10 +718,10 @@ hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int spl
     // than anything else).  Up to 32 rows single tiles are faster at every N measured, walked two
     // or three to a workgroup with the next tile's weights already requested ((1, 7168, 2048):
     // 5.8 us against 6.2, (1, 24576, 1536): 9.4 against 10.4, (32, 24576, 1536): 11.1 against 12.2).
-    int rows = tuning_value(tuning, "r");
-    if(rows != 1 && rows != 2)
-        rows = mt >= 3 ? 2 : 1;
-    p.n_groups = (p.n_tiles + rows - 1) / rows;
+    d.rows = tuning_value(tuning, "r");
+    if(d.rows != 1 && d.rows != 2)
+        d.rows = d.mt >= 3 ? 2 : 1;
+    d.n_groups = (d.n_tiles + d.rows - 1) / d.rows;
 
     int splits = tuning_value(tuning, "s");
     if(splits <= 0)
@@ -725,52 +732,93 @@ hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int spl
         {
             // Split K across workgroups only while every workgroup still gets a compute unit of
             // its own (one workgroup fills a compute unit's registers) and at least two steps.
-            splits = kChipCus / p.n_groups;
-            if(splits > steps / 2)
-                splits = steps / 2;
+            splits = kChipCus / d.n_groups;
+            if(splits > d.steps / 2)
+                splits = d.steps / 2;
             if(splits < 1)
                 splits = 1;
         }
     }
-    if(splits > steps)
-        splits = steps;
-    int steps_per_split = (steps + splits - 1) / splits;
-    splits              = (steps + steps_per_split - 1) / steps_per_split;
-    p.kb_per_split      = steps_per_split * kStepKb;
-    p.splits            = splits;
+    if(splits > d.steps)
+        splits = d.steps;
+    d.steps_per_split = (d.steps + splits - 1) / splits;
+    d.splits          = (d.steps + d.steps_per_split - 1) / d.steps_per_split;
 
-    int waves = tuning_value(tuning, "w");
-    if(waves <= 0 || waves > max_waves)
-        waves = steps_per_split < max_waves ? steps_per_split : max_waves;
-    const bool single = steps_per_split <= waves;
-    const bool full   = (g.kblocks % kStepKb) == 0;
+    d.waves = tuning_value(tuning, "w");
+    if(d.waves <= 0 || d.waves > max_waves)
+        d.waves = d.steps_per_split < max_waves ? d.steps_per_split : max_waves;
+    d.single = d.steps_per_split <= d.waves;
+    d.full   = (g.kblocks % kStepKb) == 0;
     // more than 64 rows are walked in chunks: 32 rows at a time when the weights stay in registers
     // across chunks (that path also stages the next chunk), else 64
-    if(g.M > 64 && single)
-        mt = 2;
-    p.m_chunks = g.M > 64 ? (g.M + mt * 16 - 1) / (mt * 16) : 1;
+    if(g.M > 64 && d.single)
+        d.mt = 2;
+    d.m_chunks = g.M > 64 ? (g.M + d.mt * 16 - 1) / (d.mt * 16) : 1;
 
     int gx = tuning_value(tuning, "g");
     if(gx <= 0)
     {
-        gx = p.n_groups;
-        if(single && rows == 1 && mt <= 2 && splits == 1 && p.n_groups >= 2 * (kChipCus - kChipCus / 8))
+        gx = d.n_groups;
+        if(d.single && d.rows == 1 && d.mt <= 2 && d.splits == 1 && d.n_groups >= 2 * (kChipCus - kChipCus / 8))
         {
             // single tiles, short K: at least two tiles per workgroup, at most two workgroups per
             // compute unit at a time
-            int iters = (p.n_groups + 2 * kChipCus - 1) / (2 * kChipCus);
+            int iters = (d.n_groups + 2 * kChipCus - 1) / (2 * kChipCus);
             iters     = iters < 2 ? 2 : iters;
-            gx        = (p.n_groups + iters - 1) / iters;
+            gx        = (d.n_groups + iters - 1) / iters;
         }
-        else if(single && p.n_groups * splits > 2 * kChipCus)
+        else if(d.single && d.n_groups * d.splits > 2 * kChipCus)
         {
-            const int per_split = (kChipCus + splits - 1) / splits;
-            const int iters     = (p.n_groups + per_split - 1) / per_split;
-            gx                  = (p.n_groups + iters - 1) / iters;
+            const int per_split = (kChipCus + d.splits - 1) / d.splits;
+            const int iters     = (d.n_groups + per_split - 1) / per_split;
+            gx                  = (d.n_groups + iters - 1) / iters;
         }
     }
-    if(gx > p.n_groups)
-        gx = p.n_groups;
+    d.grid_x = gx > d.n_groups ? d.n_groups : gx;
+    return d;
+}
+
+// Rough duration (us) of the launch this file would choose, fitted per regime (one K step per
+// workgroup; one step per wave; several steps per wave) to event timings of M = 16 ... 64 on
+// fourteen weight shapes from 1.8 MB to 117 MB coming from HBM (about 10 % off on average).  Terms:
+// the weights over the share of the chip the workgroups cover, the activation re-reads, the MFMA
+// work (m tiles x weights), the parked partial tiles and the output.  Only used to decide between
+// this kernel and the mid_* family.
+float gemm_decode_estimate_us(const GemmKernelParams& g)
+{
+    const DecodePlan d = plan_decode(g, -1, nullptr);
+    const float mb    = 1e-6f;
+    const float w     = (float)g.N * (float)g.K * mb;
+    const float a     = (float)(d.single ? d.grid_x : d.n_groups) * (float)g.M * (float)g.K * mb;
+    const float wgs   = (float)d.grid_x * (float)d.splits;
+    const float share = std::max(0.05f, std::min(1.f, wgs * (float)d.waves / 4.f / 256.f));
+    const float part  = d.splits > 1 ? (float)d.splits * (float)g.M * (float)g.N * 4.f * mb : 0.f;
+    const float out   = (float)g.M * (float)g.N * 2.f * mb;
+    const float wide_split = (d.mt >= 3 && d.splits > 1) ? (float)d.splits : 0.f;
+    const float mt    = (float)d.mt;
+    if(d.waves == 1)
+        return 2.53f + 0.096f * w / share + 0.028f * mt * w + 0.67f * out + 0.62f * mt;
+    if(d.single)
+        return 3.59f + 0.107f * w / share + 0.038f * mt * w + 2.9f * part + 0.44f * wide_split + 0.10f * mt;
+    return 4.67f + 0.141f * w / share + 0.021f * a + 0.029f * mt * w + 3.78f * out + 0.65f * wide_split + 0.38f * mt;
+}
+
+hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int split_k_log2, const LaunchCtx& ctx,
+                                   const char* tuning)
+{
+    const hipStream_t stream = ctx.stream;
+    DecodeParams p{};
+    p.g           = g;
+    p.bf16_out    = out_dtype == In16::bf16 ? 1 : 0;
+    p.xs_vec4     = (g.xs_k == 1 && (g.xs_m & 3) == 0 && ((uintptr_t)g.xs & 15) == 0) ? 1 : 0;
+    const DecodePlan d = plan_decode(g, split_k_log2, tuning);
+    p.n_tiles      = d.n_tiles;
+    p.n_groups     = d.n_groups;
+    p.kb_per_split = d.steps_per_split * kStepKb;
+    p.splits       = d.splits;
+    p.m_chunks     = d.m_chunks;
+    const int  mt = d.mt, rows = d.rows, splits = d.splits, waves = d.waves, gx = d.grid_x;
+    const bool single = d.single, full = d.full;
 
     const size_t tile_set = (size_t)rows * mt * 64 * 16; // bytes of one group's fp32 tile set
     WorkspaceLock lock(splits > 1);

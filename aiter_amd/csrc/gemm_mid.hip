@@ -493,8 +493,10 @@ bool gemm_mid_supports(const GemmKernelParams& p)
            (uint64_t)p.M * (uint64_t)p.lda < (1ull << 32) && (uint64_t)p.M * (uint64_t)p.kblocks < (1ull << 30);
 }
 
-// Rough duration (us) of one tiling on a 256-CU part, fitted to in-kernel timelines on the
-// DeepSeek-V3 projection shapes with the weights coming from HBM.  A launch costs a fixed share
+// Rough duration (us) of one tiling on a 256-CU part, fitted to event timings of every tiling and
+// K range count at M = 16 ... 1536 on the DeepSeek-V3 projection shapes and nine more, with the
+// weights coming from HBM (9 % off on average; the tiling it picks is 1 % slower than the best one
+// on average).  A launch costs a fixed share
 // (first wave running, first stage landing: about 2 us from HBM, output stores draining, end of
 // kernel) plus an iteration per K block whose cost is set by what a compute unit can pull in
 // (about 40 KB/us, so it hardly depends on how many workgroups run).  K ranges beyond the first
@@ -509,21 +511,28 @@ static MidPlan plan_cost(const GemmKernelParams& g, int tile, int splits)
 {
     const int   bm = tile == 128 ? 128 : 64, bn = tile == 64 ? 64 : 128;
     const int   occupancy = tile == 64 ? 2 : 1;
-    const float fixed     = tile == 64 ? 3.8f : tile == 64128 ? 4.7f : 5.5f;
-    const float iter1     = tile == 64 ? 0.f : tile == 64128 ? 0.13f : 0.16f;
-    const int   tiles     = ((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn);
+    const float fixed     = tile == 64 ? 3.1f : tile == 64128 ? 3.67f : 4.31f;
+    const float iter1     = tile == 64 ? 0.f : tile == 64128 ? 0.075f : 0.128f;
+    // a single row of tiles (M <= BM): no second workgroup asks for the same weight slab
+    const float solo      = tile == 64 ? 0.049f : tile == 64128 ? 0.12f : 0.f;
+    const int   tiles_m   = (g.M + bm - 1) / bm;
+    const int   tiles     = tiles_m * ((g.N + bn - 1) / bn);
     const int   wgs = tiles * splits, slots = 256 * occupancy;
     // (64x64 with a compute unit per workgroup runs the six-stage ring)
-    const float iter0 = tile == 64 ? (wgs <= 256 ? 0.35f : 0.525f) : tile == 64128 ? 0.35f : 0.535f;
+    const float iter0 = tile == 64 ? (wgs <= 256 ? 0.367f : 0.535f) : tile == 64128 ? 0.422f : 0.555f;
     const int   rounds    = (wgs + slots - 1) / slots;
     const float per_cu    = (float)(wgs < slots ? wgs : slots) / 256.f;
     const int   iters     = (g.kblocks + splits - 1) / splits;
-    float       cost      = fixed + (float)rounds * (float)iters * (iter0 + iter1 * per_cu) +
-                 (float)(rounds - 1) * (fixed - 2.4f);
+    float       iter      = iter0 + (iter1 + (tiles_m == 1 ? solo : 0.f)) * per_cu;
+    if(!g.w_shuffled && (g.ldb & 8191) == 0) // weight rows 8 KiB apart or a multiple: every row of a slab on the same channels
+        iter *= 1.35f;
+    float cost = fixed + (float)rounds * (float)iters * iter + (float)(rounds - 1) * (fixed - 2.4f);
     if(splits > 1)
     {
-        // partial tiles written and read back at about 6 TB/s, plus the second launch
-        cost += (tile == 64 ? 3.8f : 3.05f) + (float)splits * (float)g.M * (float)g.N * 4.f / 6.0e6f;
+        // the second launch, and the partial tiles written and read back
+        const float launch = tile == 64 ? 2.19f : tile == 64128 ? 1.78f : 1.97f;
+        const float rate   = tile == 128 ? 2.92e6f : 2.0e6f; // bytes per us
+        cost += launch + (float)splits * (float)g.M * (float)g.N * 4.f / rate;
     }
     return MidPlan{tile, splits, cost};
 }

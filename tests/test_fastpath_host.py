@@ -36,7 +36,10 @@ def test_kernel_choice_query_on_the_headline_shapes():
     names = set(aiter_amd.gemm_kernel_names())
     for m in (1, 16, 64):
         for n, k in ((7168, 2048), (24576, 1536), (2112, 7168)):
-            assert aiter_amd.get_CKGEMM_config(m, n, k)["kernelName"] == "decode_stream"
+            # the weight-streaming kernel up to 16 rows; at 64 rows only where N / 32 row groups with one K
+            # step per wave cover the chip, elsewhere the mid_* tilings are modelled (and measured) faster
+            want = "decode_stream" if m <= 16 or (n, k) == (7168, 2048) else "mid_"
+            assert aiter_amd.get_CKGEMM_config(m, n, k)["kernelName"].startswith(want)
     assert aiter_amd.get_CKGEMM_config(8192, 36864, 7168)["kernelName"] == "prefill_256x256"
     cfg5 = aiter_amd.get_CKGEMM_config(2048, 4096, 7168)  # 128 tiles: two K ranges per tile
     assert cfg5["kernelName"] == "prefill_256x256:s=2" and cfg5["kRanges"] == 2
