@@ -333,12 +333,50 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
         for(int j = 0; j < TJ; ++j)
             scp[j] = sc[j];
     }
-    if(fetches)
+    // One K range, 16-byte aligned output rows: the tile goes through LDS so that all eight waves
+    // store whole 128-byte (or longer) row segments, 16 bytes per lane; otherwise the waves that
+    // multiplied store their fragments as they hold them (8 bytes per lane, 32 per row and instruction).
+    const bool staged = p.splits == 1 && (g.N & 7) == 0 && ((uintptr_t)g.out & 15) == 0;
+    if(fetches && !staged)
         return;
-    // drain the two products still in flight (>= 11 wait states after the last MFMA)
-    asm volatile("s_nop 15\n s_nop 15\n s_nop 15" ::: "memory");
-    fma4_asm(acc[(NQ - 2) / TJ][(NQ - 2) % TJ], P[(NQ - 2) & 3], scp[(NQ - 2) % TJ]);
-    fma4_asm(acc[(NQ - 1) / TJ][(NQ - 1) % TJ], P[(NQ - 1) & 3], scp[(NQ - 1) % TJ]);
+    if(!fetches)
+    {
+        // drain the two products still in flight (>= 11 wait states after the last MFMA)
+        asm volatile("s_nop 15\n s_nop 15\n s_nop 15" ::: "memory");
+        fma4_asm(acc[(NQ - 2) / TJ][(NQ - 2) % TJ], P[(NQ - 2) & 3], scp[(NQ - 2) % TJ]);
+        fma4_asm(acc[(NQ - 1) / TJ][(NQ - 1) % TJ], P[(NQ - 1) & 3], scp[(NQ - 1) % TJ]);
+    }
+    if(staged)
+    {
+        constexpr int kPitch = BN * 2 + 16; // bytes between two rows of the staged tile
+        static_assert(BM * kPitch <= S::kSmem, "the staged tile takes the ring's place");
+        __syncthreads(); // every wave is done with the ring's last stage
+        if(!fetches)
+        {
+#pragma unroll
+            for(int j = 0; j < TJ; ++j)
+#pragma unroll
+                for(int i = 0; i < TI; ++i)
+                {
+                    const float(&a)[4] = acc[i][j];
+                    const u32x2 o = p.bf16_out ? u32x2{pack2<In16::bf16>(a[0], a[1]), pack2<In16::bf16>(a[2], a[3])}
+                                               : u32x2{pack2<In16::fp16>(a[0], a[1]), pack2<In16::fp16>(a[2], a[3])};
+                    const int r = wm * (BM / 2) + j * 16 + l16, c = wn * (BN / 2) + i * 16 + kg * 4;
+                    *(u32x2*)(smem + r * kPitch + c * 2) = o;
+                }
+        }
+        __syncthreads();
+        constexpr int kChunks = BN / 8, kRowsPerPass = kThreads / kChunks; // 16-byte chunks per row
+#pragma unroll
+        for(int r0 = 0; r0 < BM; r0 += kRowsPerPass)
+        {
+            const int r = r0 + t / kChunks, c = t % kChunks;
+            const int m = m0 + r, n = n0 + c * 8;
+            if(m < g.M && n < g.N) // N is a multiple of 8: the chunk is inside the row
+                *(u32x4*)(g.out + (size_t)m * g.N + n) = *(const u32x4*)(smem + r * kPitch + c * 16);
+        }
+        return;
+    }
 
     // ---- epilogue: lane owns out[m][n .. n+3] for each of its TI x TJ tiles
     auto store_tile = [&](int i, int j, const float(&a)[4]) {
