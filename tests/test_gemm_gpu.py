@@ -315,6 +315,25 @@ def test_decode_shapes(m, n, k):
     assert_close_to_f64(out, xq, wq, xs, ws, f"decode {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("m,n,k", [(17, 24576, 1536), (40, 2112, 7168), (64, 576, 7168), (33, 32768, 512), (8, 32768, 512)])
+def test_small_batches_that_the_library_sends_to_the_mid_tilings(m, n, k):
+    # below 65 rows the choice between the weight-streaming kernel and the mid_* tilings is by modelled
+    # duration; these go to the tilings (one 64-row tile, mostly padding rows that are never stored)
+    assert _ffi.gemm_choice(m, n, k).startswith("mid_")
+    xq, wq, xs, ws = make_problem(m, n, k, seed=m + n + k)
+    out = run_gpu(xq, wq, xs, ws)
+    assert_close_to_f64(out, xq, wq, xs, ws, f"small batch {m}x{n}x{k}")
+    dev = [t.to(DEV) for t in (xq, wq, xs, ws)]
+    stream = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    aiter_amd.gemm_a8w8_blockscale_ck(*dev, stream, splitK=-1, kernelName="decode_stream")
+    # same products, fp32 sums grouped differently: a few results round to the neighbouring 16-bit value
+    assert (out.to(DEV).view(torch.int16) != stream.view(torch.int16)).float().mean().item() < 0.05
+    wsh = aiter_amd.shuffle_weight(dev[1].view(torch.uint8)).view(dev[1].dtype)
+    assert _ffi.gemm_choice(m, n, k, True).startswith("mid_")
+    pre = aiter_amd.gemm_a8w8_blockscale_bpreshuffle(dev[0], wsh, dev[2].t().contiguous().t(), dev[3])
+    assert torch.equal(pre.view(torch.int16), out.to(DEV).view(torch.int16))
+
+
 def test_fused_config_shape_sampled_rows():
     # benchmark config 5 GEMM: [2048,7168] x [4096,7168]^T; 64 sampled rows vs fp32 torch
     m, n, k = 2048, 4096, 7168
