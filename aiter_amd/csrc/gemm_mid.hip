@@ -583,7 +583,8 @@ static MidPlan best_plan(const GemmKernelParams& g, int tile)
     {
         if(tile != 0 && t != tile)
             continue;
-        const int max_splits = can_split ? (g.kblocks / 4 < 16 ? g.kblocks / 4 : 16) : 1;
+        // (more than eight K ranges never measured best; the model is not fitted beyond)
+        const int max_splits = can_split ? (g.kblocks / 4 < 8 ? g.kblocks / 4 : 8) : 1;
         for(int sp = 1; sp <= (max_splits < 1 ? 1 : max_splits); ++sp)
         {
             const MidPlan c = plan_cost(g, t, sp);
