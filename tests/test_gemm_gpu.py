@@ -236,6 +236,28 @@ def test_mid_kernel(kernel, m, n, k, splitk):
         assert (out.view(torch.int16) != tile.view(torch.int16)).float().mean().item() < 0.02
 
 
+@pytest.mark.parametrize("kernel", ["mid_64x64:s=1", "mid_64x128:s=1", "mid_128x128:s=1"])
+@pytest.mark.parametrize("m,n,dtype,shift", [
+    (130, 520, torch.float16, 0),   # rows 16-byte aligned: the tile goes through LDS and all eight waves store it
+    (130, 260, torch.bfloat16, 0),  # rows 8-byte aligned only: the multiplying waves store their fragments
+    (70, 1002, torch.bfloat16, 0),  # rows 4-byte aligned: element-wise stores at the ragged edge
+    (70, 520, torch.bfloat16, 4),   # 16-byte aligned rows behind a base that is not: fragment stores again
+])
+def test_mid_kernel_output_paths(kernel, m, n, dtype, shift):
+    k = 384
+    xq, wq, xs, ws = make_problem(m, n, k, seed=m + n)
+    a = [t.to(DEV) for t in (xq, wq, xs, ws)]
+    flat = torch.full((m * n + 64,), float("nan"), dtype=dtype, device=DEV)
+    out = flat[shift : shift + m * n].view(m, n)
+    aiter_amd.gemm_a8w8_blockscale_ck(*a, out, splitK=0, kernelName=kernel)
+    torch.cuda.synchronize()
+    assert_close_to_f64(out, xq, wq, xs, ws, f"{kernel} {m}x{n} {dtype} +{shift}")
+    assert torch.isnan(flat[:shift]).all() and torch.isnan(flat[shift + m * n :]).all()  # nothing outside the matrix
+    base = torch.empty(m, n, dtype=dtype, device=DEV)
+    aiter_amd.gemm_a8w8_blockscale_ck(*a, base, splitK=0, kernelName="tile_128x128")
+    assert torch.equal(out.view(torch.int16), base.view(torch.int16))
+
+
 @pytest.mark.parametrize("kblocks", [1, 2, 3, 4, 5, 6, 7, 8, 9, 11, 12, 13, 18])
 def test_mid_64x64_lone_workgroups_every_k_length(kblocks):
     # no more workgroups than compute units: the 64x64 tile runs its six-stage ring, filled two K
