@@ -562,8 +562,10 @@ static MidPlan plan_cost(const GemmKernelParams& g, int tile, int splits)
     const float per_cu    = (float)(wgs < slots ? wgs : slots) / 256.f;
     const int   iters     = (g.kblocks + splits - 1) / splits;
     float       iter      = iter0 + (iter1 + (tiles_m == 1 ? solo : 0.f)) * per_cu;
-    if(!g.w_shuffled && (g.ldb & 8191) == 0) // weight rows 8 KiB apart or a multiple: every row of a slab on the same channels
-        iter *= 1.35f;
+    // row-major weights with long rows: a slab's 128-byte pieces lie further apart (more DRAM pages per K
+    // block); 64x128 tiles on (7168, 16384) and (7168, 16256) take 0.8 us per K block where 7168-byte rows take 0.6
+    if(!g.w_shuffled && g.ldb > 8192)
+        iter *= 1.f + 0.35f * (g.ldb >= 16384 ? 1.f : (float)(g.ldb - 8192) / 8192.f);
     float cost = fixed + (float)rounds * (float)iters * iter + (float)(rounds - 1) * (fixed - 2.4f);
     if(splits > 1)
     {
