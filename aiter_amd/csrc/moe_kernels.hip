@@ -25,6 +25,7 @@
 #include "moe_launch.h"
 
 #include <atomic>
+#include <cmath>
 
 namespace fp8bs {
 
@@ -1392,12 +1393,17 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
     p.activation        = a.activation;
     p.lda               = a.x16 ? a.dim : a.lda;
     {
-        // (expert, block) pairs to expect: every expert that can be hit once, plus the full blocks
-        const int64_t pairs = (int64_t)a.M * a.topk;
-        const int64_t est_blocks = (pairs < a.experts ? pairs : a.experts) + pairs / 32;
-        int           nt = a.gate_tiles;
+        // (expert, block) pairs to expect under a routing that spreads evenly: the experts hit at least once,
+        // plus the full blocks.  Wide units (64 columns; one workgroup per compute unit at a time) where
+        // they cover the chip and their last round is not a nearly empty one; the narrowest otherwise
+        // (DeepSeek-V3 layer, us at 8 / 16 / 24 / 32 tokens: wide 69 / 117 / 161 / 177, narrow 72 / 119 /
+        // 151 / 179, the 32-column units in between or behind both).
+        const double pairs  = (double)a.M * a.topk;
+        const double blocks = (double)a.experts * (1.0 - exp(-pairs / (double)a.experts)) + pairs / 32.0;
+        const double wide   = blocks * (a.inter / 64), rounds = wide / 256.0;
+        int          nt     = a.gate_tiles;
         if(nt != 1 && nt != 2 && nt != 4)
-            nt = est_blocks * (a.inter / 64) >= 1024 ? 4 : est_blocks * (a.inter / 32) >= 1024 ? 2 : 1;
+            nt = (wide >= 230.0 && (rounds <= 1.05 || rounds - floor(rounds) >= 0.4 || rounds >= 4.0)) ? 4 : 1;
         p.n_groups = a.inter / (16 * nt);
         const dim3 grid((unsigned)((size_t)a.max_blocks * p.n_groups));
         switch(nt)
