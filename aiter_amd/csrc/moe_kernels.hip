@@ -536,9 +536,10 @@ __device__ __forceinline__ float activate(float g, int activation)
 }
 
 // First GEMM + activation.  Workgroup = (block of 32 sorted rows, NT x 16 inter columns): NT
-// gate tiles and the NT matching up tiles; NT is picked at launch (small units when few (expert,
-// block) pairs exist, so that the last units to finish do not set the kernel's duration; wide
-// units otherwise, which re-read the activations less often).  The waves take every eighth K
+// gate tiles and the NT matching up tiles; NT is picked at launch (wide units, which re-read the
+// activations less often, where they cover the chip and their last round of workgroups is expected
+// to be reasonably full; the narrowest otherwise, so that the last units to finish do not set the
+// kernel's duration).  The waves take every eighth K
 // block each and add their partial tiles through LDS in wave order.  One operand set per wave:
 // several workgroups share a compute unit and cover each other's load latency.  A block whose
 // second half is padding (the usual case when few tokens are routed) multiplies one 16-row tile
