@@ -858,13 +858,16 @@ __global__ __launch_bounds__(256) void moe_down_long_k_kernel(MoeGemmParams p)
 
 // Second GEMM fused with the per-token sum, for decode-size batches.  Workgroup = two neighbouring
 // 16-column weight tiles of every expert (8 KiB of an expert's weights are contiguous in memory and
-// requested together: 2-3 % faster than one tile, while four tiles leave too few workgroups for
-// the compute units' ingest); a wave multiplies one K block of one tile.  A wave walks the (block, 16-row
-// half) units that hold real pairs, in sorted order, with the next kColsDepth units' operands
-// already requested (a unit is 2 KiB of weights per wave: the depth is what keeps a wave's share
-// of HBM in flight), and adds each weighted product row into its own [tokens][16] fp32 table in
-// LDS: one wave per table and a fixed walk, so the sum is deterministic.  The tables are added in
-// K-block order onto `out`.  No rows are written to memory and no position table is needed.
+// requested together, while four tiles leave too few workgroups for the compute units' ingest); wave =
+// (walker, K block): it multiplies its K block of both tiles, so a unit's activation rows are
+// fetched once for the two (a compute unit's intake counts them like the weights), and with two
+// walkers per K block, each taking every other unit, a compute unit still has four waves at work.
+// A wave walks its (block, 16-row half) units that hold real pairs, in sorted order, with the next
+// kColsDepth units' operands already requested (a unit is 4 KiB of weights per wave: the depth is
+// what keeps a wave's share of HBM in flight), and adds each weighted product row into its own
+// [tokens][16] fp32 table per tile in LDS: one wave per table and a fixed walk, so the sum is
+// deterministic.  The tables are added in K-block order, a K block's walkers in order, onto `out`.
+// No rows are written to memory and no position table is needed.
 struct DownColsParams
 {
     const uint8_t*  xq;  // [slots][K] fp8 by sorted slot
@@ -878,16 +881,17 @@ struct DownColsParams
     int64_t         out_stride;
     int32_t         M, K, N, kblocks, max_blocks, experts;
     int32_t         block_rows, expert_shift; // as in MoeGemmParams
+    int32_t         walkers; // waves per K block: each walks every walkers-th unit into tables of its own
 };
 
-constexpr int kColsDepth     = 8;
-constexpr int kColsTiles     = 2;    // 16-column tiles per workgroup
+constexpr int kColsDepth     = 7;
+constexpr int kColsTiles     = 2;    // 16-column tiles per workgroup, both multiplied by every wave
 constexpr int kColsMaxBlocks = 1024; // blocks the unit scan takes (16 per lane)
 constexpr size_t kColsTableBytes = (size_t)140 << 10; // LDS for the per-token tables; the unit list (16 KiB at most) comes on top
 
 struct ColsStage
 {
-    i32x4    wlo, whi, xlo, xhi;
+    i32x4    wlo[kColsTiles], whi[kColsTiles], xlo, xhi;
     float    xs, ws;
     u32x2    sw_tok; // routing weight (as bits) and token id
     uint32_t mask;
@@ -917,14 +921,15 @@ __device__ __forceinline__ void cols_load8_at16(u32x2& d, const void* p)
 {
     asm volatile("global_load_dwordx2 %0, %1, off offset:16" : "=v"(d) : "v"(p) : "memory");
 }
-constexpr int kColsLoadsPerStage = 7; // loads the walk requests per unit, counted by cols_wait_oldest
+constexpr int kColsLoadsPerStage = 9; // loads the walk requests per unit, counted by cols_wait_oldest
 // the stage requested kColsDepth - 1 stages ago has arrived once at most (kColsDepth - 1) *
-// kColsLoadsPerStage = 49 younger loads are outstanding (loads return in order); the stage's
+// kColsLoadsPerStage = 54 younger loads are outstanding (loads return in order); the stage's
 // registers are operands so that nothing that reads them is moved above the wait
 __device__ __forceinline__ void cols_wait_oldest(ColsStage& s)
 {
-    asm volatile("s_waitcnt vmcnt(49)"
-                 : "+v"(s.wlo), "+v"(s.whi), "+v"(s.xlo), "+v"(s.xhi), "+v"(s.xs), "+v"(s.ws), "+v"(s.sw_tok)
+    asm volatile("s_waitcnt vmcnt(54)"
+                 : "+v"(s.wlo[0]), "+v"(s.whi[0]), "+v"(s.wlo[1]), "+v"(s.whi[1]), "+v"(s.xlo), "+v"(s.xhi), "+v"(s.xs),
+                   "+v"(s.ws), "+v"(s.sw_tok)
                  :
                  : "memory");
 }
@@ -933,14 +938,15 @@ __device__ __forceinline__ void cols_wait_oldest(ColsStage& s)
 __device__ __forceinline__ void cols_drain(ColsStage& s)
 {
     asm volatile("s_waitcnt vmcnt(0)"
-                 : "+v"(s.wlo), "+v"(s.whi), "+v"(s.xlo), "+v"(s.xhi), "+v"(s.xs), "+v"(s.ws), "+v"(s.sw_tok)
+                 : "+v"(s.wlo[0]), "+v"(s.whi[0]), "+v"(s.wlo[1]), "+v"(s.whi[1]), "+v"(s.xlo), "+v"(s.xhi), "+v"(s.xs),
+                   "+v"(s.ws), "+v"(s.sw_tok)
                  :
                  : "memory");
 }
-static_assert((kColsDepth - 1) * kColsLoadsPerStage == 49, "cols_wait_oldest counts 49 younger loads");
+static_assert((kColsDepth - 1) * kColsLoadsPerStage == 54 && kColsTiles == 2, "cols_wait_oldest counts 54 younger loads");
 
 template <In16 DT>
-__global__ __launch_bounds__(512) void moe_down_cols_kernel(DownColsParams p)
+__global__ __launch_bounds__(256) void moe_down_cols_kernel(DownColsParams p)
 {
     extern __shared__ __attribute__((aligned(16))) uint32_t cols_lds[];
     __shared__ int n_units_s;
@@ -948,7 +954,9 @@ __global__ __launch_bounds__(512) void moe_down_cols_kernel(DownColsParams p)
     uint32_t*      unit_b = cols_lds + 2 * p.max_blocks; // expert << 16 | the half's row mask
     float*         acc    = (float*)(cols_lds + 4 * p.max_blocks); // [waves][M + 16][16], rows M.. are spares
     const int      t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
-    const int      kb = wave % p.kblocks, tile = blockIdx.x * kColsTiles + wave / p.kblocks;
+    // wave = K block; it multiplies both of the workgroup's tiles, so a unit's activation rows are
+    // fetched once for the two (a compute unit's intake counts them like the weights)
+    const int      walker = wave / p.kblocks, kb = wave - walker * p.kblocks, tile = blockIdx.x * kColsTiles;
 
     if(wave == 0) // list the units in sorted order
     {
@@ -990,29 +998,35 @@ __global__ __launch_bounds__(512) void moe_down_cols_kernel(DownColsParams p)
         if(lane == 0)
             n_units_s = base;
     }
-    for(int i = t; i < kColsTiles * p.kblocks * (p.M + 16) * 16; i += blockDim.x)
+    for(int i = t; i < p.walkers * kColsTiles * p.kblocks * (p.M + 16) * 16; i += blockDim.x)
         acc[i] = 0.f;
     __syncthreads();
-    const int units = n_units_s;
+    // this wave's units: walker, walker + walkers, ... of the list
+    const int units = (n_units_s - walker + p.walkers - 1) / p.walkers;
 
     const int      n0     = tile * 16;
     const size_t   wexp   = (size_t)p.N * (size_t)p.K;
     const uint8_t* wlane  = p.w + (size_t)tile * 16 * (size_t)p.K + (size_t)kb * 2048 + kg * 512 + l16 * 16;
-    const float*   wslane = p.wsc + (size_t)(n0 / 128) * p.kblocks + kb;
+    const float*   wslane = p.wsc + (size_t)(n0 / 128) * p.kblocks + kb; // (both tiles lie in one 128-column block)
     const size_t   wsexp  = (size_t)(p.N / 128) * p.kblocks;
-    float*         mine   = acc + (size_t)wave * (p.M + 16) * 16 + kg * 4;
+    const size_t   wtile  = (size_t)16 * (size_t)p.K; // bytes between the two tiles
+    // table of (walker, tile tw, K block kb): (walker * tiles + tw) * kblocks + kb
+    float* const   mine   = acc + ((size_t)walker * kColsTiles * p.kblocks + kb) * (p.M + 16) * 16 + kg * 4;
+    const size_t   table1 = (size_t)p.kblocks * (p.M + 16) * 16; // floats from tile 0's table to tile 1's
 
     // The walk is free of branches (the compiler then keeps the requested depth of loads in flight):
     // past the last unit the last unit is requested again and its product goes to spare rows.
     auto issue = [&](ColsStage& s, int u) {
-        u = u < units ? u : units - 1;
+        u = (u < units ? u : units - 1) * p.walkers + walker;
         const uint32_t a = __builtin_amdgcn_readfirstlane(unit_a[u]);
         const uint32_t b = __builtin_amdgcn_readfirstlane(unit_b[u]);
         const int      expert = (int)(b >> 16);
         s.mask                = b & 0xffffu;
         const uint8_t* wp     = wlane + (size_t)expert * wexp;
-        cols_load16(s.wlo, wp);
-        cols_load16_at256(s.whi, wp);
+        cols_load16(s.wlo[0], wp);
+        cols_load16_at256(s.whi[0], wp);
+        cols_load16(s.wlo[1], wp + wtile);
+        cols_load16_at256(s.whi[1], wp + wtile);
         cols_load4(s.ws, wslane + (size_t)expert * wsexp);
         // rows that are padding read the unit's first real row instead: same cache lines, no traffic
         const int    row  = (s.mask >> l16) & 1u ? l16 : __builtin_ctz(s.mask);
@@ -1026,9 +1040,15 @@ __global__ __launch_bounds__(512) void moe_down_cols_kernel(DownColsParams p)
     };
     auto consume = [&](ColsStage& s, bool live) {
         cols_wait_oldest(s);
-        const i32x8 w = i32x8{s.wlo[0], s.wlo[1], s.wlo[2], s.wlo[3], s.whi[0], s.whi[1], s.whi[2], s.whi[3]};
         const i32x8 x = i32x8{s.xlo[0], s.xlo[1], s.xlo[2], s.xlo[3], s.xhi[0], s.xhi[1], s.xhi[2], s.xhi[3]};
-        const f32x4 prod = mfma_16x16x128_fp8(w, x, f32x4{0.f, 0.f, 0.f, 0.f});
+        f32x4       prod[kColsTiles];
+#pragma unroll
+        for(int tw = 0; tw < kColsTiles; ++tw)
+        {
+            const i32x8 w = i32x8{s.wlo[tw][0], s.wlo[tw][1], s.wlo[tw][2], s.wlo[tw][3],
+                                  s.whi[tw][0], s.whi[tw][1], s.whi[tw][2], s.whi[tw][3]};
+            prod[tw]      = mfma_16x16x128_fp8(w, x, f32x4{0.f, 0.f, 0.f, 0.f});
+        }
         // Padding rows go to a spare row per lane.  The table update is a plain read-add-write (LDS
         // float atomics cost 0.3 us per instruction here): right as long as the 16 rows of a unit are
         // 16 different tokens.  A routing that names an expert twice for a token puts the two pairs
@@ -1039,15 +1059,19 @@ __global__ __launch_bounds__(512) void moe_down_cols_kernel(DownColsParams p)
         const int   row  = real ? key : p.M + l16;
         const float sc   = s.xs * s.ws;
         float*      dst  = mine + (size_t)row * 16;
-        f32x4       add;
+        f32x4       add[kColsTiles];
 #pragma unroll
-        for(int c = 0; c < 4; ++c)
-            add[c] = prod[c] * sc * __uint_as_float(s.sw_tok[0]);
+        for(int tw = 0; tw < kColsTiles; ++tw)
+#pragma unroll
+            for(int c = 0; c < 4; ++c)
+                add[tw][c] = prod[tw][c] * sc * __uint_as_float(s.sw_tok[0]);
         if(__builtin_expect(__ballot(real && prev == key) == 0, 1))
         {
-            f32x4 cur = *(f32x4*)dst;
-            cur += add;
-            *(f32x4*)dst = cur;
+            f32x4 cur0 = *(f32x4*)dst, cur1 = *(f32x4*)(dst + table1);
+            cur0 += add[0];
+            cur1 += add[1];
+            *(f32x4*)dst            = cur0;
+            *(f32x4*)(dst + table1) = cur1;
         }
         else
         {
@@ -1058,9 +1082,13 @@ __global__ __launch_bounds__(512) void moe_down_cols_kernel(DownColsParams p)
                 asm volatile("" ::: "memory");
                 if(l16 == r)
                 {
-                    f32x4 cur = *(volatile f32x4*)dst;
-                    cur += add;
-                    *(volatile f32x4*)dst = cur;
+#pragma unroll
+                    for(int tw = 0; tw < kColsTiles; ++tw)
+                    {
+                        f32x4 cur = *(volatile f32x4*)(dst + tw * table1);
+                        cur += add[tw];
+                        *(volatile f32x4*)(dst + tw * table1) = cur;
+                    }
                 }
             }
         }
@@ -1093,7 +1121,8 @@ __global__ __launch_bounds__(512) void moe_down_cols_kernel(DownColsParams p)
         const int tw = i / (p.M * 4), tok = (i - tw * p.M * 4) >> 2, q = i & 3;
         f32x4     sum = f32x4{0.f, 0.f, 0.f, 0.f};
         for(int k = 0; k < p.kblocks; ++k)
-            sum += *(const f32x4*)(acc + ((size_t)(tw * p.kblocks + k) * (p.M + 16) + tok) * 16 + q * 4);
+            for(int wk = 0; wk < p.walkers; ++wk)
+                sum += *(const f32x4*)(acc + ((size_t)((wk * kColsTiles + tw) * p.kblocks + k) * (p.M + 16) + tok) * 16 + q * 4);
         uint16_t*   dst  = p.out + (size_t)tok * p.out_stride + (blockIdx.x * kColsTiles + tw) * 16 + q * 4;
         const u32x2 prev = *(const u32x2*)dst;
         float       o[4];
@@ -1184,10 +1213,20 @@ size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 // them between the weight reads costs 5 % of the layer's time in fp32.
 bool rows_in_f32(const MoeArgs& a) { return (size_t)a.M * a.topk * a.dim * 4 <= ((size_t)32 << 20); }
 
+// Walkers per K block of moe_down_cols_kernel: two where their tables ([2 walkers][2 tiles][inter/128]
+// [tokens + 16][16] fp32) and the unit list (16 bytes per block) fit the LDS the kernel may ask for and the
+// workgroup stays within four waves, else one.
+constexpr size_t kColsLdsBytes = kColsTableBytes + (size_t)kColsMaxBlocks * 16;
+int cols_walkers(const MoeArgs& a)
+{
+    const int    kblocks = a.inter / 128;
+    const size_t one     = (size_t)kColsTiles * kblocks * (a.M + 16) * 64;
+    return (2 * one + (size_t)a.max_blocks * 16 <= kColsLdsBytes && 2 * kblocks <= 4) ? 2 : 1;
+}
+
 // Decode-size batches take the second GEMM that owns output columns and sums per token in LDS
-// (moe_down_cols_kernel): its tables, [2 * inter/128][tokens + 16][16] fp32 (at most 140 KiB: 544 tokens at
-// inter = 256), and its unit list (16 bytes per block, at most 16 KiB) have to fit the 160 KiB of LDS.  Beyond, rows go through memory and moe_combine_kernel adds them.  down_mode 1 / 2
-// force the one / the other (2 only where it fits).
+// (moe_down_cols_kernel): its tables and its unit list have to fit the LDS.  Beyond, rows go through
+// memory and moe_combine_kernel adds them.  down_mode 1 / 2 force the one / the other (2 only where it fits).
 bool down_by_columns(const MoeArgs& a)
 {
     const int  kblocks = a.inter / 128;
@@ -1195,9 +1234,10 @@ bool down_by_columns(const MoeArgs& a)
                       a.max_blocks <= kColsMaxBlocks && a.dim % (16 * kColsTiles) == 0;
     if(a.down_mode == 1 || !fits)
         return false;
-    // measured on the DeepSeek-V3 layer against rows through memory: 12 % faster at 1 token, 3 % at 128 and
-    // 192, 2 % at 256, even at 384, 8 % slower at 512 (the tables' clearing and final sum grow with the tokens)
-    return a.down_mode == 2 || a.M <= 320;
+    // measured on the DeepSeek-V3 layer against rows through memory: with two walkers 4 % faster at 1 token,
+    // 6 % at 16-192, 8 % at 256 and 264 (275 against 297 us); with one walker (the tables of two no longer
+    // fit) 2 % slower at 272-320 tokens
+    return a.down_mode == 2 || cols_walkers(a) == 2;
 }
 
 } // namespace
@@ -1451,8 +1491,12 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
         c.block_rows        = a.block_rows;
         c.expert_shift      = a.expert_shift;
         c.experts           = a.experts;
-        const size_t lds    = (size_t)a.max_blocks * 16 + (size_t)kColsTiles * c.kblocks * (a.M + 16) * 64;
-        const dim3   grid((unsigned)(a.dim / (16 * kColsTiles))), block((unsigned)(64 * c.kblocks * kColsTiles));
+        // two walkers per K block where their tables fit and the workgroup stays within four waves (DeepSeek-V3
+        // layer, 16 / 64 / 256 tokens: 112 / 224 / 275 us with two, 118 / 240 / 299 with one, 114 / 226 / - with four)
+        const size_t one    = (size_t)kColsTiles * c.kblocks * (a.M + 16) * 64;
+        c.walkers           = cols_walkers(a);
+        const size_t lds    = (size_t)a.max_blocks * 16 + (size_t)c.walkers * one;
+        const dim3   grid((unsigned)(a.dim / (16 * kColsTiles))), block((unsigned)(64 * c.kblocks * c.walkers));
         auto kernel = a.out_dtype == In16::bf16 ? moe_down_cols_kernel<In16::bf16> : moe_down_cols_kernel<In16::fp16>;
         constexpr int            kMaxDevices = 64;
         static std::atomic<bool> raised[kMaxDevices][2]; // dynamic LDS above the default limit needs opting in, once
@@ -1461,8 +1505,7 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
             return hipErrorInvalidDevice;
         if(!raised[a.device_id][inst])
         {
-            e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)(kColsTableBytes + kColsMaxBlocks * 16));
+            e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kColsLdsBytes);
             if(e != hipSuccess)
                 return e;
             raised[a.device_id][inst] = true;

@@ -308,7 +308,8 @@ int moe_sorting_fwd(aiter_tensor_t* topk_ids, aiter_tensor_t* topk_weights, aite
  *   tuning hint here ("nt=1|2|4", "dw=2|4|8", "dc=2|4|8", "down=rows", "down=cols"; anything
  *   else: choose).
  * The product of the first GEMM is quantised 1x128 to fp8 for the second.  Each token's k
- * contributions are added in a fixed order (sorted order up to 320 tokens, slot order beyond):
+ * contributions are added in a fixed order (sorted order while the per-token tables of the second GEMM fit
+ * the LDS, about 280 tokens at inter = 256; slot order beyond):
  * results do not depend on timing.  Scratch memory: see the top of this file.
  */
 int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_tensor_t* gate, aiter_tensor_t* down,
