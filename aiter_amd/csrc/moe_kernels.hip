@@ -1236,7 +1236,7 @@ bool down_by_columns(const MoeArgs& a)
         return false;
     // measured on the DeepSeek-V3 layer against rows through memory: with two walkers 4 % faster at 1 token,
     // 6 % at 16-192, 8 % at 256 and 264 (275 against 297 us); with one walker (the tables of two no longer
-    // fit) 2 % slower at 272-320 tokens
+    // fit) 2 % slower at 288-320 tokens
     return a.down_mode == 2 || cols_walkers(a) == 2;
 }
 
