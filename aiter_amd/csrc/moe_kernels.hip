@@ -1205,6 +1205,73 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const void* __restrict
     *(u32x2*)dst = u32x2{pack2<DT>(o[0] + acc[0], o[1] + acc[1]), pack2<DT>(o[2] + acc[2], o[3] + acc[3])};
 }
 
+// The same sum for rows kept in 16 bits, eight elements per lane: 16-byte loads, and a token's rows are all
+// requested before the first is added (the additions stay in slot order: the same bits as above).
+template <In16 DT>
+__global__ __launch_bounds__(256) void moe_combine8_kernel(const uint16_t* __restrict__ y, const float* __restrict__ sorted_weights,
+                                                           const int32_t* __restrict__ where,
+                                                           const int32_t* __restrict__ sorted_ids,
+                                                           const int32_t* __restrict__ num_valid, int32_t max_padded,
+                                                           uint16_t* __restrict__ out, int32_t M, int32_t topk,
+                                                           int32_t dim, int64_t out_stride)
+{
+    const int octs  = dim / 8;
+    const int token = blockIdx.x;
+    const int q     = blockIdx.y * 256 + threadIdx.x;
+    if(q >= octs)
+        return;
+    const int32_t valid = num_valid[0] < max_padded ? num_valid[0] : max_padded;
+    float         acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    constexpr int kChunk = 8;
+    for(int k0 = 0; k0 < topk; k0 += kChunk)
+    {
+        u32x4 v[kChunk];
+        float w[kChunk];
+        bool  ok[kChunk];
+#pragma unroll
+        for(int i = 0; i < kChunk; ++i)
+        {
+            const int     k  = k0 + i;
+            const int32_t at = k < topk ? where[(size_t)token * topk + k] : -1;
+            ok[i]            = at >= 0 && at < valid && sorted_ids[at] == ((k << 24) | token);
+            const int32_t r  = ok[i] ? at : 0; // (row 0 exists; what is read there is not used)
+            w[i]             = ok[i] ? sorted_weights[r] : 0.f;
+            v[i]             = *(const u32x4*)(y + (size_t)r * dim + (size_t)q * 8);
+        }
+#pragma unroll
+        for(int i = 0; i < kChunk; ++i)
+            if(ok[i])
+            {
+#pragma unroll
+                for(int c = 0; c < 4; ++c)
+                {
+                    acc[2 * c]     = __builtin_fmaf(w[i], __uint_as_float(v[i][c] << 16), acc[2 * c]);
+                    acc[2 * c + 1] = __builtin_fmaf(w[i], __uint_as_float(v[i][c] & 0xffff0000u), acc[2 * c + 1]);
+                }
+            }
+    }
+    uint16_t*   dst  = out + (size_t)token * out_stride + (size_t)q * 8;
+    const u32x4 prev = *(const u32x4*)dst;
+    u32x4       res;
+#pragma unroll
+    for(int c = 0; c < 4; ++c)
+    {
+        float lo, hi;
+        if constexpr(DT == In16::bf16)
+        {
+            lo = __uint_as_float(prev[c] << 16);
+            hi = __uint_as_float(prev[c] & 0xffff0000u);
+        }
+        else
+        {
+            lo = (float)__builtin_bit_cast(_Float16, (unsigned short)(prev[c] & 0xffffu));
+            hi = (float)__builtin_bit_cast(_Float16, (unsigned short)(prev[c] >> 16));
+        }
+        res[c] = pack2<DT>(lo + acc[2 * c], hi + acc[2 * c + 1]);
+    }
+    *(u32x4*)dst = res;
+}
+
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
 // The second GEMM's rows wait in memory for the per-token sum: in fp32 while the real rows
@@ -1547,6 +1614,14 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
                            stream, d);
     }
 
+    if(!y32 && (a.dim & 7) == 0 && (a.out_stride & 7) == 0 && ((uintptr_t)a.out & 15) == 0 && ((uintptr_t)y & 15) == 0)
+    {
+        const dim3 grid8((unsigned)a.M, (unsigned)((a.dim / 8 + 255) / 256));
+        auto combine8 = a.out_dtype == In16::bf16 ? moe_combine8_kernel<In16::bf16> : moe_combine8_kernel<In16::fp16>;
+        hipLaunchKernelGGL(combine8, grid8, dim3(256), 0, stream, (const uint16_t*)y, a.sorted_weights, where, a.sorted_ids,
+                           a.num_valid, a.max_padded, (uint16_t*)a.out, a.M, a.topk, a.dim, a.out_stride);
+        return hipGetLastError();
+    }
     const dim3 cgrid((unsigned)a.M, (unsigned)((a.dim / 4 + 255) / 256));
     auto combine = a.out_dtype == In16::bf16
                        ? (y32 ? moe_combine_kernel<In16::bf16, true> : moe_combine_kernel<In16::bf16, false>)
