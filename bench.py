@@ -804,7 +804,7 @@ def main():
         w5 = MoeWorkload()
         w5.setup(torch, dev)
         moe = []
-        for tokens in (32, 128):
+        for tokens in (16, 32, 128):
             w5.prepare(tokens)
             s5 = time_launches(torch, w5.step, 16, 3)
             moe.append({"tokens": tokens, "replay_us_per_launch": s5 * 1e6, "GB/s": w5.bytes() / s5 / 1e9,
