@@ -251,6 +251,21 @@ def test_fmoe_sorted_in_other_block_sizes(block, tokens, dim, inter, experts, to
     assert_close(out, refs, f"fused_moe, block {block}")
 
 
+@pytest.mark.parametrize("tokens", [272, 400])
+def test_fmoe_column_kernel_with_two_walkers_and_one(tokens):
+    # inter = 256: up to about 280 tokens the per-token tables of two walkers per K block fit the LDS and the
+    # library takes the column kernel by itself; beyond it takes rows through memory, and the column kernel
+    # asked for by name runs with one walker
+    p = make_moe(tokens, 512, 256, 16, 4, seed=tokens)
+    refs = reference(p)
+    auto, cols, rows = run_moe(p), run_moe(p, kernel_name="down=cols"), run_moe(p, kernel_name="down=rows")
+    assert_close(cols, refs, f"{tokens} tokens, columns")
+    assert_close(rows, refs, f"{tokens} tokens, rows")
+    same_as = cols if tokens == 272 else rows
+    assert torch.equal(auto.view(torch.int16), same_as.view(torch.int16))
+    assert torch.equal(cols.view(torch.int16), run_moe(p, kernel_name="down=cols").view(torch.int16))  # run to run
+
+
 def test_fmoe_both_second_gemms_on_the_reference_shape():
     p = make_moe(48, 7168, 256, 32, 8, seed=3)
     refs = reference(p)
