@@ -27,7 +27,6 @@ _TP = ctypes.POINTER(aiter_tensor_t)
 _SIGNATURES = {
     # name: argtypes before the trailing stream
     "dynamic_per_token_scaled_quant": [_TP, _TP, _TP, _TP, ctypes.c_int, _TP, ctypes.c_int64],
-    "aiter_fp8bs_stream_probe": [_TP, _TP, ctypes.c_int64],
     "rmsnorm": [_TP, _TP, _TP, ctypes.c_float, ctypes.c_int],
     "rmsnorm_quant": [_TP, _TP, _TP, _TP, ctypes.c_float, ctypes.c_int64, ctypes.c_int, ctypes.c_int],
     "add_rmsnorm": [_TP, _TP, _TP, _TP, _TP, ctypes.c_float, ctypes.c_int],

@@ -553,28 +553,6 @@ int dynamic_per_token_scaled_quant(aiter_tensor_t* out, aiter_tensor_t* input,
     });
 }
 
-int aiter_fp8bs_stream_probe(aiter_tensor_t* dst, aiter_tensor_t* src, int64_t mode, aiter_stream_t stream)
-{
-    return guarded([&] {
-        const char* fn = "aiter_fp8bs_stream_probe";
-        check_tensor(fn, dst, "dst");
-        check_tensor(fn, src, "src");
-        same_device(fn, {dst, src});
-        if(mode < 0 || mode > 2)
-            fail(fn, "mode must be 0 (read), 1 (write) or 2 (read + write), got ", mode);
-        if(!contiguous(dst) || !contiguous(src))
-            fail(fn, "dst and src must be contiguous");
-        const size_t dst_bytes = dst->numel_ * dtype_size(dst->dtype_), src_bytes = src->numel_ * dtype_size(src->dtype_);
-        if(dst_bytes == 0 || dst_bytes % 16 != 0 || src_bytes != 2 * dst_bytes)
-            fail(fn, "dst must span a positive multiple of 16 bytes and src twice as many, got ", dst_bytes, " and ",
-                 src_bytes);
-        check_aligned(fn, dst, "dst", 16);
-        check_aligned(fn, src, "src", 16);
-        DeviceGuard guard(src->device_id);
-        check_hip(fn, fp8bs::launch_stream_probe((int)mode, src->ptr, dst->ptr, dst_bytes / 16, (hipStream_t)stream));
-    });
-}
-
 int rmsnorm(aiter_tensor_t* out, aiter_tensor_t* input, aiter_tensor_t* weight, float epsilon,
             int gemma_norm, aiter_stream_t stream)
 {

@@ -29,10 +29,6 @@ struct QuantArgs
 };
 hipError_t launch_group_quant(const QuantArgs& a, hipStream_t stream);
 
-// Streaming probe with the quant kernel's access pattern and no arithmetic: per unit 32 bytes read from
-// src and 16 bytes written to dst (mode 2), read only (0) or written only (1).
-hipError_t launch_stream_probe(int mode, const void* src, void* dst, uint64_t n_units, hipStream_t stream);
-
 struct WeightQuantArgs
 {
     const void* w;     // [N, K] 16-bit floats, row stride ldw elements

@@ -359,48 +359,6 @@ hipError_t launch_group_quant(const QuantArgs& a, hipStream_t stream)
     }
 }
 
-// ---------------------------------------------------------------- streaming probe
-// The group quant kernel with its arithmetic taken out: the same grid, the same 32 bytes in and
-// 16 bytes out per lane, the same non-temporal accesses.  What this reaches is the ceiling the
-// quant kernel is measured against (mode 2), beside a read-only (0) and a write-only (1) pass.
-template <int MODE>
-__global__ __launch_bounds__(kQuantBlock) void stream_probe_kernel(const u32x4* __restrict__ x, u32x4* __restrict__ y,
-                                                                   uint32_t n_units)
-{
-    const uint32_t i = blockIdx.x * kQuantBlock + threadIdx.x;
-    if(i >= n_units)
-        return;
-    u32x4 o = u32x4{i, i, i, i};
-    if constexpr(MODE != 1)
-    {
-        const u32x4 a = __builtin_nontemporal_load(x + 2 * (size_t)i);
-        const u32x4 b = __builtin_nontemporal_load(x + 2 * (size_t)i + 1);
-        o             = a ^ b;
-    }
-    if constexpr(MODE == 0)
-    {
-        if((o[0] ^ o[1] ^ o[2] ^ o[3]) == 0x9e3779b9u && (o[0] + o[1]) == 0x7f4a7c15u) // practically never: keeps the loads alive
-            y[0] = o;
-    }
-    else
-        __builtin_nontemporal_store(o, y + i);
-}
-
-hipError_t launch_stream_probe(int mode, const void* src, void* dst, uint64_t n_units, hipStream_t stream)
-{
-    if(n_units == 0 || n_units >= (1ull << 32))
-        return hipErrorInvalidValue;
-    const dim3 grid((unsigned)((n_units + kQuantBlock - 1) / kQuantBlock)), block(kQuantBlock);
-    switch(mode)
-    {
-    case 0: hipLaunchKernelGGL(stream_probe_kernel<0>, grid, block, 0, stream, (const u32x4*)src, (u32x4*)dst, (uint32_t)n_units); break;
-    case 1: hipLaunchKernelGGL(stream_probe_kernel<1>, grid, block, 0, stream, (const u32x4*)src, (u32x4*)dst, (uint32_t)n_units); break;
-    case 2: hipLaunchKernelGGL(stream_probe_kernel<2>, grid, block, 0, stream, (const u32x4*)src, (u32x4*)dst, (uint32_t)n_units); break;
-    default: return hipErrorInvalidValue;
-    }
-    return hipGetLastError();
-}
-
 // ---------------------------------------------------------------- weight-side 128x128 block quant
 // One workgroup per 128x128 block of a [N, K] weight matrix: one scale per block, codes by the
 // same exact division as the activation quant.  Rows past N count as zeros (they do not move the

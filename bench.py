@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the FP8 block-scale path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload quant|prefill|decode|decode9|sweep|moe|fused|stream]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload quant|prefill|decode|decode9|sweep|moe|fused|stream|ceiling]
                     [--no-also] [--no-cpu]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
@@ -20,6 +20,12 @@ Workloads (the benchmark configurations):
   fused    config 5  RMSNorm + 1x128 quant on [2048,7168], then GEMM N=4096
   stream   (calibration) read-only / write-only / 2:1 mixed streaming rates of the quant kernel's
                      access pattern without its arithmetic, on config 2's byte counts
+  ceiling  (calibration) the prefill GEMM's arithmetic (fp8 MFMA + four scale FMAs per MFMA) on
+                     register-resident operands -- no LDS, no global memory -- run for seconds with
+                     the shader clock and socket power sampled beside it, then the prefill kernel
+                     itself under the same sampling
+The two calibration workloads use kernels of their own (bench_probes.hip -> libbench_probes.so,
+built by __graft_entry__.build()); they are not part of the product library.
 
 Timing uses HIP events recorded on the stream the kernels are launched on (torch's current
 stream) around exactly K launches-worth of steps, bracketed by device synchronisation.
@@ -50,7 +56,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="quant", choices=["quant", "prefill", "decode", "decode9", "sweep", "moe", "fused", "copy", "stream"],
+    ap.add_argument("--workload", default="quant", choices=["quant", "prefill", "decode", "decode9", "sweep", "moe", "fused", "copy", "stream", "ceiling"],
                     help="'copy' is a plain 1 GiB device copy used to calibrate the rocprofv3 FETCH_SIZE / "
                     "WRITE_SIZE counters; it is not part of the path")
     ap.add_argument("--no-also", action="store_true", help="time only the primary workload")
@@ -142,6 +148,158 @@ def quant_weight_gpu(torch, fp8, n, k, seed, dev):
     return aiter_amd.weight_per_128x128_quant(w, quant_dtype=fp8)
 
 
+PROBES_PATH = os.path.join(ROOT, "libbench_probes.so")
+_probes = None
+
+
+def load_probes():
+    """ctypes handle of libbench_probes.so (bench_probes.hip): the calibration kernels of the
+    `stream` and `ceiling` workloads.  Built by __graft_entry__.build(); never built here."""
+    global _probes
+    if _probes is None:
+        import ctypes
+
+        if not os.path.exists(PROBES_PATH):
+            raise RuntimeError(f"{PROBES_PATH} is missing: run `python __graft_entry__.py` (build) first")
+        lib = ctypes.CDLL(PROBES_PATH)
+        lib.probe_stream.restype = ctypes.c_int
+        lib.probe_stream.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
+        lib.probe_mfma.restype = ctypes.c_int
+        lib.probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                   ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+        _probes = lib
+    return _probes
+
+
+class GpuSampler:
+    """Samples the shader clock and the socket power of GPU 0 from a host thread while a
+    measurement runs: the amdgpu hwmon files where they can be read (freq1_input in Hz,
+    power1_average / power1_input in microwatts; about a millisecond per sample), else
+    `rocm-smi --showclocks --showpower --json` (a quarter of a second per sample)."""
+
+    def __init__(self, period=0.02):
+        import glob
+
+        self.period = period
+        self.samples = []  # (t, sclk_mhz or None, watts or None)
+        self.source = None
+        self._stop = False
+        self._thread = None
+        self.freq_file = self.power_file = None
+        for hw in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")):
+            f = os.path.join(hw, "freq1_input")
+            pw = [os.path.join(hw, n) for n in ("power1_average", "power1_input")]
+            pw = [q for q in pw if self._readable(q)]
+            if self._readable(f) or pw:
+                self.freq_file = f if self._readable(f) else None
+                self.power_file = pw[0] if pw else None
+                self.source = "hwmon " + hw
+                break
+        if self.source is None:
+            import shutil
+
+            if shutil.which("rocm-smi"):
+                self.source = "rocm-smi"
+                self.period = max(period, 0.25)
+
+    @staticmethod
+    def _readable(path):
+        try:
+            with open(path) as f:
+                float(f.read().strip())
+            return True
+        except (OSError, ValueError):
+            return False
+
+    def _read_once(self):
+        if self.source is None:
+            return None, None
+        if self.source.startswith("hwmon"):
+            mhz = watts = None
+            try:
+                if self.freq_file:
+                    with open(self.freq_file) as f:
+                        mhz = float(f.read()) / 1e6
+                if self.power_file:
+                    with open(self.power_file) as f:
+                        watts = float(f.read()) / 1e6
+            except (OSError, ValueError):
+                pass
+            return mhz, watts
+        import re
+        import subprocess
+
+        try:
+            out = subprocess.run(["rocm-smi", "--showclocks", "--showpower", "--json"], capture_output=True, text=True,
+                                 timeout=5).stdout
+            card = json.loads(out)
+            card = card[sorted(card)[0]]
+        except Exception:
+            return None, None
+        mhz = watts = None
+        for k, v in card.items():
+            kl = k.lower()
+            if "sclk" in kl and mhz is None:
+                m = re.search(r"(\d+(?:\.\d+)?)\s*mhz", str(v).lower())
+                if m:
+                    mhz = float(m.group(1))
+            if "power" in kl and watts is None:
+                try:
+                    watts = float(str(v).split()[0])
+                except ValueError:
+                    pass
+        return mhz, watts
+
+    def __enter__(self):
+        import threading
+
+        def loop():
+            while not self._stop:
+                mhz, watts = self._read_once()
+                self.samples.append((time.perf_counter(), mhz, watts))
+                time.sleep(self.period)
+
+        self._thread = threading.Thread(target=loop, daemon=True)
+        self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        self._thread.join()
+
+    def summary(self, t_from, t_to):
+        """Mean clock (MHz) and power (W) over the samples taken in [t_from, t_to]."""
+        sel = [x for x in self.samples if t_from <= x[0] <= t_to]
+        clk = [x[1] for x in sel if x[1] is not None]
+        pw = [x[2] for x in sel if x[2] is not None]
+        return {"sclk_mhz": sum(clk) / len(clk) if clk else None, "socket_watts": sum(pw) / len(pw) if pw else None,
+                "samples": len(sel), "source": self.source}
+
+
+def sustained(torch, fn, seconds, launches_per_sync=4):
+    """Keeps calling fn for `seconds`, then reports the seconds per call over the second half
+    of that time (HIP events) with the clock and power sampled over the same half."""
+    with GpuSampler() as sampler:
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds / 2:
+            for _ in range(launches_per_sync):
+                fn()
+            torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t1 = time.perf_counter()
+        a.record()
+        n = 0
+        while time.perf_counter() - t1 < seconds / 2:
+            for _ in range(launches_per_sync):
+                fn()
+            n += launches_per_sync
+            torch.cuda.synchronize()
+        b.record()
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+    return a.elapsed_time(b) * 1e-3 / n, n, sampler.summary(t1, t2)
+
+
 # ---------------------------------------------------------------- workloads
 
 
@@ -159,13 +317,14 @@ class QuantWorkload:
         # rotate over several inputs so that no pass finds its input in the 256 MB last-level cache
         base = self.x_cpu.to(dev)
         self.xs = [base, base.clone(), base.clone()]
-        self.y = torch.empty(self.M, self.K, dtype=dtypes.fp8, device=dev)
-        self.s = torch.empty(self.M, self.K // 128, dtype=torch.float32, device=dev)
+        # ... and over as many outputs (3 x (235 + 117 + 3.7) MB in rotation)
+        self.ys = [torch.empty(self.M, self.K, dtype=dtypes.fp8, device=dev) for _ in self.xs]
+        self.ss = [torch.empty(self.M, self.K // 128, dtype=torch.float32, device=dev) for _ in self.xs]
         self.i = 0
 
     def step(self):
         self.i = (self.i + 1) % len(self.xs)
-        self.aiter.dynamic_per_token_scaled_quant(self.y, self.xs[self.i].view(-1, 128), self.s)
+        self.aiter.dynamic_per_token_scaled_quant(self.ys[self.i], self.xs[self.i].view(-1, 128), self.ss[self.i])
 
     def algorithmic_bytes(self):
         return self.M * self.K * 2 + self.M * self.K + self.M * (self.K // 128) * 4
@@ -195,8 +354,8 @@ class QuantWorkload:
     def cpu_baseline(self, torch):
         from oracle import torch_ref as tr
 
-        rows = 4096  # bounded sample: a quarter of the rows, same distribution
-        x = self.x_cpu[:rows]
+        rows = self.M  # the whole input
+        x = self.x_cpu
         tr.per_1x128_quant(x)
         ts = []
         for _ in range(5):
@@ -210,8 +369,8 @@ class QuantWorkload:
             "unit": "GB/s",
             "cores": torch.get_num_threads(),
             "kind": "port",
-            "sample": f"torch-CPU restatement of pertoken_quant on rows 0..{rows - 1} of the same "
-            f"input ([{rows},{self.K}] bf16), median of 5 runs, {sec * 1e3:.1f} ms each",
+            "sample": f"torch-CPU restatement of pertoken_quant on the whole input "
+            f"([{rows},{self.K}] bf16), median of 5 runs, {sec * 1e3:.1f} ms each",
         }
 
 
@@ -417,7 +576,7 @@ class CopyCalibration:
 
 
 class StreamCeilings:
-    """The quant kernel with its arithmetic taken out (aiter_fp8bs_stream_probe: same grid, same
+    """The quant kernel with its arithmetic taken out (probe_stream of bench_probes.hip: same grid, same
     32 bytes in and 16 bytes out per lane, same cache policy) on config 2's byte counts: a
     read-only pass over the 235 MB input, a write-only pass over the 117 MB output, and the 2 : 1
     mix of both.  The ceiling the quant kernel is held against."""
@@ -426,26 +585,29 @@ class StreamCeilings:
     M, K = 16384, 7168
 
     def setup(self, torch, dev):
-        from aiter_amd import _ffi
-
-        self.call = _ffi.call
+        self.torch = torch
+        self.lib = load_probes()
         n = self.M * self.K
         self.xs = [torch.randn(n, device=dev).bfloat16() for _ in range(3)]
-        self.y = torch.empty(n, dtype=torch.uint8, device=dev)
+        self.ys = [torch.empty(n, dtype=torch.uint8, device=dev) for _ in range(3)]
         self.i = 0
 
-    def _next(self):
+    def _probe(self, mode):
         self.i = (self.i + 1) % len(self.xs)
-        return self.xs[self.i]
+        x, y = self.xs[self.i], self.ys[self.i]
+        rc = self.lib.probe_stream(mode, x.data_ptr(), y.data_ptr(), y.numel() // 16,
+                                   self.torch.cuda.current_stream().cuda_stream)
+        if rc != 0:
+            raise RuntimeError(f"probe_stream: hipError {rc}")
 
     def step(self):  # the mix
-        self.call("aiter_fp8bs_stream_probe", self.y, self._next(), 2)
+        self._probe(2)
 
     def step_read(self):
-        self.call("aiter_fp8bs_stream_probe", self.y, self._next(), 0)
+        self._probe(0)
 
     def step_write(self):
-        self.call("aiter_fp8bs_stream_probe", self.y, self._next(), 1)
+        self._probe(1)
 
     def describe(self):
         return {"workload": "streaming ceilings for config 2's byte mix (the quant kernel without arithmetic): "
@@ -467,6 +629,102 @@ class StreamCeilings:
             sec = time_steps(torch, fn, steps, warmup, settle=True)
             out.append({"what": what, "bytes": by, "us": sec * 1e6, "GB/s": by / sec / 1e9,
                         "frac_of_hbm_peak": by / sec / 1e9 / HBM_PEAK_GBS})
+        return out
+
+    def cpu_baseline(self, torch):
+        return None
+
+
+class ComputeCeiling:
+    """What the chip gives the prefill GEMM's arithmetic alone.  probe_mfma (bench_probes.hip) runs the
+    product kernel's inner instruction stream -- v_mfma_f32_16x16x128_f8f6f4 on real fp8 codes, each
+    product folded into fp32 accumulators by four v_fmac_f32 two MFMA slots later -- on operands that
+    never leave the registers: one workgroup per compute unit, no LDS, no global memory, no barrier.
+    Every variant runs for SECONDS with the shader clock and the socket power sampled beside it;
+    then the prefill kernel itself (config 4, both weight layouts) runs under the same sampling."""
+
+    name = "ceiling"
+    SECONDS = 4.0
+    ITERS = 60000  # passes of 32 MFMAs per wave and launch: about 60 ms per launch
+
+    def setup(self, torch, dev):
+        import aiter_amd
+        from aiter_amd import dtypes
+
+        self.torch, self.dev = torch, dev
+        self.lib = load_probes()
+        self.cus = torch.cuda.get_device_properties(0).multi_processor_count
+        g = torch.Generator(device=dev).manual_seed(0)
+        # operands with the code distribution of config 4: x ~ N(0,1) with 1 % of the channels x 50,
+        # quantised 1 x 128; w ~ N(0, 0.02) quantised 128 x 128
+        x = torch.randn(512, 7168, generator=g, device=dev)
+        ch = torch.randperm(7168, generator=g, device=dev)[:71]
+        x[:, ch] *= 50.0
+        xq, _ = aiter_amd.get_hip_quant(aiter_amd.QuantType.per_1x128)(x.bfloat16(), quant_dtype=dtypes.fp8)
+        wq, _ = quant_weight_gpu(torch, dtypes.fp8, 512, 7168, 10, dev)
+        self.real = (wq.view(torch.uint8).flatten()[: 8 * 512 * 32].contiguous(),
+                     xq.view(torch.uint8).flatten()[: 4 * 512 * 32].contiguous())
+        self.zero = (torch.zeros_like(self.real[0]), torch.zeros_like(self.real[1]))
+        self.scales = torch.full((4 * 512,), 1e-9, dtype=torch.float32, device=dev)
+        self.sink = torch.empty(self.cus * 512, dtype=torch.float32, device=dev)
+        self.variant = (4, 512, self.real)
+
+    def _launch(self, fmas, threads, codes, iters):
+        rc = self.lib.probe_mfma(fmas, threads, codes[0].data_ptr(), codes[1].data_ptr(), self.scales.data_ptr(),
+                                 self.sink.data_ptr(), iters, self.cus, self.torch.cuda.current_stream().cuda_stream)
+        if rc != 0:
+            raise RuntimeError(f"probe_mfma: hipError {rc}")
+
+    def flops_per_launch(self, threads, iters):
+        return self.cus * (threads // 64) * iters * 32 * 65536.0
+
+    def step(self):  # the headline: MFMA + 4 FMA, two waves per SIMD, real codes
+        self._launch(4, 512, self.real, self.ITERS // 8)
+
+    def describe(self):
+        return {"workload": "compute ceiling of the prefill GEMM's arithmetic: register-resident fp8 MFMA + 4 scale "
+                            "FMAs per MFMA, one workgroup of 8 waves per compute unit, no LDS, no global memory; "
+                            "headline value is a short run, the sustained figures with clock and power ride in per_shape",
+                "kernel": "mfma_ceiling_kernel (bench_probes.hip)"}
+
+    def result(self, sec):
+        tf = self.flops_per_launch(512, self.ITERS // 8) / sec / 1e12
+        return tf, "TFLOP/s", {"bound": "mfma", "achieved": tf, "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                               "frac": tf / FP8_PEAK_TFLOPS, "traffic": None}
+
+    def per_shape(self, torch, steps, warmup):
+        out = []
+        variants = [
+            ("MFMA + 4 FMA, 8 waves per CU, config-4 codes", 4, 512, self.real),
+            ("MFMA only, 8 waves per CU, config-4 codes", 0, 512, self.real),
+            ("MFMA + 4 FMA, 4 waves per CU, config-4 codes", 4, 256, self.real),
+            ("MFMA only, 4 waves per CU, config-4 codes", 0, 256, self.real),
+            ("MFMA + 4 FMA, 8 waves per CU, all-zero codes", 4, 512, self.zero),
+        ]
+        for what, fmas, threads, codes in variants:
+            iters = self.ITERS if threads == 512 else 2 * self.ITERS
+            sec, n, smp = sustained(torch, lambda: self._launch(fmas, threads, codes, iters), self.SECONDS, 2)
+            tf = self.flops_per_launch(threads, iters) / sec / 1e12
+            row = {"what": what, "ms_per_launch": sec * 1e3, "launches_timed": n, "TFLOP/s": tf,
+                   "frac_of_fp8_peak": tf / FP8_PEAK_TFLOPS,
+                   # clocks per MFMA slot and SIMD if the matrix pipe were never idle: 32
+                   "mfma_issue_ghz": (threads // 256) * iters * 32 * 32 / sec / 1e9}
+            row.update(smp)
+            out.append(row)
+        del self.sink
+        for layout in ("plain", "preshuffled"):
+            torch.cuda.empty_cache()
+            w = GemmWorkload("prefill", 8192, 36864, 7168, "config 4")
+            w.layout = layout
+            w.setup(torch, self.dev)
+            sec, n, smp = sustained(torch, w.step, self.SECONDS, 8)
+            tf = w.flops() / sec / 1e12
+            row = {"what": f"prefill kernel, config 4, {layout} weights", "ms_per_launch": sec * 1e3, "launches_timed": n,
+                   "TFLOP/s": tf, "frac_of_fp8_peak": tf / FP8_PEAK_TFLOPS,
+                   "frac_of_ceiling": tf / out[0]["TFLOP/s"]}
+            row.update(smp)
+            out.append(row)
+            del w
         return out
 
     def cpu_baseline(self, torch):
@@ -680,6 +938,8 @@ def make_workload(name):
         return CopyCalibration()
     if name == "stream":
         return StreamCeilings()
+    if name == "ceiling":
+        return ComputeCeiling()
     if name == "quant":
         return QuantWorkload()
     if name == "prefill":
@@ -740,12 +1000,12 @@ def main():
     }
     if args.workload == "prefill":
         line["vs_reference_tuned_csv"] = value / REF_PREFILL_TFLOPS
-    if args.workload in ("decode9", "sweep", "moe", "stream"):
+    if args.workload in ("decode9", "sweep", "moe", "stream", "ceiling"):
         # shape after shape: steps + warmup launches each, in DECODE_SHAPES order
         line["per_shape"] = wl.per_shape(torch, args.steps, args.warmup)
         args.no_also = True
 
-    if not args.no_cpu and args.workload not in ("copy", "stream"):
+    if not args.no_cpu and args.workload not in ("copy", "stream", "ceiling"):
         torch.set_num_threads(os.cpu_count() or 1)
         line["cpu_baseline"] = wl.cpu_baseline(torch)
 
@@ -753,17 +1013,19 @@ def main():
         also = {}
         del wl
         torch.cuda.empty_cache()
-        for name in ("quant", "prefill", "fused"):
+        for name in ("quant", "prefill", "prefill_preshuffled", "fused"):
             if name == args.workload:
                 continue
-            w2 = make_workload(name)
+            w2 = make_workload(name.split("_")[0])
+            if name == "prefill_preshuffled":
+                w2.layout = "preshuffled"  # the documented fast path: shuffle_weight once, then the bpreshuffle entry
             w2.setup(torch, dev)
-            steps2 = 10 if name == "prefill" else 30
+            steps2 = 10 if name.startswith("prefill") else 30
             s2 = time_steps(torch, w2.step, steps2, 3, settle=True)
             v2, u2, r2 = w2.result(s2)
             entry = {"value": v2, "unit": u2, "us_per_step": s2 * 1e6, "steps": steps2, "roofline": r2,
                      "config": w2.describe()}
-            if name == "prefill":
+            if name.startswith("prefill"):
                 entry["vs_reference_tuned_csv"] = v2 / REF_PREFILL_TFLOPS
             if name == "fused":
                 sn = time_steps(torch, w2.step_norm_only, 30, 3, settle=True)

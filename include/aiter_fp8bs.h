@@ -99,17 +99,6 @@ int dynamic_per_token_scaled_quant(aiter_tensor_t* out, aiter_tensor_t* input,
                                    int64_t num_rows_factor, aiter_stream_t stream);
 
 /*
- * Measurement aid, no counterpart in the reference: the 1 x G quant kernel with its arithmetic taken
- * out -- the same grid, the same 32 bytes read and 16 bytes written per lane, the same cache policy.
- *   mode 2: dst[i] <- f(src[2i], src[2i+1]) in 16-byte units (2 bytes in, 1 byte out per element)
- *   mode 0: src is read and nothing written;  mode 1: dst is written and nothing read
- *   src spans twice the bytes of dst; both contiguous and 16-byte aligned.
- * bench.py --workload stream uses it to put the streaming ceiling of the memory system beside the
- * quant kernel's rate.
- */
-int aiter_fp8bs_stream_probe(aiter_tensor_t* dst, aiter_tensor_t* src, int64_t mode, aiter_stream_t stream);
-
-/*
  * RMSNorm -> bf16|fp16.  Replaces aiter::rmsnorm, csrc/include/rmsnorm_quant.h:37-41
  * (binding aiter/ops/rmsnorm.py:625-632).
  *   out, input [rows, hidden] same 16-bit dtype, last dim contiguous; weight [hidden] same dtype
