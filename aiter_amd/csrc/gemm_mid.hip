@@ -576,7 +576,8 @@ static MidPlan plan_cost(const GemmKernelParams& g, int tile, int splits)
     }
     return MidPlan{tile, splits, cost};
 }
-static MidPlan best_plan(const GemmKernelParams& g, int tile)
+// partial_cap: the most bytes of fp32 partial tiles (ranges x M x N x 4) a plan may use; 0 = no limit
+static MidPlan best_plan(const GemmKernelParams& g, int tile, size_t partial_cap = 0)
 {
     const int  tiles_to_try[3] = {128, 64128, 64};
     const bool can_split       = (g.N & 3) == 0 && ((uintptr_t)g.out & 7) == 0;
@@ -589,6 +590,8 @@ static MidPlan best_plan(const GemmKernelParams& g, int tile)
         const int max_splits = can_split ? (g.kblocks / 4 < 8 ? g.kblocks / 4 : 8) : 1;
         for(int sp = 1; sp <= (max_splits < 1 ? 1 : max_splits); ++sp)
         {
+            if(sp > 1 && partial_cap != 0 && (size_t)sp * (size_t)g.M * (size_t)g.N * 4 > partial_cap)
+                break;
             const MidPlan c = plan_cost(g, t, sp);
             if(c.cost < best.cost * 0.98f) // ties go to the earlier candidate (fewer ranges)
                 best = c;
@@ -613,7 +616,9 @@ hipError_t launch_gemm_mid(const GemmKernelParams& g, In16 out_dtype, int split_
         splits = 1 << split_k_log2;
     if(tile == 0 || splits <= 0)
     {
-        MidPlan plan = splits > 0 ? MidPlan{0, splits, 0.f} : best_plan(g, tile);
+        // a caller that may not allocate gets the best plan whose partial tiles fit the fixed buffer
+        // (a count of K ranges that the caller named is an error there instead)
+        MidPlan plan = splits > 0 ? MidPlan{0, splits, 0.f} : best_plan(g, tile, ctx.static_only ? kStaticPartialBytes : 0);
         if(splits > 0) // ranges pinned, tile free: best tile for that count
         {
             plan.cost = 1e30f;

@@ -6,10 +6,18 @@
 // streams cannot touch each other's partial results.  A block that has been handed out is never
 // freed: HIP graphs captured earlier may hold its address.
 // A call whose stream is capturing allocates, clears and synchronises nothing.  It takes its
-// scratch from the device's capture arena, which every eager call keeps at least as large as its
+// scratch from the device's graph scratch, which every eager call keeps at least as large as its
 // own request (up to a cap per kind of buffer): after one eager run of a call, on any stream, the
-// same call can be recorded on any stream; otherwise it fails with a message.  Graphs of one
-// device therefore share scratch with each other (not with eager work): replay them one at a time.
+// same call can be recorded on any stream; otherwise it fails with a message.  The graph scratch
+// has up to four lanes, as many as streams of the device have run scratch-using calls eagerly:
+// inside one capture sequence every stream that records such a call keeps a lane to itself
+// (capture_lanes.h), so calls recorded on forked streams, which may run side by side on replay,
+// never share partial results; a capture that forks wider than the warm-up did is refused with a
+// message.  Graphs of one device share the lanes with each other (not with eager work): replay
+// them one at a time.
+// An eager call that must allocate while ANOTHER host thread is capturing does so with its
+// thread's capture mode set to relaxed, which leaves that capture valid; if the runtime refuses
+// all the same, the call fails with a message.
 //
 // Callers that cannot allocate at all have the static buffer instead: a fixed array in device
 // memory, one copy per GPU, shared by every call on that GPU that asks for it (LaunchCtx::

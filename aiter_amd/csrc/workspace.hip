@@ -1,6 +1,8 @@
 // Per-(device, stream) scratch arenas.  See workspace.h for the rules they implement.
 #include "workspace.h"
 
+#include "capture_lanes.h"
+
 #include <vector>
 
 namespace fp8bs {
@@ -15,13 +17,15 @@ struct Block
     size_t bytes = 0;
 };
 
-// Blocks for eager work on one stream, or (capture = true, one per device) for work recorded into
-// graphs on any stream of the device.
+// Blocks for eager work on one stream, or (capture = true: `lane` of the device's graph scratch) for
+// work recorded into graphs.
 struct Arena
 {
-    int         device  = -1;
-    hipStream_t stream  = nullptr;
-    bool        capture = false;
+    int         device   = -1;
+    hipStream_t stream   = nullptr;
+    bool        capture  = false;
+    int         lane     = 0;
+    uint64_t    last_use = 0; // eager arenas: g_use_clock at the latest request
     Block       block[(int)WsKind::kinds];
 };
 
@@ -31,6 +35,10 @@ std::vector<Arena> g_arenas;
 std::vector<Block> g_retired;
 
 constexpr size_t kMaxArenas = 1024;
+uint64_t         g_use_clock = 0;
+// per device: which stream of which capture sequence records into which lane of the graph scratch
+constexpr int    kMaxDevices = 64;
+CaptureLaneTable g_lanes[kMaxDevices];
 // per kind: smallest block worth allocating, and the largest request served
 constexpr size_t kMinBytes[(int)WsKind::kinds] = {(size_t)1 << 20, (size_t)16 << 10, (size_t)64 << 10, (size_t)1 << 20};
 constexpr size_t kMaxBytes[(int)WsKind::kinds] = {(size_t)2 << 30, (size_t)64 << 20, (size_t)1 << 30, (size_t)64 << 30};
@@ -49,7 +57,6 @@ __global__ void __launch_bounds__(256) workspace_fill_zero_kernel(uint4* dst, si
 // for hipGetSymbolAddress; g_static_base holds each device's own address of it.
 constexpr size_t kStaticBytes = kStaticPartialBytes + kStaticTickets * sizeof(uint32_t);
 static __device__ __align__(256) unsigned char scratch[kStaticBytes];
-constexpr int  kMaxDevices = 64;
 unsigned char* g_static_base[kMaxDevices]; // guarded by g_mutex
 
 void say(const LaunchCtx& ctx, const char* msg)
@@ -73,11 +80,16 @@ WorkspaceLock::~WorkspaceLock()
 
 namespace {
 
-// The block of one kind in one arena, at least `bytes` large; allocates (never under capture: the
-// callers see to that) when there is none or it is too small.  A fresh block that must start at
-// zero is cleared with a fill kernel on `fill_stream`, or, when the work that will use it may run
-// on another stream, with a synchronous hipMemset.
-hipError_t block_for(const LaunchCtx& ctx, Arena& arena, int k, size_t bytes, bool zeroed, bool fill_in_stream)
+// The block of one kind in one arena, at least `bytes` large; allocates (never on a capturing
+// stream: the callers see to that) when there is none or it is too small.  A fresh block that must
+// start at zero is cleared with a fill kernel on ctx.stream; with `wait`, for a block that work on
+// other streams (graph replays) will use, the call also waits for that fill.
+// Another host thread may be capturing a graph in the mode that forbids allocation to every thread
+// (hipStreamCaptureModeGlobal, the default of most frameworks): the allocation is made with this
+// thread's mode set to relaxed, which leaves that capture valid.  Should the runtime refuse the
+// allocation all the same, the call fails with a message and the foreign capture is not touched
+// any further.
+hipError_t block_for(const LaunchCtx& ctx, Arena& arena, int k, size_t bytes, bool zeroed, bool wait)
 {
     Block& b = arena.block[k];
     if(b.bytes >= bytes)
@@ -88,29 +100,35 @@ hipError_t block_for(const LaunchCtx& ctx, Arena& arena, int k, size_t bytes, bo
         want = 2 * b.bytes;
     if(want < kMinBytes[k])
         want = kMinBytes[k];
-    want         = (want + 255) & ~(size_t)255;
-    void*      fresh = nullptr;
-    hipError_t e     = hipMalloc(&fresh, want);
+    want                      = (want + 255) & ~(size_t)255;
+    void*                fresh = nullptr;
+    hipStreamCaptureMode mode  = hipStreamCaptureModeRelaxed;
+    const bool           swapped = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+    hipError_t           e       = hipMalloc(&fresh, want);
+    if(swapped)
+        (void)hipThreadExchangeStreamCaptureMode(&mode);
     if(e != hipSuccess)
     {
-        say(ctx, "hipMalloc of a scratch buffer failed");
+        (void)hipGetLastError();
+        say(ctx, e == hipErrorStreamCaptureUnsupported || e == hipErrorStreamCaptureInvalidated
+                     ? "a scratch buffer must grow, and the runtime refuses to allocate while another thread captures "
+                       "a graph: run this call once before that capture begins"
+                     : "hipMalloc of a scratch buffer failed");
         return e;
     }
     if(zeroed)
     {
-        if(fill_in_stream)
-        {
-            const size_t vecs   = want / 16;
-            const size_t groups = (vecs + 255) / 256;
-            hipLaunchKernelGGL(workspace_fill_zero_kernel, dim3((unsigned)(groups > 1024 ? 1024 : groups)), dim3(256),
-                               0, ctx.stream, (uint4*)fresh, vecs);
-            e = hipGetLastError();
-        }
-        else
-            e = hipMemset(fresh, 0, want);
+        const size_t vecs   = want / 16;
+        const size_t groups = (vecs + 255) / 256;
+        hipLaunchKernelGGL(workspace_fill_zero_kernel, dim3((unsigned)(groups > 1024 ? 1024 : groups)), dim3(256), 0,
+                           ctx.stream, (uint4*)fresh, vecs);
+        e = hipGetLastError();
+        if(e == hipSuccess && wait)
+            e = hipStreamSynchronize(ctx.stream);
         if(e != hipSuccess)
         {
-            (void)hipFree(fresh); // never handed out
+            // (the fill may be in flight: the block is leaked rather than freed under it)
+            say(ctx, "clearing a fresh scratch buffer failed");
             return e;
         }
     }
@@ -121,8 +139,8 @@ hipError_t block_for(const LaunchCtx& ctx, Arena& arena, int k, size_t bytes, bo
     return hipSuccess;
 }
 
-// This device's copy of the static buffer.  First use on a device (which must be current): look
-// the address up and clear the tickets with a fill kernel on the caller's stream.
+// This device's copy of the static buffer (the device must be current).  The array is zero when
+// the code object is loaded and the kernels leave the tickets zero: nothing is cleared here.
 hipError_t static_base(const LaunchCtx& ctx, unsigned char** base)
 {
     if(ctx.device_id < 0 || ctx.device_id >= kMaxDevices)
@@ -139,38 +157,73 @@ hipError_t static_base(const LaunchCtx& ctx, unsigned char** base)
             say(ctx, "hipGetSymbolAddress of the static scratch buffer failed");
             return e != hipSuccess ? e : hipErrorInvalidSymbol;
         }
-        unsigned char* const tickets = (unsigned char*)ptr + kStaticPartialBytes;
-        const size_t         vecs    = kStaticTickets * sizeof(uint32_t) / 16;
-        hipLaunchKernelGGL(workspace_fill_zero_kernel, dim3((unsigned)((vecs + 255) / 256)), dim3(256), 0, ctx.stream,
-                           (uint4*)tickets, vecs);
-        if((e = hipGetLastError()) != hipSuccess)
-            return e;
         g_static_base[ctx.device_id] = (unsigned char*)ptr;
     }
     *base = g_static_base[ctx.device_id];
     return hipSuccess;
 }
 
-Arena* find_arena(int device, hipStream_t stream, bool capture)
+Arena* find_arena(int device, hipStream_t stream)
 {
     for(Arena& a : g_arenas)
-        if(a.device == device && a.capture == capture && (capture || a.stream == stream))
+        if(!a.capture && a.device == device && a.stream == stream)
             return &a;
     return nullptr;
 }
 
-Arena* add_arena(const LaunchCtx& ctx, bool capture)
+Arena* find_lane(int device, int lane)
+{
+    for(Arena& a : g_arenas)
+        if(a.capture && a.device == device && a.lane == lane)
+            return &a;
+    return nullptr;
+}
+
+int eager_streams_of(int device)
+{
+    int n = 0;
+    for(const Arena& a : g_arenas)
+        n += (!a.capture && a.device == device) ? 1 : 0;
+    return n;
+}
+
+// A new arena; when the table is full, the eager arena of this device that was used longest ago
+// changes hands (its stream is most likely gone: a process that creates and destroys streams).  The
+// device is brought to rest first, so that nothing still works in the blocks that change hands.
+Arena* add_arena(const LaunchCtx& ctx, bool capture, int lane)
 {
     if(g_arenas.size() >= kMaxArenas)
     {
-        say(ctx, "too many (device, stream) pairs hold scratch buffers");
-        return nullptr;
+        Arena* oldest = nullptr;
+        for(Arena& a : g_arenas)
+            if(!a.capture && a.device == ctx.device_id && (oldest == nullptr || a.last_use < oldest->last_use))
+                oldest = &a;
+        if(capture || oldest == nullptr)
+        {
+            say(ctx, "too many (device, stream) pairs hold scratch buffers");
+            return nullptr;
+        }
+        hipStreamCaptureMode mode    = hipStreamCaptureModeRelaxed;
+        const bool           swapped = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+        const hipError_t     e       = hipDeviceSynchronize();
+        if(swapped)
+            (void)hipThreadExchangeStreamCaptureMode(&mode);
+        if(e != hipSuccess)
+        {
+            (void)hipGetLastError();
+            say(ctx, "too many (device, stream) pairs hold scratch buffers, and the device could not be brought to rest "
+                     "to hand the oldest ones on");
+            return nullptr;
+        }
+        oldest->stream = ctx.stream;
+        return oldest;
     }
     g_arenas.push_back(Arena{});
     Arena& a  = g_arenas.back();
     a.device  = ctx.device_id;
     a.stream  = capture ? nullptr : ctx.stream;
     a.capture = capture;
+    a.lane    = lane;
     return &a;
 }
 
@@ -212,39 +265,80 @@ hipError_t workspace_acquire(const LaunchCtx& ctx, const WorkspaceLock& held, Ws
         say(ctx, "the call needs more scratch memory than the library serves for this kind of buffer");
         return hipErrorInvalidValue;
     }
-    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-    hipError_t             e      = hipStreamIsCapturing(ctx.stream, &status);
+    if(ctx.device_id < 0 || ctx.device_id >= kMaxDevices)
+    {
+        say(ctx, "device ordinal outside 0..63");
+        return hipErrorInvalidDevice;
+    }
+    hipStreamCaptureStatus status     = hipStreamCaptureStatusNone;
+    unsigned long long     capture_id = 0;
+    hipError_t             e          = hipStreamGetCaptureInfo(ctx.stream, &status, &capture_id);
     if(e != hipSuccess)
         return e;
     if(status != hipStreamCaptureStatusNone)
     {
-        // Work recorded into a graph uses the device's capture arena, which only eager calls size.
-        Arena* cap = find_arena(ctx.device_id, nullptr, true);
-        if(cap == nullptr || cap->block[k].bytes < bytes)
+        // Work recorded into a graph uses the device's graph scratch, which only eager calls size:
+        // one lane per stream of the capture sequence that records scratch-using calls.
+        int lanes_ready = 0;
+        while(lanes_ready < kCaptureLanes)
+        {
+            const Arena* l = find_lane(ctx.device_id, lanes_ready);
+            if(l == nullptr || l->block[k].bytes < bytes)
+                break;
+            ++lanes_ready;
+        }
+        if(lanes_ready == 0)
         {
             say(ctx, "this call needs scratch memory that has not been allocated, and its stream is capturing: "
                      "nothing is allocated under capture -- run the same call once (on any stream of this device) "
                      "before the capture");
             return hipErrorStreamCaptureUnsupported;
         }
-        *out = cap->block[k].ptr;
+        const int lane = g_lanes[ctx.device_id].lane_of((uint64_t)capture_id, (const void*)ctx.stream, lanes_ready);
+        if(lane < 0)
+        {
+            say(ctx, "this capture records scratch-using calls on more streams than ran such calls before it (each "
+                     "such stream of a capture needs scratch of its own, up to four, and nothing is allocated under "
+                     "capture): run the calls once on as many streams as the capture forks, or record them on one");
+            return hipErrorStreamCaptureUnsupported;
+        }
+        *out = find_lane(ctx.device_id, lane)->block[k].ptr;
         return hipSuccess;
     }
-    Arena* arena = find_arena(ctx.device_id, ctx.stream, false);
-    if(arena == nullptr && (arena = add_arena(ctx, false)) == nullptr)
+    Arena* arena = find_arena(ctx.device_id, ctx.stream);
+    if(arena == nullptr && (arena = add_arena(ctx, false, 0)) == nullptr)
         return hipErrorOutOfMemory;
-    if((e = block_for(ctx, *arena, k, bytes, zeroed, true)) != hipSuccess)
+    arena->last_use = ++g_use_clock;
+    if((e = block_for(ctx, *arena, k, bytes, zeroed, false)) != hipSuccess)
         return e;
     void* const mine = arena->block[k].ptr; // (add_arena below may move the table)
-    // Keep the capture arena large enough for this call to be recorded later (the usual order: an
-    // eager warm-up, then the capture on a stream of the framework's choosing).
+    // Keep the graph scratch large enough for this call to be recorded later (the usual order: an
+    // eager warm-up, then the capture on a stream of the framework's choosing): as many lanes as
+    // streams of this device have run scratch-using calls, so that a warm-up which forks side
+    // streams as the capture will prepares a lane for each of them.
     if(bytes <= kMaxCaptureBytes[k])
     {
-        Arena* cap = find_arena(ctx.device_id, nullptr, true);
-        if(cap == nullptr && (cap = add_arena(ctx, true)) == nullptr)
-            return hipErrorOutOfMemory;
-        if((e = block_for(ctx, *cap, k, bytes, zeroed, false)) != hipSuccess)
-            return e;
+        int lanes = eager_streams_of(ctx.device_id);
+        lanes     = lanes < 1 ? 1 : (lanes > kCaptureLanes ? kCaptureLanes : lanes);
+        for(int lane = 0; lane < lanes; ++lane)
+        {
+            Arena* cap = find_lane(ctx.device_id, lane);
+            if(cap == nullptr && (cap = add_arena(ctx, true, lane)) == nullptr)
+                return hipErrorOutOfMemory;
+            // every kind this device has used so far, so that a new lane is as large as lane 0
+            for(int kk = 0; kk < (int)WsKind::kinds; ++kk)
+            {
+                const Arena* first = find_lane(ctx.device_id, 0);
+                size_t       need  = kk == k ? bytes : 0;
+                if(first != nullptr && first != cap && first->block[kk].bytes > need)
+                    need = first->block[kk].bytes;
+                if(need == 0)
+                    continue;
+                const bool clear = kk == (int)WsKind::split_tickets || (kk == k && zeroed);
+                if((e = block_for(ctx, *cap, kk, need, clear, true)) != hipSuccess)
+                    return e;
+            }
+        }
     }
     *out = mine;
     return hipSuccess;

@@ -165,98 +165,106 @@ def load_probes():
         lib.probe_stream.restype = ctypes.c_int
         lib.probe_stream.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
         lib.probe_mfma.restype = ctypes.c_int
-        lib.probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
-                                   ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+        lib.probe_mfma.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+                                   ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
         _probes = lib
     return _probes
 
 
 class GpuSampler:
-    """Samples the shader clock and the socket power of GPU 0 from a host thread while a
-    measurement runs: the amdgpu hwmon files where they can be read (freq1_input in Hz,
-    power1_average / power1_input in microwatts; about a millisecond per sample), else
-    `rocm-smi --showclocks --showpower --json` (a quarter of a second per sample)."""
+    """Samples the socket power and the shader clock of GPU 0 from a host thread while a
+    measurement runs.  Power: the amdgpu hwmon file power1_average / power1_input (microwatts).
+    Clock: hwmon freq1_input (Hz) or the starred line of pp_dpm_sclk where one of them can be read;
+    otherwise `rocm-smi --showclocks --json`, asked every tenth sample (it takes a quarter of a
+    second)."""
 
     def __init__(self, period=0.02):
         import glob
+        import shutil
 
         self.period = period
         self.samples = []  # (t, sclk_mhz or None, watts or None)
-        self.source = None
         self._stop = False
         self._thread = None
-        self.freq_file = self.power_file = None
-        for hw in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")):
-            f = os.path.join(hw, "freq1_input")
-            pw = [os.path.join(hw, n) for n in ("power1_average", "power1_input")]
-            pw = [q for q in pw if self._readable(q)]
-            if self._readable(f) or pw:
-                self.freq_file = f if self._readable(f) else None
-                self.power_file = pw[0] if pw else None
-                self.source = "hwmon " + hw
+        self.power_file = self.freq_file = self.dpm_file = None
+        for dev in sorted(glob.glob("/sys/class/drm/card*/device")):
+            for hw in sorted(glob.glob(os.path.join(dev, "hwmon", "hwmon*"))):
+                for n in ("power1_average", "power1_input"):
+                    if self.power_file is None and self._number(os.path.join(hw, n)) is not None:
+                        self.power_file = os.path.join(hw, n)
+                if self.freq_file is None and self._number(os.path.join(hw, "freq1_input")) is not None:
+                    self.freq_file = os.path.join(hw, "freq1_input")
+            if self.dpm_file is None and self._dpm(os.path.join(dev, "pp_dpm_sclk")) is not None:
+                self.dpm_file = os.path.join(dev, "pp_dpm_sclk")
+            if self.power_file or self.freq_file or self.dpm_file:
                 break
-        if self.source is None:
-            import shutil
-
-            if shutil.which("rocm-smi"):
-                self.source = "rocm-smi"
-                self.period = max(period, 0.25)
+        self.smi = shutil.which("rocm-smi") if not (self.freq_file or self.dpm_file) else None
+        self.source = {"power": self.power_file, "clock": self.freq_file or self.dpm_file or self.smi}
 
     @staticmethod
-    def _readable(path):
+    def _number(path):
         try:
             with open(path) as f:
-                float(f.read().strip())
-            return True
+                return float(f.read().strip())
         except (OSError, ValueError):
-            return False
+            return None
 
-    def _read_once(self):
-        if self.source is None:
-            return None, None
-        if self.source.startswith("hwmon"):
-            mhz = watts = None
-            try:
-                if self.freq_file:
-                    with open(self.freq_file) as f:
-                        mhz = float(f.read()) / 1e6
-                if self.power_file:
-                    with open(self.power_file) as f:
-                        watts = float(f.read()) / 1e6
-            except (OSError, ValueError):
-                pass
-            return mhz, watts
+    @staticmethod
+    def _dpm(path):
+        """MHz of the level that pp_dpm_sclk marks as current ("1: 2400Mhz *")."""
+        import re
+
+        try:
+            with open(path) as f:
+                for ln in f:
+                    if "*" in ln:
+                        m = re.search(r"(\d+(?:\.\d+)?)\s*mhz", ln.lower())
+                        if m:
+                            return float(m.group(1))
+        except OSError:
+            pass
+        return None
+
+    def _smi_clock(self):
         import re
         import subprocess
 
         try:
-            out = subprocess.run(["rocm-smi", "--showclocks", "--showpower", "--json"], capture_output=True, text=True,
-                                 timeout=5).stdout
+            out = subprocess.run([self.smi, "--showclocks", "--json"], capture_output=True, text=True, timeout=5).stdout
             card = json.loads(out)
             card = card[sorted(card)[0]]
+            for k, v in card.items():
+                if "sclk clock speed" in k.lower():
+                    m = re.search(r"(\d+(?:\.\d+)?)\s*mhz", str(v).lower())
+                    if m:
+                        return float(m.group(1))
         except Exception:
-            return None, None
-        mhz = watts = None
-        for k, v in card.items():
-            kl = k.lower()
-            if "sclk" in kl and mhz is None:
-                m = re.search(r"(\d+(?:\.\d+)?)\s*mhz", str(v).lower())
-                if m:
-                    mhz = float(m.group(1))
-            if "power" in kl and watts is None:
-                try:
-                    watts = float(str(v).split()[0])
-                except ValueError:
-                    pass
+            pass
+        return None
+
+    def _read_once(self, i):
+        watts = self._number(self.power_file) if self.power_file else None
+        if watts is not None:
+            watts /= 1e6
+        mhz = None
+        if self.freq_file:
+            mhz = self._number(self.freq_file)
+            mhz = mhz / 1e6 if mhz is not None else None
+        elif self.dpm_file:
+            mhz = self._dpm(self.dpm_file)
+        elif self.smi and i % 10 == 5:
+            mhz = self._smi_clock()
         return mhz, watts
 
     def __enter__(self):
         import threading
 
         def loop():
+            i = 0
             while not self._stop:
-                mhz, watts = self._read_once()
+                mhz, watts = self._read_once(i)
                 self.samples.append((time.perf_counter(), mhz, watts))
+                i += 1
                 time.sleep(self.period)
 
         self._thread = threading.Thread(target=loop, daemon=True)
@@ -272,8 +280,8 @@ class GpuSampler:
         sel = [x for x in self.samples if t_from <= x[0] <= t_to]
         clk = [x[1] for x in sel if x[1] is not None]
         pw = [x[2] for x in sel if x[2] is not None]
-        return {"sclk_mhz": sum(clk) / len(clk) if clk else None, "socket_watts": sum(pw) / len(pw) if pw else None,
-                "samples": len(sel), "source": self.source}
+        return {"sclk_mhz": sum(clk) / len(clk) if clk else None, "sclk_samples": len(clk),
+                "socket_watts": sum(pw) / len(pw) if pw else None, "power_samples": len(pw), "source": self.source}
 
 
 def sustained(torch, fn, seconds, launches_per_sync=4):
@@ -669,8 +677,8 @@ class ComputeCeiling:
         self.sink = torch.empty(self.cus * 512, dtype=torch.float32, device=dev)
         self.variant = (4, 512, self.real)
 
-    def _launch(self, fmas, threads, codes, iters):
-        rc = self.lib.probe_mfma(fmas, threads, codes[0].data_ptr(), codes[1].data_ptr(), self.scales.data_ptr(),
+    def _launch(self, fmas, threads, codes, iters, wide=0):
+        rc = self.lib.probe_mfma(fmas, threads, wide, codes[0].data_ptr(), codes[1].data_ptr(), self.scales.data_ptr(),
                                  self.sink.data_ptr(), iters, self.cus, self.torch.cuda.current_stream().cuda_stream)
         if rc != 0:
             raise RuntimeError(f"probe_mfma: hipError {rc}")
@@ -700,14 +708,17 @@ class ComputeCeiling:
             ("MFMA + 4 FMA, 4 waves per CU, config-4 codes", 4, 256, self.real),
             ("MFMA only, 4 waves per CU, config-4 codes", 0, 256, self.real),
             ("MFMA + 4 FMA, 8 waves per CU, all-zero codes", 4, 512, self.zero),
+            ("32x32x64 MFMA + 4 FMA per 16x16 of output, 8 waves per CU, config-4 codes", 4, 512, self.real, 1),
+            ("32x32x64 MFMA only, 8 waves per CU, config-4 codes", 0, 512, self.real, 1),
         ]
-        for what, fmas, threads, codes in variants:
+        for what, fmas, threads, codes, *wide in variants:
+            wide = wide[0] if wide else 0
             iters = self.ITERS if threads == 512 else 2 * self.ITERS
-            sec, n, smp = sustained(torch, lambda: self._launch(fmas, threads, codes, iters), self.SECONDS, 2)
+            sec, n, smp = sustained(torch, lambda: self._launch(fmas, threads, codes, iters, wide), self.SECONDS, 2)
             tf = self.flops_per_launch(threads, iters) / sec / 1e12
             row = {"what": what, "ms_per_launch": sec * 1e3, "launches_timed": n, "TFLOP/s": tf,
                    "frac_of_fp8_peak": tf / FP8_PEAK_TFLOPS,
-                   # clocks per MFMA slot and SIMD if the matrix pipe were never idle: 32
+                   # the clock at which a matrix pipe that is never idle would deliver this rate
                    "mfma_issue_ghz": (threads // 256) * iters * 32 * 32 / sec / 1e9}
             row.update(smp)
             out.append(row)

@@ -8,7 +8,8 @@
 //   probe_mfma     the prefill GEMM's arithmetic (v_mfma_f32_16x16x128_f8f6f4 on fp8 codes, four
 //                  v_fmac_f32 per MFMA that fold the product into fp32 accumulators with a scale, in
 //                  the product kernel's issue order) on operands that stay in registers: no LDS, no
-//                  global memory inside the loop, no barriers
+//                  global memory inside the loop, no barriers; also with the 32 x 32 x 64 shape of
+//                  the matrix instruction
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -128,11 +129,94 @@ __global__ __launch_bounds__(THREADS) void mfma_ceiling_kernel(const i32x8* __re
     sink[(size_t)blockIdx.x * THREADS + t] = s;
 }
 
+
+// The same arithmetic with v_mfma_f32_32x32x64_f8f6f4: a wave's 128 x 64 block is 4 x 2 tiles of
+// 32 x 32, each the sum of two chained matrix instructions per K block (64 of the 128 K values each),
+// folded into 16 accumulators per lane by 16 FMAs.  Same flops, same FMAs per flop, half as many
+// matrix instructions, twice as long each.  Tiles go in pairs (first halves of both, then second
+// halves), so a chained instruction never follows the one it depends on; a tile's FMAs trail its
+// second half by two slots.
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 template <int FMAS, int THREADS>
+__global__ __launch_bounds__(THREADS) void mfma32_ceiling_kernel(const i32x8* __restrict__ wcodes,
+                                                                 const i32x8* __restrict__ xcodes,
+                                                                 const float* __restrict__ scales,
+                                                                 float* __restrict__ sink, int iters)
+{
+    extern __shared__ uint8_t holds_the_compute_unit[];
+    const int t = threadIdx.x;
+    i32x8     aw[3], bx[2];
+    float     sc[2];
+#pragma unroll
+    for(int i = 0; i < 3; ++i)
+        aw[i] = wcodes[i * THREADS + t];
+#pragma unroll
+    for(int j = 0; j < 2; ++j)
+    {
+        bx[j] = xcodes[j * THREADS + t];
+        sc[j] = scales[j * THREADS + t];
+    }
+    f32x16 acc[8], P[4];
+#pragma unroll
+    for(int i = 0; i < 8; ++i)
+#pragma unroll
+        for(int r = 0; r < 16; ++r)
+            acc[i][r] = 0.f;
+#pragma unroll
+    for(int q = 0; q < 4; ++q)
+#pragma unroll
+        for(int r = 0; r < 16; ++r)
+            P[q][r] = 0.f;
+#pragma unroll
+    for(int i = 0; i < 3; ++i)
+        asm volatile("" : "+v"(aw[i]));
+#pragma unroll
+    for(int j = 0; j < 2; ++j)
+        asm volatile("" : "+v"(bx[j]), "+v"(sc[j]));
+#pragma unroll
+    for(int q = 0; q < 4; ++q)
+        asm volatile("" : "+v"(P[q]));
+    asm volatile("s_nop 7" ::: "memory");
+
+    for(int it = 0; it < iters; ++it)
+    {
+#pragma unroll
+        for(int s = 0; s < 16; ++s)
+        {
+            const int pair = s >> 2, tile = 2 * pair + (s & 1); // tile = (n tile i = tile >> 1, m tile j = tile & 1)
+            if((s & 2) == 0) // first half of the K block
+                asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, 0" : "=&v"(P[tile & 3]) : "v"(aw[(tile >> 1) % 3]), "v"(bx[tile & 1]));
+            else             // second half, onto the first (other fragments: the codes differ as in a real K block)
+                asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, %0" : "+v"(P[tile & 3]) : "v"(aw[((tile >> 1) + 1) % 3]), "v"(bx[(tile & 1) ^ 1]));
+            if constexpr(FMAS == 4)
+            {
+                // the tile whose second half was issued two slots ago: tile - 2 (the previous pair) for
+                // the slots of first halves
+                if((s & 2) == 0)
+                {
+                    const int done = (tile + 6) & 7;
+#pragma unroll
+                    for(int r = 0; r < 16; ++r)
+                        asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(acc[done][r]) : "v"(P[done & 3][r]), "v"(sc[done & 1]));
+                }
+            }
+        }
+    }
+    asm volatile("s_nop 15\n s_nop 15\n s_nop 15\n s_nop 15\n s_nop 15" ::: "memory");
+    float sum = P[0][0] + P[1][1] + P[2][2] + P[3][3];
+#pragma unroll
+    for(int i = 0; i < 8; ++i)
+#pragma unroll
+        for(int r = 0; r < 16; ++r)
+            sum += acc[i][r];
+    sink[(size_t)blockIdx.x * THREADS + t] = sum;
+}
+
+template <int FMAS, int THREADS, bool WIDE>
 hipError_t launch_mfma(const void* wcodes, const void* xcodes, const float* scales, float* sink, int iters,
                        int workgroups, hipStream_t stream)
 {
-    auto kernel = mfma_ceiling_kernel<FMAS, THREADS>;
+    auto kernel = WIDE ? mfma32_ceiling_kernel<FMAS, THREADS> : mfma_ceiling_kernel<FMAS, THREADS>;
     // 96 KiB of the 160 KiB of LDS: a second workgroup does not fit beside this one
     constexpr int kLds = 96 * 1024;
     hipError_t    e    = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
@@ -167,24 +251,31 @@ int probe_stream(int mode, const void* src, void* dst, uint64_t n_units, void* s
 }
 
 // `workgroups` workgroups of `threads` (256 or 512) lanes, one per compute unit, each wave running
-// `iters` passes of 32 matrix instructions (+ 128 FMAs with fmas = 4, none with fmas = 0).
+// `iters` passes of 32 matrix instructions (+ 128 FMAs with fmas = 4, none with fmas = 0); with
+// wide != 0, 16 instructions of the 32 x 32 x 64 shape per pass instead (512 lanes only).
 //   wcodes  8 * threads fragments of 32 bytes (fp8 codes), xcodes 4 * threads fragments,
 //   scales  4 * threads floats, sink workgroups * threads floats (written once at the end).
 // Flops per launch: workgroups * threads / 64 * iters * 32 * 65536.  Returns a hipError_t.
-int probe_mfma(int fmas, int threads, const void* wcodes, const void* xcodes, const float* scales, float* sink,
+int probe_mfma(int fmas, int threads, int wide, const void* wcodes, const void* xcodes, const float* scales, float* sink,
                int iters, int workgroups, void* stream)
 {
     hipStream_t s = (hipStream_t)stream;
     if(iters < 1 || workgroups < 1)
         return (int)hipErrorInvalidValue;
+    if(wide && fmas == 4 && threads == 512)
+        return (int)launch_mfma<4, 512, true>(wcodes, xcodes, scales, sink, iters, workgroups, s);
+    if(wide && fmas == 0 && threads == 512)
+        return (int)launch_mfma<0, 512, true>(wcodes, xcodes, scales, sink, iters, workgroups, s);
+    if(wide)
+        return (int)hipErrorInvalidValue;
     if(fmas == 4 && threads == 512)
-        return (int)launch_mfma<4, 512>(wcodes, xcodes, scales, sink, iters, workgroups, s);
+        return (int)launch_mfma<4, 512, false>(wcodes, xcodes, scales, sink, iters, workgroups, s);
     if(fmas == 0 && threads == 512)
-        return (int)launch_mfma<0, 512>(wcodes, xcodes, scales, sink, iters, workgroups, s);
+        return (int)launch_mfma<0, 512, false>(wcodes, xcodes, scales, sink, iters, workgroups, s);
     if(fmas == 4 && threads == 256)
-        return (int)launch_mfma<4, 256>(wcodes, xcodes, scales, sink, iters, workgroups, s);
+        return (int)launch_mfma<4, 256, false>(wcodes, xcodes, scales, sink, iters, workgroups, s);
     if(fmas == 0 && threads == 256)
-        return (int)launch_mfma<0, 256>(wcodes, xcodes, scales, sink, iters, workgroups, s);
+        return (int)launch_mfma<0, 256, false>(wcodes, xcodes, scales, sink, iters, workgroups, s);
     return (int)hipErrorInvalidValue;
 }
 

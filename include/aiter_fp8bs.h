@@ -19,9 +19,19 @@
  * reserved for graphs, which every eager call keeps at least as large as its own need (up to
  * 256 MiB of split-K partial tiles, 1 GiB of expert-layer intermediates).  So: run a call once
  * eagerly, on any stream of the device, before recording it; a call recorded without that fails
- * with a message.  Graphs of one device share that buffer with each other (never with eager
- * work): do not replay two of them concurrently.  Nothing else allocates, and nothing
- * synchronises.
+ * with a message.  Calls recorded on forked streams of ONE capture may run side by side when the
+ * graph is replayed: each stream of a capture that records a scratch-using call gets a part (lane)
+ * of the graph buffer to itself, and there are as many lanes (at most four) as streams of the
+ * device have run scratch-using calls eagerly -- a warm-up that forks side streams the way the
+ * capture will prepares them; a capture that forks wider is refused with a message (status -1,
+ * the capture stays valid).  Graphs of one device share the graph buffer with each other (never
+ * with eager work): do not replay two of them concurrently.  An eager call that has to allocate
+ * while another host thread is capturing a graph allocates with its own thread's capture mode
+ * set to relaxed (hipThreadExchangeStreamCaptureMode), which does not invalidate that capture;
+ * if the runtime refuses the allocation all the same, the call returns -1 with a message that
+ * says so.  When more than 1024 (device, stream) pairs have held scratch, the pair used longest
+ * ago hands its buffers on (after a device synchronisation).  Nothing else allocates, and
+ * nothing else synchronises.
  * Return value: 0 on success, -1 on failure with the message available from
  * aiter_get_last_error() (thread local).  No C++ exception crosses this boundary.
  *
@@ -183,8 +193,8 @@ int gemm_a8w8_blockscale(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t*
  * library routine).  A problem whose kernel needs more than the buffer holds is rejected with a
  * message (status -1).  Every call on a GPU uses that GPU's one buffer: calls that overlap on one
  * GPU (different streams, or a graph replay beside eager calls) race; calls on one stream are
- * ordered and safe.  The first call on a GPU enqueues one small fill kernel (which clears the
- * tickets) before the GEMM, on the caller's stream.
+ * ordered and safe.  Where the library chooses the K ranges itself (no count named by kernelName or
+ * splitK), it takes the best plan whose partial tiles fit the buffer.
  */
 int gemm_a8w8_blockscale_noalloc(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t* x_scale,
                                  aiter_tensor_t* w_scale, aiter_tensor_t* Out, int64_t splitK,

@@ -28,6 +28,15 @@ def test_fast_division_is_ieee_exact(checker, mode):
     assert out.stdout.startswith("OK")
 
 
+def test_capture_lane_bookkeeping(tmp_path):
+    """Streams of one capture sequence get scratch lanes of their own (two streams, two pointers),
+    a stream keeps its lane, a new sequence starts at lane 0: aiter_amd/csrc/capture_lanes.h on the host."""
+    exe = str(tmp_path / "capture_lanes_check")
+    subprocess.check_call(["g++", "-O1", "-std=c++17", "-o", exe, os.path.join(HERE, "host_math", "capture_lanes_check.cpp")])
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0 and out.stdout.startswith("OK"), out.stdout + out.stderr
+
+
 def test_kernel_choice_query_on_the_headline_shapes():
     """The shape rule that stands in for the reference's tuned-table lookup (get_CKGEMM_config,
     aiter/ops/gemm_op_a8w8.py:448-490) can be asked without a GPU."""

@@ -143,6 +143,107 @@ def test_growth_keeps_recorded_graphs_valid():
         assert torch.equal(out.view(torch.int16), eager.view(torch.int16))
 
 
+def test_forked_streams_of_one_capture_get_scratch_of_their_own():
+    # two split-K calls recorded on two forked streams of one capture may run side by side on replay:
+    # each stream of the capture gets a lane of the graph scratch to itself, provided as many streams
+    # ran scratch-using calls eagerly before (here: the warm-up forks the same way)
+    shapes = [(16, 1024, 7168), (32, 512, 4096)]
+    problems = [on_device(*make_problem(m, n, k, seed=51 + i)) for i, (m, n, k) in enumerate(shapes)]
+    main, side = torch.cuda.Stream(), torch.cuda.Stream()
+    eager = []
+    for st, p, (m, n, k) in zip((main, side), problems, shapes):
+        with torch.cuda.stream(st):
+            eager.append(gemm(p, n, m))
+    torch.cuda.synchronize()
+    outs = [torch.zeros(m, n, dtype=torch.bfloat16, device=DEV) for (m, n, k) in shapes]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(main):
+        with torch.cuda.graph(graph, stream=main):
+            side.wait_stream(main)
+            with torch.cuda.stream(side):
+                for _ in range(4):
+                    aiter_amd.gemm_a8w8_blockscale_ck(*problems[1], outs[1], splitK=-1)
+            for _ in range(4):
+                aiter_amd.gemm_a8w8_blockscale_ck(*problems[0], outs[0], splitK=-1)
+            main.wait_stream(side)
+    for _ in range(20):
+        for o in outs:
+            o.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for o, e in zip(outs, eager):
+            assert torch.equal(o.view(torch.int16), e.view(torch.int16))
+    # a capture that records such calls on more streams than there are lanes is refused with a message,
+    # and stays usable
+    forks = [torch.cuda.Stream() for _ in range(5)]
+    graph2 = torch.cuda.CUDAGraph()
+    refused = 0
+    with torch.cuda.stream(main):
+        with torch.cuda.graph(graph2, stream=main):
+            aiter_amd.gemm_a8w8_blockscale_ck(*problems[0], outs[0], splitK=-1)  # takes its lane first
+            for f in forks:
+                f.wait_stream(main)
+                with torch.cuda.stream(f):
+                    try:
+                        aiter_amd.gemm_a8w8_blockscale_ck(*problems[1], outs[1], splitK=-1)
+                    except RuntimeError as e:
+                        assert "more streams" in str(e)
+                        refused += 1
+                main.wait_stream(f)
+    assert refused >= 2  # at most four lanes, one of them the first stream's
+    outs[0].zero_()
+    graph2.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0].view(torch.int16), eager[0].view(torch.int16))
+
+
+def test_eager_growth_beside_another_threads_capture():
+    # thread A records a warmed call while thread B, on a stream that never held scratch, makes a call that
+    # must allocate: B's allocation happens with the thread's capture mode relaxed, so A's capture (global
+    # mode, torch's default) stays valid; should the runtime refuse B all the same, B gets the documented error
+    m, n, k = 16, 1024, 7168
+    a = on_device(*make_problem(m, n, k, seed=61))
+    want_a = gemm(a, n, m)
+    mb, nb, kb = 256, 2112, 7168
+    b = on_device(*make_problem(mb, nb, kb, seed=62))
+    want_b = gemm(b, nb, mb, kernel="mid_64x64:s=7")
+    torch.cuda.synchronize()
+    out_a = torch.zeros(m, n, dtype=torch.bfloat16, device=DEV)
+    out_b = torch.zeros(mb, nb, dtype=torch.bfloat16, device=DEV)
+    stream_a, stream_b = torch.cuda.Stream(), torch.cuda.Stream()
+    capture_open, b_done = threading.Event(), threading.Event()
+    b_error = []
+
+    def thread_b():
+        capture_open.wait(timeout=60)
+        try:
+            with torch.cuda.stream(stream_b):  # a fresh stream: its first scratch-using call allocates
+                aiter_amd.gemm_a8w8_blockscale_ck(*b, out_b, splitK=-1, kernelName="mid_64x64:s=7")
+        except RuntimeError as e:
+            b_error.append(str(e))
+        finally:
+            b_done.set()
+
+    tb = threading.Thread(target=thread_b)
+    tb.start()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream_a):
+        with torch.cuda.graph(graph, stream=stream_a):
+            capture_open.set()
+            assert b_done.wait(timeout=60)
+            aiter_amd.gemm_a8w8_blockscale_ck(*a, out_a, splitK=-1)
+    tb.join()
+    for _ in range(3):
+        out_a.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_a.view(torch.int16), want_a.view(torch.int16))
+    if b_error:
+        assert "another thread captures" in b_error[0], b_error
+    else:
+        assert torch.equal(out_b.view(torch.int16), want_b.view(torch.int16))
+
+
 @pytest.mark.parametrize("m,n,k,s", [(1040, 128, 7168, 2), (1934, 128, 7168, 1), (2000, 128, 7168, 2), (3258, 128, 7168, 3)])
 def test_tuned_rows_with_split_hint(m, n, k, s):
     # rows of the reference's tuned table with splitK > 0 and M >= 1024, forwarded as its callers do
