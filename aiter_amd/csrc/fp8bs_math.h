@@ -68,6 +68,18 @@ FP8BS_HD bool amax_allows_fast_path(uint32_t amax_bits)
     return amax_bits >= kFastAmaxMinBits && amax_bits <= kFastAmaxMaxBits;
 }
 
+// amax / 448 as IEEE division rounds it, without the division: the same three-operation sequence
+// as div_by_scale below with the constant RN(1/448).  Holds for every amax that is a 16-bit float
+// (bf16 or fp16, widened) inside the fast range; the CPU tests compare it with the division for
+// every such value.
+FP8BS_HD float amax_over_448(float m)
+{
+    const float c  = bits_f32(0x3b124925u); // RN(1 / 448)
+    const float q0 = m * c;
+    const float t  = fma32(q0, 448.0f, -m);
+    return fma32(-t, c, q0);
+}
+
 // Correctly rounded x / s from the correctly rounded reciprocal r = RN(1 / s):
 //     q0 = RN(x * r);  t = q0 * s - x (exact, one FMA);  q = RN(q0 - t * r)
 // With r = RN(1/s) this sequence returns RN(x / s) for binary32 operands whenever no

@@ -7,6 +7,7 @@
 //     bf16  every bf16 amax in the fast range x every bf16 |x| <= amax  (sampled exponents: all
 //           128 significands of amax at each of a set of exponents, all x codes)
 //     fp16  every fp16 amax x every fp16 |x| <= amax
+//     scale amax / 448 by multiplication and correction vs the IEEE division, every bf16 and fp16 amax
 //     cvt   software conversion vs oracle on structured fp32 inputs
 // Prints "OK <count>" or the first mismatches and exits non-zero.
 #include "../../aiter_amd/csrc/fp8bs_math.h"
@@ -85,6 +86,25 @@ int main(int argc, char** argv)
                 n += check_pair(oracle_f16_to_f32((uint16_t)xc), amax, bad);
             n += check_pair(amax, amax, bad);
         }
+    }
+    else if(strcmp(mode, "scale") == 0)
+    {
+        // amax / 448 without the division: every bf16 and every fp16 amax inside the fast range
+        for(int kind = 0; kind < 2; ++kind)
+            for(uint32_t ac = 1; ac < (kind == 0 ? 0x7f80u : 0x7c00u); ++ac)
+            {
+                const float amax = kind == 0 ? bf16f((uint16_t)ac) : oracle_f16_to_f32((uint16_t)ac);
+                if(!fp8bs::amax_allows_fast_path(fp8bs::f32_bits(amax)))
+                    continue;
+                const float want = amax / 448.0f, got = fp8bs::amax_over_448(amax);
+                ++n;
+                if(fp8bs::f32_bits(want) != fp8bs::f32_bits(got))
+                {
+                    if(bad < 10)
+                        fprintf(stderr, "amax=%a want=%a got=%a\n", amax, want, got);
+                    ++bad;
+                }
+            }
     }
     else if(strcmp(mode, "cvt") == 0)
     {
