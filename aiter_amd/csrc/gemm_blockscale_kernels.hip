@@ -171,9 +171,9 @@ const char* gemm_kernel_names() { return kKernelNames; }
 // faster: the streaming kernel where N / 16 row tiles with one K step per wave cover the chip
 // ((1 ... 64, 7168, 2048): 6.0 ... 8.6 us against 8.8 ... 10.0), the tilings from 17 rows on where K
 // is long or very short or N is large ((64, 24576, 1536): 12.6 us against 15.0; (64, 32768, 512): 7.1
-// against 17.5; (32, 4608, 7168): 11.8 against 17.3; (8, 4096, 11008): 13.9 against 17.9).  Below 8 rows
-// the tilings, which multiply 64 rows whatever M is, must be modelled 25 % faster to be taken (the
-// streaming kernel's model is fitted from 8 rows up and it gets faster below).  Above 64 rows, the 256-row
+// against 17.5; (32, 4608, 7168): 11.8 against 17.3; (8, 4096, 11008): 13.9 against 17.9; from one row
+// on where the weights are large: (1, 16384, 4096) 16.2 against 18.2, (1, 32768, 512) 6.2 against 6.9).
+// Above 64 rows, the 256-row
 // tiling or the mid_* tilings, whichever is modelled faster.  Measured on the DeepSeek shapes, a
 // 256x256 iteration over one K block takes 1.7 us while the tiles of a round cover up to 56 % of
 // the compute units and up to 2.1 us when they cover all of them, against 0.8 us for a quarter of
@@ -182,8 +182,7 @@ const char* gemm_kernel_names() { return kKernelNames; }
 static const char* automatic_choice(const GemmKernelParams& p)
 {
     const float prefill_us = gemm_prefill_plan(p, 256).us; // fitted on a 256-CU part, like the mid model
-    if(p.M <= 64 && gemm_decode_supports(p) &&
-       (!gemm_mid_supports(p) || gemm_mid_estimate_us(p) * (p.M < 8 ? 1.25f : 1.0f) >= gemm_decode_estimate_us(p)))
+    if(p.M <= 64 && gemm_decode_supports(p) && (!gemm_mid_supports(p) || gemm_mid_estimate_us(p) >= gemm_decode_estimate_us(p)))
         return "decode_stream";
     if(gemm_mid_supports(p) && (!gemm_prefill_supports(p) || gemm_mid_estimate_us(p) * 1.03f < prefill_us))
         return "mid_auto";

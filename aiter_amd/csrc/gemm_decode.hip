@@ -41,9 +41,8 @@ struct DecodeParams
     int32_t   m_chunks;     // chunks of MT x 16 activation rows a workgroup walks per row group
     int32_t   grid_x, waves; // launch dimensions, passed explicitly: the implicit ones cost a dependent load
     int32_t   xs_vec4;      // x_scale rows can be read four K blocks at a time (16-byte aligned)
-    float*    partial;      // [splits][n_groups][R * MT * 64] x 4 fp32 when splits > 1
+    float*    partial;      // [splits - 1][items][R * MT * 64] x 4 fp32 when splits > 1: all zero between launches
     uint32_t  partial_bytes;
-    uint32_t* tickets;      // [n_groups], zero between launches
 };
 
 __device__ __forceinline__ u32x2 pack4(const f32x4& v, bool bf)
@@ -63,7 +62,9 @@ constexpr int decode_max_waves()
 // SHUF: the weights are pre-shuffled (16,16): a lane's MFMA fragment is then two coalesced 16-byte
 // loads and needs no transposition.
 // CHUNKED (SINGLE only): more than 64 activation rows, walked in chunks of MT x 16 per row group.
-template <int MT, int R, bool SINGLE, bool FULL, bool SHUF, bool CHUNKED>
+// SPLIT: K is shared out over workgroups (p.splits > 1).  A template parameter so that the kernels
+// without K ranges carry none of the exchange code: its mere presence cost them 2-5 %.
+template <int MT, int R, bool SINGLE, bool FULL, bool SHUF, bool CHUNKED, bool SPLIT>
 __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kernel(DecodeParams p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -78,7 +79,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
     FP8BS_TOUCH(g.K); FP8BS_TOUCH(g.xs_m); FP8BS_TOUCH(g.xs_k);
     FP8BS_TOUCH(p.n_tiles); FP8BS_TOUCH(p.n_groups); FP8BS_TOUCH(p.kb_per_split); FP8BS_TOUCH(p.splits);
     FP8BS_TOUCH(p.bf16_out); FP8BS_TOUCH(p.xs_vec4); FP8BS_TOUCH(p.partial); FP8BS_TOUCH(p.partial_bytes);
-    FP8BS_TOUCH(p.tickets); FP8BS_TOUCH(p.grid_x); FP8BS_TOUCH(p.waves); FP8BS_TOUCH(p.m_chunks);
+    FP8BS_TOUCH(p.grid_x); FP8BS_TOUCH(p.waves); FP8BS_TOUCH(p.m_chunks);
 #undef FP8BS_TOUCH
 
     const int t = threadIdx.x, lane = t & 63;
@@ -111,28 +112,6 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
         const i32x4 hi = *(const i32x4*)(slot + lds_off(l16, 2 * kg + 1));
         return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     };
-
-    // activation rows this lane fetches (two per m tile: rows crow and 8 + crow of the tile) and
-    // the row whose scales it needs (rows past M re-read the last one, never stored), for the
-    // chunk of 64 rows that starts at m_base
-    const uint8_t* xrow[MT][2];
-    const float*   xsrow[MT];
-    auto           set_chunk = [&](int m_base) {
-#pragma unroll
-        for(int j = 0; j < MT; ++j)
-        {
-#pragma unroll
-            for(int h = 0; h < 2; ++h)
-                xrow[j][h] =
-                    g.xq + (size_t)min(m_base + j * 16 + h * 8 + crow, g.M - 1) * g.lda + cchunk[h] * 16;
-            xsrow[j] = g.xs + (size_t)min(m_base + j * 16 + l16, g.M - 1) * g.xs_m;
-        }
-    };
-    set_chunk(0);
-
-    i32x8 bx[MT][kStepKb];
-    float xsv[MT][kStepKb];
-    f32x4 acc[R][MT];
 
     // K block i of a step that starts at kb0 and holds nk (1..4) blocks; slots past the end
     // re-read the last block (a cache hit) and are never multiplied
@@ -177,6 +156,47 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                 s[r][i] = wsp[kslot(kb0, nk, i)];
         }
     };
+
+    // Long K (several steps per wave): the workgroup's first weight requests go out before anything
+    // else is set up (activation addresses, the reduction's bookkeeping: a few hundred instructions,
+    // which the requests' latency then covers; (16, 2112, 7168): 8.0 -> 7.5 us).  With one step per
+    // wave the requests of the first group, the activations and the second group stay together
+    // further down (hoisted, (1, 7168, 2048) ran 3 % slower).
+    // No branch around the requests: values that flow out of a branch get copied, and a copy waits
+    // for its load.  A wave whose step lies beyond the K range requests the row's last blocks and
+    // never uses them.
+    u32x4 raw_h[SINGLE ? 1 : R][kStepKb][2];
+    float ws_h[SINGLE ? 1 : R][kStepKb];
+    if constexpr(!SINGLE)
+    {
+        const int first_kb0 = kb_lo + wave * kStepKb;
+        const int first_nk  = max(0, min(kStepKb, kb_hi - first_kb0));
+        issue_w(blockIdx.x, min(first_kb0, FULL ? g.kblocks - kStepKb : g.kblocks - 1), max(first_nk, 1), raw_h, ws_h);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // activation rows this lane fetches (two per m tile: rows crow and 8 + crow of the tile) and
+    // the row whose scales it needs (rows past M re-read the last one, never stored), for the
+    // chunk of 64 rows that starts at m_base
+    const uint8_t* xrow[MT][2];
+    const float*   xsrow[MT];
+    auto           set_chunk = [&](int m_base) {
+#pragma unroll
+        for(int j = 0; j < MT; ++j)
+        {
+#pragma unroll
+            for(int h = 0; h < 2; ++h)
+                xrow[j][h] =
+                    g.xq + (size_t)min(m_base + j * 16 + h * 8 + crow, g.M - 1) * g.lda + cchunk[h] * 16;
+            xsrow[j] = g.xs + (size_t)min(m_base + j * 16 + l16, g.M - 1) * g.xs_m;
+        }
+    };
+    set_chunk(0);
+
+    i32x8 bx[MT][kStepKb];
+    float xsv[MT][kStepKb];
+    f32x4 acc[R][MT];
+
     auto issue_x = [&](int kb0, int nk, u32x4(&raw)[MT][kStepKb][2], float(&xs_out)[MT][kStepKb], int j_lo,
                        int j_hi) {
 #pragma unroll
@@ -296,9 +316,8 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
         }
     };
 
-    __shared__ uint32_t s_ticket;
     const __amdgpu_buffer_rsrc_t part_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(p.partial, 0, p.splits > 1 ? (int)p.partial_bytes : 0, 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc(p.partial, 0, SPLIT ? (int)p.partial_bytes : 0, 0x00020000);
     constexpr int kCoherent = 16; // cache-policy bit sc1: served by memory, not by a per-XCD L2
 
     // Per-wave partial tiles of a row group are parked in one of two LDS slots; they are added up
@@ -327,35 +346,50 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
             sum = w < nw ? sum + v[w] : sum;
         return sum;
     };
+    // K ranges of one item meet without a counter.  The workgroup of every range but the last
+    // writes its tile set to the exchange buffer and is done; the workgroup of the LAST range
+    // (dispatched after the others: it can only wait for workgroups that are already running or
+    // finished) reads them in range order, adds its own on top and stores the output -- so the
+    // result does not depend on timing.  The buffer is all zero between launches and a tile set
+    // is written as the complement of its bits: a 16-byte piece that still reads zero in any of
+    // its words has not arrived.  The reader polls lane by lane, past the caches, and puts the
+    // zeros back once it has the value.  (A partial sum whose bits are all ones -- one particular
+    // NaN, which no arithmetic here produces -- would read as zero for good: the wait is bounded,
+    // and a piece that never turns up is taken as it stands, which is that NaN.)  The workgroups
+    // of an item run on different XCDs, whose L2 caches are not coherent with each other: every
+    // access to the exchanged tiles bypasses them (sc1).
     auto flush_group_split = [&](int grp /* item */, const f32x4* red) {
         const size_t n_items = (size_t)p.n_groups * p.m_chunks;
-        // The workgroups that share a row group run on different XCDs, whose L2 caches are not
-        // coherent with each other; every access to the exchanged tiles therefore bypasses them
-        // (sc1), and the stores are waited for before the ticket is taken.
-        for(int e = t; e < E; e += (nw * 64))
+        const int    last    = p.splits - 1;
+        if(split != last)
         {
-            const f32x4    s   = wave_sum(red, e);
-            const uint32_t off = (uint32_t)(((size_t)split * n_items + grp) * E + e) * 16u;
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, s), part_rsrc, off, 0, kCoherent);
-        }
-        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): the stores above have reached memory
-        __syncthreads();
-        if(t == 0)
-            s_ticket = __hip_atomic_fetch_add(p.tickets + grp, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        if(s_ticket != (uint32_t)p.splits - 1)
+            for(int e = t; e < E; e += (nw * 64))
+            {
+                const u32x4    s   = ~__builtin_bit_cast(u32x4, wave_sum(red, e));
+                const uint32_t off = (uint32_t)(((size_t)split * n_items + grp) * E + e) * 16u;
+                __builtin_amdgcn_raw_buffer_store_b128(s, part_rsrc, off, 0, kCoherent);
+            }
             return;
-        if(t == 0) // leave the ticket ready for the next launch
-            __hip_atomic_store(p.tickets + grp, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        constexpr int kPollCoherent = 17;      // sc0 | sc1: never served by a cache
+        constexpr int kMaxPolls     = 1 << 16; // a tenth of a second, a thousand times a launch
         for(int e = t; e < E; e += (nw * 64))
         {
-            f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
-            for(int sp = 0; sp < p.splits; ++sp) // split order, whoever arrived last
+            const f32x4 own = wave_sum(red, e);
+            f32x4       s   = f32x4{0.f, 0.f, 0.f, 0.f};
+            for(int sp = 0; sp < last; ++sp) // range order, whenever they arrive
             {
                 const uint32_t off = (uint32_t)(((size_t)sp * n_items + grp) * E + e) * 16u;
-                s += __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, off, 0, kCoherent));
+                u32x4          v   = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, off, 0, kPollCoherent);
+                for(int polls = 0; (v[0] == 0u || v[1] == 0u || v[2] == 0u || v[3] == 0u) && polls < kMaxPolls; ++polls)
+                {
+                    __builtin_amdgcn_s_sleep(2);
+                    v = __builtin_amdgcn_raw_buffer_load_b128(part_rsrc, off, 0, kPollCoherent);
+                }
+                __builtin_amdgcn_raw_buffer_store_b128(u32x4{0u, 0u, 0u, 0u}, part_rsrc, off, 0, kCoherent);
+                s += __builtin_bit_cast(f32x4, ~v);
             }
-            store_out(grp, e, s);
+            store_out(grp, e, s + own);
         }
     };
     // adds up and stores the group parked in `slot`; the barrier makes every wave's tiles visible
@@ -363,7 +397,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
     auto flush_one = [&](int fgrp, int which) {
         __syncthreads();
         const f32x4* red = parked + (size_t)which * nw * E;
-        if(p.splits == 1)
+        if constexpr(!SPLIT)
         {
             // four elements per thread and pass, all LDS reads of a pass issued together
             const int T = (nw * 64);
@@ -585,6 +619,7 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
     else
     {
         // long K: every wave takes several steps; activations are re-read per item
+        bool first_step = true;
         for(; grp < p.n_groups; grp += stride)
             for(int chunk = 0; chunk < p.m_chunks; ++chunk)
             {
@@ -595,10 +630,12 @@ __global__ __launch_bounds__(64 * decode_max_waves<MT>()) void gemm_decode_kerne
                 for(int kb0 = kb_lo + wave * kStepKb; kb0 < kb_hi; kb0 += nw * kStepKb)
                 {
                     const int nk = min(kStepKb, kb_hi - kb0);
-                    u32x4     wraw[R][kStepKb][2];
+                    auto&     wraw = raw_h;
+                    auto&     wsv  = ws_h;
                     u32x4     xraw[MT][kStepKb][2];
-                    float     wsv[R][kStepKb];
-                    issue_w(grp, kb0, nk, wraw, wsv);
+                    if(!first_step) // (the workgroup's first step was requested at the top)
+                        issue_w(grp, kb0, nk, wraw, wsv);
+                    first_step = false;
                     issue_x(kb0, nk, xraw, xsv, 0, MT);
                     if(!flushed) // the previous item's sum, behind this item's first requests
                     {
@@ -636,10 +673,10 @@ int tuning_value(const char* tuning, const char* key)
     return 0;
 }
 
-template <int MT, int R, bool SINGLE, bool FULL, bool SHUF, bool CHUNKED = false>
-hipError_t launch_one(const DecodeParams& p, dim3 grid, int waves, size_t smem, hipStream_t stream)
+template <int MT, int R, bool SINGLE, bool FULL, bool SHUF, bool CHUNKED, bool SPLIT>
+hipError_t launch_split(const DecodeParams& p, dim3 grid, int waves, size_t smem, hipStream_t stream)
 {
-    auto        kernel = gemm_decode_kernel<MT, R, SINGLE, FULL, SHUF, CHUNKED>;
+    auto        kernel = gemm_decode_kernel<MT, R, SINGLE, FULL, SHUF, CHUNKED, SPLIT>;
     static std::atomic<bool> raised[kMaxDevices]; // dynamic LDS above the default limit needs opting in, once
     int         dev = 0;
     (void)hipGetDevice(&dev);
@@ -653,6 +690,13 @@ hipError_t launch_one(const DecodeParams& p, dim3 grid, int waves, size_t smem, 
     }
     hipLaunchKernelGGL(kernel, grid, dim3(64 * waves), smem, stream, p);
     return hipGetLastError();
+}
+
+template <int MT, int R, bool SINGLE, bool FULL, bool SHUF, bool CHUNKED = false>
+hipError_t launch_one(const DecodeParams& p, dim3 grid, int waves, size_t smem, hipStream_t stream)
+{
+    return p.splits > 1 ? launch_split<MT, R, SINGLE, FULL, SHUF, CHUNKED, true>(p, grid, waves, smem, stream)
+                        : launch_split<MT, R, SINGLE, FULL, SHUF, CHUNKED, false>(p, grid, waves, smem, stream);
 }
 
 template <int MT, int R, bool SHUF>
@@ -730,11 +774,18 @@ static DecodePlan plan_decode(const GemmKernelParams& g, int split_k_log2, const
             splits = 1 << split_k_log2;
         else
         {
-            // Split K across workgroups only while every workgroup still gets a compute unit of
-            // its own (one workgroup fills a compute unit's registers) and at least two steps.
-            splits = kChipCus / d.n_groups;
-            if(splits > d.steps / 2)
-                splits = d.steps / 2;
+            // K ranges across workgroups while the row groups alone leave compute units idle.  Best
+            // is one step per wave (four steps per range: every wave of a workgroup requests its whole
+            // share at once and the waves finish together), as long as that keeps the launch within
+            // about two workgroups per compute unit; otherwise as many ranges as that limit allows.
+            // ((1, 512 ... 1536, 7168): four ranges 5.4 / 5.8 / 6.4 us against 6.0 / 5.8 / 6.7 with 7 / 4 / 2;
+            // (1, 2112, 7168): three ranges 7.4 us against 8.5 with one; (1, 3072, 7168): two, 8.4 against 9.2;
+            // (1, 1024, 4096): two, 4.7 against 5.1 with four; one step per range is never worth the exchange.)
+            const int one_step_per_wave = (d.steps + max_waves - 1) / max_waves;
+            if(d.n_groups * one_step_per_wave <= 2 * kChipCus - kChipCus / 4)
+                splits = one_step_per_wave;
+            else
+                splits = std::min(one_step_per_wave, (2 * kChipCus) / d.n_groups);
             if(splits < 1)
                 splits = 1;
         }
@@ -803,7 +854,10 @@ float gemm_decode_estimate_us(const GemmKernelParams& g)
     const float ragged_k = d.full ? 1.f : 1.3f;
     if(d.single)
         return ragged_k * (3.59f + 0.107f * w / share + 0.038f * mt * w + 2.9f * part + 0.44f * wide_split + 0.10f * mt);
-    return ragged_k *
+    // (K ranges that meet without a counter: 15 % below what the terms, fitted with a counter, say --
+    // (1 ... 32, 4096, 7168) 8.8 ... 10.8 us against 10.1 ... 13.5)
+    const float ranges = d.splits > 1 ? 0.85f : 1.f;
+    return ragged_k * ranges *
            (4.67f + 0.141f * w / share + 0.021f * a + 0.029f * mt * w + 3.78f * out + 0.65f * wide_split + 0.38f * mt);
 }
 
@@ -828,16 +882,19 @@ hipError_t launch_gemm_decode(const GemmKernelParams& g, In16 out_dtype, int spl
     WorkspaceLock lock(splits > 1);
     if(splits > 1)
     {
-        const size_t bytes = (size_t)splits * p.n_groups * p.m_chunks * tile_set;
+        // the exchange buffer of the K ranges: zero between launches (the kernel puts the zeros back)
+        const size_t bytes = (size_t)(splits - 1) * p.n_groups * p.m_chunks * tile_set;
         if(bytes >= ((size_t)1 << 31))
         {
             if(ctx.why)
                 *ctx.why = "decode_stream: the partial tiles of this many K ranges exceed 2 GiB";
             return hipErrorInvalidValue;
         }
-        hipError_t e = split_workspace(ctx, lock, bytes, (size_t)p.n_groups * p.m_chunks, &p.partial, &p.tickets);
+        void*      block = nullptr;
+        hipError_t e     = workspace_acquire(ctx, lock, WsKind::split_tickets, bytes, true, &block);
         if(e != hipSuccess)
             return e;
+        p.partial       = (float*)block;
         p.partial_bytes = (uint32_t)bytes;
     }
 

@@ -38,7 +38,7 @@ namespace fp8bs {
 enum class WsKind : int
 {
     split_partial = 0, // fp32 partial tiles of K split across workgroups
-    split_tickets,     // arrival counters, zero between launches
+    split_tickets,     // arrival counters and exchange slots: all zero between launches (their users put the zeros back)
     moe_sort,          // histograms and expert offsets of the sorting kernels
     moe_layer,         // intermediates of the expert layer
     kinds
@@ -46,7 +46,7 @@ enum class WsKind : int
 
 // what the static buffer holds: partial tiles, then tickets
 constexpr size_t kStaticPartialBytes = (size_t)32 << 20;
-constexpr size_t kStaticTickets      = 16384;
+constexpr size_t kStaticTickets      = (size_t)1 << 20; // 32-bit words: 4 MiB
 
 // What a launcher needs to know about the call it serves besides the operands.
 struct LaunchCtx

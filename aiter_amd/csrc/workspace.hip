@@ -249,8 +249,8 @@ hipError_t workspace_acquire(const LaunchCtx& ctx, const WorkspaceLock& held, Ws
             say(ctx, partial ? "the kernel for this problem needs more than the 32 MiB of split-K partial tiles that "
                                "the static scratch buffer holds: use the allocating entry point, or ask for fewer K "
                                "ranges (kernelName / splitK)"
-                             : "the kernel for this problem needs more than the 16384 split-K tickets that the static "
-                               "scratch buffer holds: use the allocating entry point");
+                             : "the kernel for this problem needs more than the 4 MiB of split-K counters and exchange "
+                               "slots that the static scratch buffer holds: use the allocating entry point");
             return hipErrorInvalidValue;
         }
         unsigned char* base = nullptr;

@@ -188,7 +188,7 @@ int gemm_a8w8_blockscale(aiter_tensor_t* XQ, aiter_tensor_t* WQ, aiter_tensor_t*
  * capture that was never run eagerly, tight serving loops, harnesses that forbid hipMalloc).  It
  * has no counterpart in the reference.  Same operands, same kernels, same results bit for bit;
  * the split-K scratch (fp32 partial tiles, tickets) comes from a fixed buffer in device memory
- * that the library's code object carries: 32 MiB of partial tiles and 16384 tickets per GPU, held
+ * that the library's code object carries: 32 MiB of partial tiles and 4 MiB of counters and exchange slots per GPU, held
  * until the process ends.  The call allocates nothing (no hipMalloc, hipFree or allocating
  * library routine).  A problem whose kernel needs more than the buffer holds is rejected with a
  * message (status -1).  Every call on a GPU uses that GPU's one buffer: calls that overlap on one

@@ -45,10 +45,10 @@ def test_kernel_choice_query_on_the_headline_shapes():
     names = set(aiter_amd.gemm_kernel_names())
     for m in (1, 16, 64):
         for n, k in ((7168, 2048), (24576, 1536), (2112, 7168)):
-            # the weight-streaming kernel for single rows, and everywhere on the shape whose N / 16 row tiles
+            # the weight-streaming kernel up to 16 rows, and everywhere on the shape whose N / 16 row tiles
             # with one K step per wave cover the chip; the mid_* tilings where they are modelled (and
-            # measured) faster: at 64 rows on the other two shapes, from 8 rows on with K = 7168
-            want = "decode_stream" if m == 1 or (n, k) == (7168, 2048) or (m, n) == (16, 24576) else "mid_"
+            # measured) faster: at 64 rows on the other two shapes
+            want = "decode_stream" if m <= 16 or (n, k) == (7168, 2048) else "mid_"
             assert aiter_amd.get_CKGEMM_config(m, n, k)["kernelName"].startswith(want)
     assert aiter_amd.get_CKGEMM_config(8192, 36864, 7168)["kernelName"] == "prefill_256x256"
     cfg5 = aiter_amd.get_CKGEMM_config(2048, 4096, 7168)  # 128 tiles: two K ranges per tile

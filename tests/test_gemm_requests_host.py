@@ -59,3 +59,25 @@ def test_split_hint_range_and_names():
         _ffi.gemm_resolve(16, 256, 512, 0, "mid_128x128:s=0")
     assert _ffi.gemm_resolve(16, 256, 512, 2, "decode_stream:r=2,s=4") == ("decode_stream:r=2,s=4", 2)
     assert _ffi.gemm_resolve(300, 256, 512, 1, "prefill_256x256:s=2") == ("prefill_256x256:s=2", 1)
+
+
+def test_choice_below_65_rows_against_measured_durations():
+    """The automatic choice between the weight-streaming kernel and the mid_* tilings, held against
+    durations of both measured on an MI355X (tests/golden/choice_grid_m1_to_64.json, written by
+    tests/golden/measure_choice_grid.py: 1 ... 64 rows x fourteen weight shapes): what the choice
+    loses against the faster family is 1 % at most on average and 10 % at worst, and where one
+    family is ahead by a quarter the choice takes it."""
+    import json
+
+    with open(os.path.join(os.path.dirname(__file__), "golden", "choice_grid_m1_to_64.json")) as f:
+        rows = json.load(f)["rows"]
+    assert len(rows) == 98
+    losses = []
+    for r in rows:
+        chosen = "decode_stream" if _ffi.gemm_choice(r["M"], r["N"], r["K"]).startswith("decode_stream") else "mid_auto"
+        other = "mid_auto" if chosen == "decode_stream" else "decode_stream"
+        losses.append(r[chosen] / min(r["decode_stream"], r["mid_auto"]) - 1.0)
+        assert r[chosen] <= 1.10 * r[other], (r, chosen)
+        if r[other] > 1.25 * r[chosen] or r[chosen] > 1.25 * r[other]:
+            assert r[chosen] < r[other], (r, chosen)
+    assert sum(losses) / len(losses) <= 0.01, sum(losses) / len(losses)
