@@ -513,11 +513,18 @@ struct MoeGemmParams
 };
 
 // fragment of a pre-shuffled weight tile's K block: 2 KiB, lane (l16, kg) takes the 16 bytes at
-// kg*512 + l16*16 and the 16 bytes 256 further on
+// kg*512 + l16*16 and the 16 bytes 256 further on.  STREAM: the expert's weights are read by this
+// block of rows only, so the loads are non-temporal (long-lived workgroups that stream with
+// ordinary loads reach 5.7 TB/s here, with non-temporal ones 6.3-6.5 TB/s, whatever the order in
+// which a workgroup walks its tiles); an expert with several blocks is read with ordinary loads,
+// which let the later blocks find the weights in a cache.
+template <bool STREAM>
 __device__ __forceinline__ i32x8 load_w_fragment(const uint8_t* tile_kb, int l16, int kg)
 {
-    const i32x4 lo = *(const i32x4*)(tile_kb + kg * 512 + l16 * 16);
-    const i32x4 hi = *(const i32x4*)(tile_kb + kg * 512 + 256 + l16 * 16);
+    const i32x4* lo_at = (const i32x4*)(tile_kb + kg * 512 + l16 * 16);
+    const i32x4* hi_at = (const i32x4*)(tile_kb + kg * 512 + 256 + l16 * 16);
+    const i32x4  lo    = STREAM ? __builtin_nontemporal_load(lo_at) : *lo_at;
+    const i32x4  hi    = STREAM ? __builtin_nontemporal_load(hi_at) : *hi_at;
     return i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 }
 // fragment of a row-major activation row's K block: 32 contiguous bytes at kg*32
@@ -535,6 +542,15 @@ __device__ __forceinline__ float activate(float g, int activation)
     return 0.5f * g * (1.f + erff(g * 0.70710678118654752f)); // gelu (erf form)
 }
 
+// whether block `blk` is the only block of rows of its expert (its neighbours in the sorted order
+// belong to other experts or lie past the valid rows)
+__device__ __forceinline__ bool only_block_of_its_expert(const MoeGemmParams& p, int blk, int expert)
+{
+    const bool prev = blk > 0 && p.sorted_expert_ids[(blk - 1) >> p.expert_shift] == expert;
+    const bool next = (blk + 1) * p.block_rows < p.num_valid[0] && p.sorted_expert_ids[(blk + 1) >> p.expert_shift] == expert;
+    return !prev && !next;
+}
+
 // First GEMM + activation.  Workgroup = (block of 32 sorted rows, NT x 16 inter columns): NT
 // gate tiles and the NT matching up tiles; NT is picked at launch (wide units, which re-read the
 // activations less often, where they cover the chip and their last round of workgroups is expected
@@ -550,7 +566,7 @@ __device__ __forceinline__ float activate(float g, int activation)
 // the unit's share of HBM
 constexpr int kGateUpWaves = 8;
 
-template <int MT, int NT>
+template <int MT, int NT, bool STREAM>
 __device__ __forceinline__ void gate_up_body(const MoeGemmParams& p, float* red, int blk, int grp, int expert)
 {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
@@ -585,8 +601,8 @@ __device__ __forceinline__ void gate_up_body(const MoeGemmParams& p, float* red,
 #pragma unroll
         for(int i = 0; i < NT; ++i)
         {
-            w[i]      = load_w_fragment(wg + i * tile_stride + (size_t)kb * 2048, l16, kg);
-            w[NT + i] = load_w_fragment(wu + i * tile_stride + (size_t)kb * 2048, l16, kg);
+            w[i]      = load_w_fragment<STREAM>(wg + i * tile_stride + (size_t)kb * 2048, l16, kg);
+            w[NT + i] = load_w_fragment<STREAM>(wu + i * tile_stride + (size_t)kb * 2048, l16, kg);
         }
 #pragma unroll
         for(int j = 0; j < MT; ++j)
@@ -672,16 +688,17 @@ __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmP
     }
     // rows of a block are real pairs first, padding after: the second 16 rows matter only if row 16 is real
     const bool second_half = p.block_rows == 32 && (p.sorted_ids[blk * 32 + 16] & 0xffffff) < p.M;
+    const bool once = only_block_of_its_expert(p, blk, expert);
     if(second_half)
-        gate_up_body<2, NT>(p, red_dyn, blk, grp, expert);
+        once ? gate_up_body<2, NT, true>(p, red_dyn, blk, grp, expert) : gate_up_body<2, NT, false>(p, red_dyn, blk, grp, expert);
     else
-        gate_up_body<1, NT>(p, red_dyn, blk, grp, expert);
+        once ? gate_up_body<1, NT, true>(p, red_dyn, blk, grp, expert) : gate_up_body<1, NT, false>(p, red_dyn, blk, grp, expert);
 }
 
 // Second GEMM.  Workgroup = (block of 32 sorted rows, 512 output columns), wave = 128 columns =
 // 8 weight tiles walked two at a time with the next two already requested; the block's
 // activation rows (K = inter_dim, at most 4 K blocks on this path) stay in registers.
-template <int MT, int KB>
+template <int MT, int KB, bool STREAM>
 __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int grp, int expert)
 {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
@@ -714,7 +731,7 @@ __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int g
         for(int i = 0; i < 2; ++i)
 #pragma unroll
             for(int kb = 0; kb < KB; ++kb)
-                w[i][kb] = load_w_fragment(wt + (size_t)(pair * 2 + i) * tile_stride + (size_t)kb * 2048, l16, kg);
+                w[i][kb] = load_w_fragment<STREAM>(wt + (size_t)(pair * 2 + i) * tile_stride + (size_t)kb * 2048, l16, kg);
     };
     auto finish = [&](int pair, const i32x8 (&w)[2][KB]) {
 #pragma unroll
@@ -772,21 +789,17 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeGemmParams p)
     if(expert < 0 || expert >= p.experts)
         return;
     const bool second_half = p.block_rows == 32 && (p.sorted_ids[blk * 32 + 16] & 0xffffff) < p.M;
+    const bool once = only_block_of_its_expert(p, blk, expert);
     if(second_half)
-        down_body<2, KB>(p, blk, grp, expert);
+        once ? down_body<2, KB, true>(p, blk, grp, expert) : down_body<2, KB, false>(p, blk, grp, expert);
     else
-        down_body<1, KB>(p, blk, grp, expert);
+        once ? down_body<1, KB, true>(p, blk, grp, expert) : down_body<1, KB, false>(p, blk, grp, expert);
 }
 
 // The same for any K: workgroup = (block, 256 columns), wave = 64 columns, K blocks walked in turn.
-__global__ __launch_bounds__(256) void moe_down_long_k_kernel(MoeGemmParams p)
+template <bool STREAM>
+__device__ __forceinline__ void down_long_k_body(const MoeGemmParams& p, int blk, int grp, int expert)
 {
-    const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
-    if(blk * p.block_rows >= p.num_valid[0])
-        return;
-    const int expert = p.sorted_expert_ids[blk >> p.expert_shift];
-    if(expert < 0 || expert >= p.experts)
-        return;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
     const int n0 = grp * 256 + wave * 64;
     if(n0 >= p.N)
@@ -818,7 +831,7 @@ __global__ __launch_bounds__(256) void moe_down_long_k_kernel(MoeGemmParams p)
         i32x8 w[4], x[2];
 #pragma unroll
         for(int i = 0; i < 4; ++i)
-            w[i] = load_w_fragment(wt + (size_t)i * 16 * (size_t)p.K + (size_t)kb * 2048, l16, kg);
+            w[i] = load_w_fragment<STREAM>(wt + (size_t)i * 16 * (size_t)p.K + (size_t)kb * 2048, l16, kg);
         float       sc[2];
         const float wsv = wsr[kb];
 #pragma unroll
@@ -853,6 +866,20 @@ __global__ __launch_bounds__(256) void moe_down_long_k_kernel(MoeGemmParams p)
                 *(u32x2*)(p.out + slot * p.N + col) = u32x2{pack2<In16::bf16>(acc[j][i][0], acc[j][i][1]),
                                                             pack2<In16::bf16>(acc[j][i][2], acc[j][i][3])};
         }
+}
+
+__global__ __launch_bounds__(256) void moe_down_long_k_kernel(MoeGemmParams p)
+{
+    const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
+    if(blk * p.block_rows >= p.num_valid[0])
+        return;
+    const int expert = p.sorted_expert_ids[blk >> p.expert_shift];
+    if(expert < 0 || expert >= p.experts)
+        return;
+    if(only_block_of_its_expert(p, blk, expert))
+        down_long_k_body<true>(p, blk, grp, expert);
+    else
+        down_long_k_body<false>(p, blk, grp, expert);
 }
 
 
@@ -905,13 +932,18 @@ __device__ __forceinline__ void cols_load16(i32x4& d, const void* p)
 {
     asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(d) : "v"(p) : "memory");
 }
+// weights: read once, non-temporal (see load_w_fragment)
+__device__ __forceinline__ void cols_load16_nt(i32x4& d, const void* p)
+{
+    asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(d) : "v"(p) : "memory");
+}
 __device__ __forceinline__ void cols_load16_at16(i32x4& d, const void* p)
 {
     asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=v"(d) : "v"(p) : "memory");
 }
 __device__ __forceinline__ void cols_load16_at256(i32x4& d, const void* p)
 {
-    asm volatile("global_load_dwordx4 %0, %1, off offset:256" : "=v"(d) : "v"(p) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, off offset:256 nt" : "=v"(d) : "v"(p) : "memory");
 }
 __device__ __forceinline__ void cols_load4(float& d, const void* p)
 {
@@ -1023,9 +1055,9 @@ __global__ __launch_bounds__(256) void moe_down_cols_kernel(DownColsParams p)
         const int      expert = (int)(b >> 16);
         s.mask                = b & 0xffffu;
         const uint8_t* wp     = wlane + (size_t)expert * wexp;
-        cols_load16(s.wlo[0], wp);
+        cols_load16_nt(s.wlo[0], wp);
         cols_load16_at256(s.whi[0], wp);
-        cols_load16(s.wlo[1], wp + wtile);
+        cols_load16_nt(s.wlo[1], wp + wtile);
         cols_load16_at256(s.whi[1], wp + wtile);
         cols_load4(s.ws, wslane + (size_t)expert * wsexp);
         // rows that are padding read the unit's first real row instead: same cache lines, no traffic
