@@ -660,8 +660,13 @@ template <int NT>
 __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmParams p)
 {
     __shared__ __attribute__((aligned(16))) float red_dyn[kGateUpWaves * 2 * NT * 64 * 4];
-    const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
-    if(blk * p.block_rows >= p.num_valid[0])
+    // Blocks are taken from the last valid one down: the experts with the highest ids come first.  A
+    // shared expert, which every token is routed to and which conventionally has the last id, has the
+    // most blocks, each of two full row tiles and read with ordinary loads: started first, they are not
+    // what the launch ends on.
+    const int at = blockIdx.x / p.n_groups, grp = blockIdx.x - at * p.n_groups;
+    const int blk = (p.num_valid[0] + p.block_rows - 1) / p.block_rows - 1 - at;
+    if(blk < 0)
         return;
     const int expert = p.sorted_expert_ids[blk >> p.expert_shift];
     if(expert < 0 || expert >= p.experts)
