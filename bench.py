@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the FP8 block-scale path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload quant|prefill|decode|decode9|sweep|moe|fused|stream|ceiling]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload quant|prefill|decode|decode9|sweep|moe|fused|norm|stream|ceiling]
                     [--no-also] [--no-cpu]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
@@ -56,7 +56,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="quant", choices=["quant", "prefill", "decode", "decode9", "sweep", "moe", "fused", "copy", "stream", "ceiling"],
+    ap.add_argument("--workload", default="quant", choices=["quant", "prefill", "decode", "decode9", "sweep", "moe", "fused", "norm", "copy", "stream", "ceiling"],
                     help="'copy' is a plain 1 GiB device copy used to calibrate the rocprofv3 FETCH_SIZE / "
                     "WRITE_SIZE counters; it is not part of the path")
     ap.add_argument("--no-also", action="store_true", help="time only the primary workload")
@@ -68,6 +68,7 @@ def parse_args():
                     "(16,16) with column-major x_scale (gemm_a8w8_blockscale_bpreshuffle)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--kernel-name", default="", help="kernelName handed to the expert kernel of --workload moe")
+    ap.add_argument("--rows", type=int, default=2048, help="rows of --workload norm (config 5 has 2048)")
     return ap.parse_args()
 
 
@@ -507,6 +508,22 @@ class FusedWorkload:
         self.aiter.gemm_a8w8_blockscale_ck(self.y, self.wq, self.s, self.ws, self.out, splitK=-1)
 
     def step_norm_only(self):
+        # For the norm's own share of HBM: rows, codes and scales rotate through enough sets (640 MB, more
+        # than twice the 256 MB last-level cache) that no launch finds its input in a cache.  The fused
+        # step above keeps one set, as a layer does whose input the previous kernel has just written.
+        if not hasattr(self, "rot"):
+            import torch
+
+            sets = -(-640_000_000 // self.norm_bytes())
+            self.rot = [(self.x.clone(), torch.empty_like(self.y), torch.empty_like(self.s)) for _ in range(sets)]
+            self.rot_i = 0
+        x, y, s = self.rot[self.rot_i]
+        self.rot_i = (self.rot_i + 1) % len(self.rot)
+        self.aiter.rmsnorm2d_fwd_with_dynamicquant(y, x, s, self.nw, 1e-6, 0, group_size=128)
+
+    def step_norm_cached(self):
+        # the same on the fused step's one set of buffers: what the kernel takes inside a layer, where the
+        # 256 MB last-level cache still holds the rows the previous kernel wrote
         self.aiter.rmsnorm2d_fwd_with_dynamicquant(self.y, self.x, self.s, self.nw, 1e-6, 0, group_size=128)
 
     def describe(self):
@@ -742,6 +759,27 @@ class ComputeCeiling:
         return None
 
 
+class NormWorkload(FusedWorkload):
+    """The norm + quant half of config 5 by itself, on rows that come from HBM (buffers rotate)."""
+    name = "norm"
+
+    def __init__(self, rows=2048):
+        self.M = rows
+
+    def step(self):
+        self.step_norm_only()
+
+    def describe(self):
+        return {"workload": f"fused RMSNorm + 1x128 FP8 quant on x bf16 [{self.M},{self.K}] (config 5's first half), "
+                "inputs and outputs rotating through 640 MB", "M": self.M, "K": self.K, "kernel": "rmsnorm_kernel"}
+
+    def result(self, sec):
+        gb = self.norm_bytes() / sec / 1e9
+        roof = {"bound": "hbm", "achieved": gb, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gb / HBM_PEAK_GBS,
+                "traffic": None}
+        return gb, "GB/s", roof
+
+
 class DecodeAllWorkload:
     """All nine decode shapes of config 3, one launch each per step (shape after shape, so a kernel
     trace of the run lists them in DECODE_SHAPES order)."""
@@ -940,6 +978,9 @@ class MoeWorkload:
         return None
 
 
+ARGS_ROWS = [2048]  # --rows, for --workload norm
+
+
 def make_workload(name):
     if name == "moe":
         return MoeWorkload()
@@ -962,6 +1003,8 @@ def make_workload(name):
                             "config 3: decode blockscale GEMM M=64 N=24576 K=1536 (largest of the nine decode shapes)")
     if name == "fused":
         return FusedWorkload()
+    if name == "norm":
+        return NormWorkload(ARGS_ROWS[0])
     if name == "decode9":
         return DecodeAllWorkload()
     raise ValueError(name)
@@ -985,6 +1028,7 @@ def main():
     GemmWorkload.layout = args.layout
     GemmWorkload.rotate_mb = args.rotate_mb
     MoeWorkload.kernel_name = args.kernel_name
+    ARGS_ROWS[0] = args.rows
     wl = make_workload(args.workload)
     wl.setup(torch, dev)
     sec = time_steps(torch, wl.step, args.steps, args.warmup)
@@ -1041,7 +1085,10 @@ def main():
             if name == "fused":
                 sn = time_steps(torch, w2.step_norm_only, 30, 3, settle=True)
                 gb = w2.norm_bytes() / sn / 1e9
-                entry["norm_quant"] = {"us": sn * 1e6, "GB/s": gb, "frac_of_hbm_peak": gb / HBM_PEAK_GBS}
+                sc = time_steps(torch, w2.step_norm_cached, 30, 3, settle=True)
+                entry["norm_quant"] = {"us": sn * 1e6, "GB/s": gb, "frac_of_hbm_peak": gb / HBM_PEAK_GBS,
+                                       "buffers": "rotating through 640 MB: every launch reads its rows from HBM",
+                                       "us_with_rows_in_last_level_cache": sc * 1e6}
             if not args.no_cpu and name in ("prefill", "fused"):
                 torch.set_num_threads(os.cpu_count() or 1)
                 entry["cpu_baseline"] = w2.cpu_baseline(torch)
