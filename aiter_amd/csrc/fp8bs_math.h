@@ -80,6 +80,33 @@ FP8BS_HD float amax_over_448(float m)
     return fma32(-t, c, q0);
 }
 
+// RN(1 / s) for 2^-100 <= |s| <= 2^100 without the division sequence (13 instructions with its scaling
+// and fix-up): the hardware's reciprocal approximation and one Newton step.  Equal to the IEEE
+// division for every float in that range (all 1.68e9 of them are compared on the GPU by
+// tests/gpu_math); outside the range callers divide.  The host form is the division itself.
+constexpr uint32_t kRecipMinBits = (127u - 100u) << 23;
+constexpr uint32_t kRecipMaxBits = (127u + 100u) << 23;
+FP8BS_HD float recip_in_range(float s)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    const float r0 = __builtin_amdgcn_rcpf(s);
+    return fma32(fma32(-s, r0, 1.0f), r0, r0);
+#else
+    return 1.0f / s;
+#endif
+}
+
+// RN(a / n) in fp64 from inv = RN(1 / n): q0 = RN(a * inv), the exact residual a - q0 * n by one FMA,
+// one correction (the quotient is then the correctly rounded one provided inv is and n's significand
+// is not all ones: n is a row length here).  An infinite a stays infinite (its residual is NaN).
+FP8BS_HD double div_by_count(double a, double n, double inv)
+{
+    const double q0 = a * inv;
+    const double r  = __builtin_fma(-q0, n, a);
+    const double q  = __builtin_fma(r, inv, q0);
+    return r == r ? q : q0;
+}
+
 // Correctly rounded x / s from the correctly rounded reciprocal r = RN(1 / s):
 //     q0 = RN(x * r);  t = q0 * s - x (exact, one FMA);  q = RN(q0 - t * r)
 // With r = RN(1/s) this sequence returns RN(x / s) for binary32 operands whenever no

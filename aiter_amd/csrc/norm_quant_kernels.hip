@@ -241,7 +241,7 @@ __device__ __forceinline__ float amax16(const float (&v)[16])
 __device__ __forceinline__ void encode16_fast(const float (&v)[16], float m, u32x4& codes, float& scale)
 {
     const float s = amax_over_448(m); // = m / 448 as IEEE division gives it
-    const float r = 1.0f / s;         // IEEE division: the correctly rounded reciprocal
+    const float r = recip_in_range(s); // the correctly rounded reciprocal: s lies within 2^-89 .. 2^92 here
     uint32_t    out[4];
 #pragma unroll
     for(int j = 0; j < 4; ++j)
@@ -525,6 +525,7 @@ struct NormKernelParams
     float           eps;
     int32_t         transpose_scale;
     int32_t         gemma_norm;
+    double          inv_hidden; // RN(1 / hidden), for div_by_count
 };
 
 template <In16 DT, bool ADD, int GS /* 0 = no quant */, int U /* 16-element units per lane */>
@@ -621,8 +622,12 @@ __global__ __launch_bounds__(512) void rmsnorm_kernel(NormKernelParams p)
         pr[w] = part[w];
     const double tot = ((pr[0] + pr[1]) + (pr[2] + pr[3])) + ((pr[4] + pr[5]) + (pr[6] + pr[7]));
 
-    const float mean = (float)(tot / (double)p.hidden);
-    const float rstd = 1.0f / sqrtf(mean + p.eps); // correctly rounded sqrt and division
+    // every wave of the block repeats this: the quotient and the reciprocal take the short forms that
+    // give the IEEE results (tot / hidden as correctly rounded; 1 / root inside recip_in_range's range)
+    const float    mean = (float)div_by_count(tot, (double)p.hidden, p.inv_hidden);
+    const float    root = sqrtf(mean + p.eps); // correctly rounded
+    const uint32_t rb   = __float_as_uint(root);
+    const float    rstd = rb >= kRecipMinBits && rb <= kRecipMaxBits ? recip_in_range(root) : 1.0f / root;
 
 #pragma unroll
     for(int j = 0; j < U; ++j)
@@ -736,6 +741,7 @@ hipError_t launch_rmsnorm(const NormArgs& a, hipStream_t stream)
     p.eps             = a.eps;
     p.transpose_scale = a.transpose_scale ? 1 : 0;
     p.gemma_norm      = a.gemma_norm ? 1 : 0;
+    p.inv_hidden      = 1.0 / (double)a.hidden;
     const int  group  = a.out8 ? a.group : 0;
     const bool add    = a.residual_in != nullptr;
     if(a.dtype == In16::bf16)

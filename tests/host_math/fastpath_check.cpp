@@ -8,6 +8,7 @@
 //           128 significands of amax at each of a set of exponents, all x codes)
 //     fp16  every fp16 amax x every fp16 |x| <= amax
 //     scale amax / 448 by multiplication and correction vs the IEEE division, every bf16 and fp16 amax
+//     mean  sum / row length by multiplication and correction vs the fp64 division, row lengths 1 .. 16384
 //     cvt   software conversion vs oracle on structured fp32 inputs
 // Prints "OK <count>" or the first mismatches and exits non-zero.
 #include "../../aiter_amd/csrc/fp8bs_math.h"
@@ -105,6 +106,34 @@ int main(int argc, char** argv)
                     ++bad;
                 }
             }
+    }
+    else if(strcmp(mode, "mean") == 0)
+    {
+        // sum of squares / row length: significands from a hash over the exponents such sums span, plus 0,
+        // inf and the exact quotient 1
+        for(uint32_t len = 1; len <= 16384; ++len)
+        {
+            const double dn = (double)len, inv = 1.0 / dn;
+            for(uint32_t i = 0; i < 256; ++i)
+            {
+                uint64_t h = ((uint64_t)len << 32) | i;
+                h ^= h >> 33; h *= 0xff51afd7ed558ccdull; h ^= h >> 33; h *= 0xc4ceb9fe1a85ec53ull; h ^= h >> 33;
+                const uint64_t bits = (h & 0x000fffffffffffffull) | ((uint64_t)(1023 - 280 + (h >> 52) % 560) << 52);
+                double a;
+                memcpy(&a, &bits, 8);
+                if(i == 0) a = 0.0;
+                if(i == 1) a = __builtin_inf();
+                if(i == 2) a = dn;
+                const double want = a / dn, got = fp8bs::div_by_count(a, dn, inv);
+                ++n;
+                if(memcmp(&want, &got, 8) != 0)
+                {
+                    if(bad < 10)
+                        fprintf(stderr, "a=%a len=%u want=%a got=%a\n", a, len, want, got);
+                    ++bad;
+                }
+            }
+        }
     }
     else if(strcmp(mode, "cvt") == 0)
     {

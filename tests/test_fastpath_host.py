@@ -21,7 +21,7 @@ def checker(tmp_path_factory):
     return exe
 
 
-@pytest.mark.parametrize("mode", ["bf16", "fp16", "scale", "cvt"])
+@pytest.mark.parametrize("mode", ["bf16", "fp16", "scale", "mean", "cvt"])
 def test_fast_division_is_ieee_exact(checker, mode):
     out = subprocess.run([checker, mode], capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stdout + out.stderr
