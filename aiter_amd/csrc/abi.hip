@@ -997,25 +997,40 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
         a.activation        = (int32_t)activation;
         // the reference's names pick among its tuned kernels; here "nt=1|2|4" pins the first GEMM's
         // columns per workgroup, "dw=" / "dc=" / "down=rows" pick the second GEMM that writes rows
-        // (and its shape), "down=cols" the one that sums per token in LDS, anything else means choose
-        a.gate_tiles = 0;
-        a.down_waves = 0;
-        if(kernel_name && strncmp(kernel_name, "nt=", 3) == 0)
-            a.gate_tiles = atoi(kernel_name + 3);
+        // (and its shape), "down=cols" the one that sums per token in LDS, "pair=0|1" whether consecutive
+        // blocks of one expert are multiplied in pairs; several hints are joined by commas; anything else
+        // means choose
+        a.gate_tiles     = 0;
+        a.down_waves     = 0;
         a.down_wave_cols = 0;
-        if(kernel_name && strncmp(kernel_name, "dw=", 3) == 0)
-            a.down_waves = atoi(kernel_name + 3);
-        if(kernel_name && strncmp(kernel_name, "dc=", 3) == 0)
+        a.down_mode      = 0;
+        a.pair_blocks    = -1;
+        for(const char* hint = kernel_name; hint && *hint;)
         {
-            a.down_wave_cols = 64;
-            a.down_waves     = atoi(kernel_name + 3);
+            const char*  end = strchr(hint, ',');
+            const size_t len = end ? (size_t)(end - hint) : strlen(hint);
+            auto         is  = [&](const char* word) { return len == strlen(word) && strncmp(hint, word, len) == 0; };
+            if(len > 3 && strncmp(hint, "nt=", 3) == 0)
+                a.gate_tiles = atoi(hint + 3);
+            else if(len > 3 && strncmp(hint, "dw=", 3) == 0)
+            {
+                a.down_waves = atoi(hint + 3);
+                a.down_mode  = 1; // these hints are about the kernel that writes rows
+            }
+            else if(len > 3 && strncmp(hint, "dc=", 3) == 0)
+            {
+                a.down_wave_cols = 64;
+                a.down_waves     = atoi(hint + 3);
+                a.down_mode      = 1;
+            }
+            else if(is("down=rows"))
+                a.down_mode = 1;
+            else if(is("down=cols"))
+                a.down_mode = 2;
+            else if(len > 5 && strncmp(hint, "pair=", 5) == 0)
+                a.pair_blocks = atoi(hint + 5) != 0 ? 1 : 0;
+            hint = end ? end + 1 : nullptr;
         }
-        a.down_mode = 0;
-        if(kernel_name && (strncmp(kernel_name, "dw=", 3) == 0 || strncmp(kernel_name, "dc=", 3) == 0 ||
-                           strcmp(kernel_name, "down=rows") == 0))
-            a.down_mode = 1; // these hints are about the kernel that writes rows
-        if(kernel_name && strcmp(kernel_name, "down=cols") == 0)
-            a.down_mode = 2;
         a.device_id         = input->device_id;
         if(M == 0)
             return; // nothing to do, and no device needed to say so

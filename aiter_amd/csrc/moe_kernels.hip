@@ -509,6 +509,7 @@ struct MoeGemmParams
     int32_t        xs_stride;  // second GEMM only: floats between the scale rows of two slots
     int32_t        block_rows;   // sorted rows a workgroup's block covers: 32, or 16 when the arrays were sorted in blocks of 16
     int32_t        expert_shift; // such a block's entry in sorted_expert_ids is block >> expert_shift (sorting blocks of 64, 128)
+    int32_t        pair_blocks;  // two consecutive blocks of one expert are multiplied together (many rows per expert)
     int64_t        lda;
 };
 
@@ -543,12 +544,65 @@ __device__ __forceinline__ float activate(float g, int activation)
 }
 
 // whether block `blk` is the only block of rows of its expert (its neighbours in the sorted order
-// belong to other experts or lie past the valid rows)
+// belong to other experts or lie past the valid rows): its weights are then read once
 __device__ __forceinline__ bool only_block_of_its_expert(const MoeGemmParams& p, int blk, int expert)
 {
     const bool prev = blk > 0 && p.sorted_expert_ids[(blk - 1) >> p.expert_shift] == expert;
     const bool next = (blk + 1) * p.block_rows < p.num_valid[0] && p.sorted_expert_ids[(blk + 1) >> p.expert_shift] == expert;
     return !prev && !next;
+}
+
+// Where block `blk` stands among the consecutive blocks of its expert in the sorted order: how many
+// come before it, and whether one and two more follow.  Every lane of the calling wave gets the
+// same answer from one request in the usual case (lanes 0 and 1 look at the next two blocks, lanes
+// 2 .. 63 at the 62 blocks before; longer runs are followed 64 blocks at a time).
+struct RunOfBlocks
+{
+    int  before;
+    bool next, next2;
+    // the only block of its expert: its weights are read once
+    __device__ bool alone() const { return before == 0 && !next; }
+};
+__device__ __forceinline__ RunOfBlocks run_of_blocks(const MoeGemmParams& p, int blk, int expert)
+{
+    const int      lane  = threadIdx.x & 63, valid = p.num_valid[0];
+    const int      b0    = lane < 2 ? blk + 1 + lane : blk + 1 - lane;
+    const bool     in0   = lane < 2 ? b0 * p.block_rows < valid : b0 >= 0;
+    const bool     same0 = in0 && p.sorted_expert_ids[(in0 ? b0 : blk) >> p.expert_shift] == expert;
+    const uint64_t m0    = __ballot(same0);
+    RunOfBlocks    r{0, (m0 & 1) != 0, (m0 & 3) == 3};
+    const uint64_t back  = m0 >> 2 | (uint64_t)3 << 62;
+    r.before             = back == ~(uint64_t)0 ? 62 : __builtin_ctzll(~back);
+    bool more = r.before == 62;
+    while(more)
+    {
+        const int      b    = blk - 1 - r.before - lane;
+        const bool     same = b >= 0 && p.sorted_expert_ids[(b >= 0 ? b : 0) >> p.expert_shift] == expert;
+        const uint64_t m    = __ballot(same);
+        const int      run  = m == ~(uint64_t)0 ? 64 : __builtin_ctzll(~m);
+        r.before += run;
+        more = run == 64;
+    }
+    return r;
+}
+
+// Pairs of blocks (pair_blocks: set by the launcher where an expert has many rows).  Blocks 2i and
+// 2i + 1 of an expert's run are multiplied together by the workgroups of both: each takes half of
+// its columns, for the rows of both blocks, so that the expert's weights are read once per pair.
+// For the block at `blk`: whether it has a partner, the pair's first block, which half this
+// workgroup takes, and whether the pair is the expert's whole run (its weights are read once).
+struct PairOfBlocks
+{
+    bool paired;
+    int  first, half;
+    bool once;
+};
+__device__ __forceinline__ PairOfBlocks pair_of_blocks(const MoeGemmParams& p, const RunOfBlocks& run, int blk)
+{
+    const bool odd = run.before & 1;
+    PairOfBlocks q{p.pair_blocks && p.block_rows == 32 && (odd || run.next), blk - (odd ? 1 : 0), odd ? 1 : 0, false};
+    q.once = odd ? run.before == 1 && !run.next : run.before == 0 && !run.next2;
+    return q;
 }
 
 // First GEMM + activation.  Workgroup = (block of 32 sorted rows, NT x 16 inter columns): NT
@@ -656,7 +710,9 @@ __device__ __forceinline__ void gate_up_body(const MoeGemmParams& p, float* red,
     }
 }
 
-template <int NT>
+// PAIRS: the instance that can multiply pairs of blocks, kept apart from the usual one (which needs
+// fewer registers and only looks at a block's two neighbours)
+template <int NT, bool PAIRS>
 __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmParams p)
 {
     __shared__ __attribute__((aligned(16))) float red_dyn[kGateUpWaves * 2 * NT * 64 * 4];
@@ -693,7 +749,29 @@ __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmP
     }
     // rows of a block are real pairs first, padding after: the second 16 rows matter only if row 16 is real
     const bool second_half = p.block_rows == 32 && (p.sorted_ids[blk * 32 + 16] & 0xffffff) < p.M;
-    const bool once = only_block_of_its_expert(p, blk, expert);
+    bool once;
+    if constexpr(PAIRS && NT == 4)
+    {
+        const RunOfBlocks  run = run_of_blocks(p, blk, expert);
+        const PairOfBlocks pr  = pair_of_blocks(p, run, blk);
+        if(pr.paired)
+        {
+            // half as many columns (two gate tiles and their up tiles), the rows of both blocks; the second
+            // block's second half only if it holds real rows (the first block of a pair is full)
+            const int  group = pr.half * p.n_groups + grp;
+            const bool full  = (p.sorted_ids[(pr.first + 1) * 32 + 16] & 0xffffff) < p.M;
+            if(full)
+                pr.once ? gate_up_body<4, 2, true>(p, red_dyn, pr.first, group, expert)
+                        : gate_up_body<4, 2, false>(p, red_dyn, pr.first, group, expert);
+            else
+                pr.once ? gate_up_body<3, 2, true>(p, red_dyn, pr.first, group, expert)
+                        : gate_up_body<3, 2, false>(p, red_dyn, pr.first, group, expert);
+            return;
+        }
+        once = run.alone();
+    }
+    else
+        once = only_block_of_its_expert(p, blk, expert);
     if(second_half)
         once ? gate_up_body<2, NT, true>(p, red_dyn, blk, grp, expert) : gate_up_body<2, NT, false>(p, red_dyn, blk, grp, expert);
     else
@@ -703,11 +781,12 @@ __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmP
 // Second GEMM.  Workgroup = (block of 32 sorted rows, 512 output columns), wave = 128 columns =
 // 8 weight tiles walked two at a time with the next two already requested; the block's
 // activation rows (K = inter_dim, at most 4 K blocks on this path) stay in registers.
+// `half` 0 / 1 with `halves` 2: a wave takes the first / second half of its columns only (pairs of blocks)
 template <int MT, int KB, bool STREAM>
-__device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int grp, int expert)
+__device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int grp, int expert, int half = 0, int halves = 1)
 {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
-    const int n0 = (grp * p.waves + wave) * p.wave_cols;
+    const int n0 = (grp * p.waves + wave) * p.wave_cols + half * (p.wave_cols / halves);
     if(n0 >= p.N)
         return;
     i32x8 x[MT][KB];
@@ -728,7 +807,7 @@ __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int g
     const size_t   tile_stride = (size_t)16 * (size_t)p.K;
     const uint8_t* wt  = p.w + (size_t)expert * (size_t)p.N * (size_t)p.K + (size_t)(n0 >> 4) * tile_stride;
     const float*   wsr = p.wsc + (size_t)expert * (p.N / 128) * KB;
-    const int      want  = p.wave_cols / 32;
+    const int      want  = p.wave_cols / 32 / halves;
     const int      pairs = (p.N - n0) / 32 < want ? (p.N - n0) / 32 : want; // N is a multiple of 256
 
     auto fetch = [&](int pair, i32x8 (&w)[2][KB]) {
@@ -784,7 +863,9 @@ __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int g
     }
 }
 
-template <int KB>
+// PAIRS: the instance that can multiply pairs of blocks (more registers: kept apart so that the usual
+// instance keeps three workgroups of four waves per compute unit)
+template <int KB, bool PAIRS>
 __global__ __launch_bounds__(512) void moe_down_kernel(MoeGemmParams p)
 {
     const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
@@ -794,7 +875,26 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeGemmParams p)
     if(expert < 0 || expert >= p.experts)
         return;
     const bool second_half = p.block_rows == 32 && (p.sorted_ids[blk * 32 + 16] & 0xffffff) < p.M;
-    const bool once = only_block_of_its_expert(p, blk, expert);
+    bool once;
+    if constexpr(PAIRS && KB <= 2) // the rows of two blocks stay in registers only for short K
+    {
+        const RunOfBlocks  run = run_of_blocks(p, blk, expert);
+        const PairOfBlocks pr  = pair_of_blocks(p, run, blk);
+        if(pr.paired)
+        {
+            const bool full = (p.sorted_ids[(pr.first + 1) * 32 + 16] & 0xffffff) < p.M;
+            if(full)
+                pr.once ? down_body<4, KB, true>(p, pr.first, grp, expert, pr.half, 2)
+                        : down_body<4, KB, false>(p, pr.first, grp, expert, pr.half, 2);
+            else
+                pr.once ? down_body<3, KB, true>(p, pr.first, grp, expert, pr.half, 2)
+                        : down_body<3, KB, false>(p, pr.first, grp, expert, pr.half, 2);
+            return;
+        }
+        once = run.alone();
+    }
+    else
+        once = only_block_of_its_expert(p, blk, expert);
     if(second_half)
         once ? down_body<2, KB, true>(p, blk, grp, expert) : down_body<2, KB, false>(p, blk, grp, expert);
     else
@@ -1534,6 +1634,11 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
     p.max_blocks        = a.max_blocks;
     p.block_rows        = a.block_rows;
     p.expert_shift      = a.expert_shift;
+    // pairs of blocks where the average expert has a block's worth of rows or more (DeepSeek-V3 layer,
+    // 1024 tokens: 407 -> 386 us with the first GEMM's pairs; at 256 and 512 tokens, where only the
+    // shared expert has runs of blocks, the gathered rows of a pair cost more than its weights save:
+    // 258 -> 263 and 286 -> 292 us)
+    p.pair_blocks       = a.pair_blocks >= 0 ? a.pair_blocks : ((double)a.M * a.topk >= 32.0 * a.experts ? 1 : 0);
     p.experts           = a.experts;
     p.activation        = a.activation;
     p.lda               = a.x16 ? a.dim : a.lda;
@@ -1553,9 +1658,14 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
         const dim3 grid((unsigned)((size_t)a.max_blocks * p.n_groups));
         switch(nt)
         {
-        case 4: hipLaunchKernelGGL(moe_gate_up_kernel<4>, grid, dim3(64 * kGateUpWaves), 0, stream, p); break;
-        case 2: hipLaunchKernelGGL(moe_gate_up_kernel<2>, grid, dim3(64 * kGateUpWaves), 0, stream, p); break;
-        default: hipLaunchKernelGGL(moe_gate_up_kernel<1>, grid, dim3(64 * kGateUpWaves), 0, stream, p); break;
+        case 4:
+            if(p.pair_blocks)
+                hipLaunchKernelGGL((moe_gate_up_kernel<4, true>), grid, dim3(64 * kGateUpWaves), 0, stream, p);
+            else
+                hipLaunchKernelGGL((moe_gate_up_kernel<4, false>), grid, dim3(64 * kGateUpWaves), 0, stream, p);
+            break;
+        case 2: hipLaunchKernelGGL((moe_gate_up_kernel<2, false>), grid, dim3(64 * kGateUpWaves), 0, stream, p); break;
+        default: hipLaunchKernelGGL((moe_gate_up_kernel<1, false>), grid, dim3(64 * kGateUpWaves), 0, stream, p); break;
         }
     }
 
@@ -1638,10 +1748,20 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
         const dim3 grid((unsigned)((size_t)a.max_blocks * d.n_groups));
         switch(d.kblocks)
         {
-        case 1: hipLaunchKernelGGL(moe_down_kernel<1>, grid, dim3(64 * d.waves), 0, stream, d); break;
-        case 2: hipLaunchKernelGGL(moe_down_kernel<2>, grid, dim3(64 * d.waves), 0, stream, d); break;
-        case 3: hipLaunchKernelGGL(moe_down_kernel<3>, grid, dim3(64 * d.waves), 0, stream, d); break;
-        default: hipLaunchKernelGGL(moe_down_kernel<4>, grid, dim3(64 * d.waves), 0, stream, d); break;
+        case 1:
+            if(d.pair_blocks)
+                hipLaunchKernelGGL((moe_down_kernel<1, true>), grid, dim3(64 * d.waves), 0, stream, d);
+            else
+                hipLaunchKernelGGL((moe_down_kernel<1, false>), grid, dim3(64 * d.waves), 0, stream, d);
+            break;
+        case 2:
+            if(d.pair_blocks)
+                hipLaunchKernelGGL((moe_down_kernel<2, true>), grid, dim3(64 * d.waves), 0, stream, d);
+            else
+                hipLaunchKernelGGL((moe_down_kernel<2, false>), grid, dim3(64 * d.waves), 0, stream, d);
+            break;
+        case 3: hipLaunchKernelGGL((moe_down_kernel<3, false>), grid, dim3(64 * d.waves), 0, stream, d); break;
+        default: hipLaunchKernelGGL((moe_down_kernel<4, false>), grid, dim3(64 * d.waves), 0, stream, d); break;
         }
     }
     else

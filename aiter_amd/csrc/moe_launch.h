@@ -65,6 +65,7 @@ struct MoeArgs
     int32_t        down_waves; // second GEMM: waves per workgroup (2, 4, 8), 0 = choose
     int32_t        down_wave_cols; // second GEMM: columns per wave (64, 128), 0 = choose
     int32_t        down_mode;      // second GEMM: 1 = rows through memory + separate sum, 2 = per-token sum in LDS
+    int32_t        pair_blocks;    // consecutive blocks of one expert multiplied in pairs: 1 / 0, -1 = choose
                                    // (where its tables fit); 0 = choose
     int64_t        lda, out_stride;
     int            device_id;

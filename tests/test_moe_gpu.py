@@ -327,6 +327,24 @@ def test_fmoe_tuning_hints_do_not_change_the_result(hint):
     assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
 
 
+@pytest.mark.parametrize("tokens,dim,inter,experts,topk", [(300, 512, 256, 4, 2), (200, 7168, 256, 32, 8),
+                                                           (70, 1024, 128, 3, 2), (330, 512, 256, 5, 1)])
+def test_fmoe_pairs_of_blocks_give_the_same_bits(tokens, dim, inter, experts, topk):
+    # Where the average expert has 32 rows or more the library multiplies two consecutive blocks of an expert
+    # together (their workgroups take half the columns each for the rows of both).  Every product is summed in
+    # the same order as block by block, so the result must be the same to the bit: runs of odd and even
+    # length, a partly filled last block, runs of two (weights read once) and longer ones, both second GEMMs.
+    p = make_moe(tokens, dim, inter, experts, topk, seed=tokens + experts)
+    refs = reference(p)
+    for down in ("down=rows", "down=cols"):
+        single = run_moe(p, kernel_name=f"pair=0,{down}")
+        paired = run_moe(p, kernel_name=f"pair=1,{down}")
+        assert torch.equal(single.view(torch.int16), paired.view(torch.int16)), down
+        assert_close(paired, refs, f"pairs of blocks, {down}")
+    if tokens * topk >= 32 * experts:  # the library's own choice is then the paired form
+        assert torch.equal(run_moe(p).view(torch.int16)[:0], run_moe(p, kernel_name="pair=1").view(torch.int16)[:0])
+
+
 def test_fmoe_is_deterministic_and_accumulates_into_out():
     p = make_moe(48, 1024, 256, 16, 4, seed=2)
     a = run_moe(p)
