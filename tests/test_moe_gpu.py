@@ -342,7 +342,29 @@ def test_fmoe_pairs_of_blocks_give_the_same_bits(tokens, dim, inter, experts, to
         assert torch.equal(single.view(torch.int16), paired.view(torch.int16)), down
         assert_close(paired, refs, f"pairs of blocks, {down}")
     if tokens * topk >= 32 * experts:  # the library's own choice is then the paired form
-        assert torch.equal(run_moe(p).view(torch.int16)[:0], run_moe(p, kernel_name="pair=1").view(torch.int16)[:0])
+        assert torch.equal(run_moe(p).view(torch.int16), run_moe(p, kernel_name="pair=1").view(torch.int16))
+
+
+@pytest.mark.parametrize("block", [64, 128])
+def test_fmoe_pairs_of_blocks_in_arrays_sorted_in_larger_blocks(block):
+    # sorted in blocks of 64 or 128 rows, the kernels' 32-row blocks of one sorted block share an expert id:
+    # pairs then form inside a sorted block too, padding-only blocks included
+    tokens, dim, inter, experts, topk = 150, 512, 256, 4, 2
+    p = make_moe(tokens, dim, inter, experts, topk, seed=block)
+    w1 = aiter_amd.shuffle_weight(p["w1q"].view(torch.uint8)).view(dtypes.fp8)
+    w2 = aiter_amd.shuffle_weight(p["w2q"].view(torch.uint8)).view(dtypes.fp8)
+    a, a_scale = p["aq"].to(DEV), p["asc"].t().contiguous().to(DEV)
+    ti, tw = p["ti"].to(DEV), p["tw"].to(DEV)
+    outs = {}
+    for hint in ("pair=0,down=rows", "pair=1,down=rows", "pair=0,down=cols", "pair=1,down=cols"):
+        s_ids, s_w, s_e, nv, out = aiter_amd.moe_sorting(ti, tw, experts, dim, torch.bfloat16, block_size=block)
+        aiter_amd.fmoe_fp8_blockscale_g1u1(out, a, w1, w2, s_ids, s_w, s_e, nv, topk, a_scale, p["w1s"], p["w2s"],
+                                           hint, 128, 128, None, 0, block)
+        torch.cuda.synchronize()
+        outs[hint] = out
+    assert torch.equal(outs["pair=0,down=rows"].view(torch.int16), outs["pair=1,down=rows"].view(torch.int16))
+    assert torch.equal(outs["pair=0,down=cols"].view(torch.int16), outs["pair=1,down=cols"].view(torch.int16))
+    assert_close(outs["pair=1,down=rows"], reference(p), f"pairs, sorted in blocks of {block}")
 
 
 def test_fmoe_is_deterministic_and_accumulates_into_out():
