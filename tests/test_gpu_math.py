@@ -10,8 +10,13 @@ LIB = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gpu_math", "libg
 
 
 def load():
-    if not os.path.exists(LIB):
-        raise RuntimeError(f"{LIB} is not built: run python -c 'import __graft_entry__ as g; g.build()'")
+    if not os.path.exists(LIB):  # a fresh checkout: build it as __graft_entry__.build() does (hipcc cross-compiles)
+        import sys
+
+        sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+        import __graft_entry__
+
+        __graft_entry__.build_gpu_math_check()
     lib = ctypes.CDLL(LIB)
     for name in ("gpu_math_recip_sweep", "gpu_math_mean_sweep"):
         fn = getattr(lib, name)
