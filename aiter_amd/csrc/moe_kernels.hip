@@ -1644,16 +1644,28 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
     p.lda               = a.x16 ? a.dim : a.lda;
     {
         // (expert, block) pairs to expect under a routing that spreads evenly: the experts hit at least once,
-        // plus the full blocks.  Wide units (64 columns; one workgroup per compute unit at a time) where
-        // they cover the chip and their last round is not a nearly empty one; the narrowest otherwise
-        // (DeepSeek-V3 layer, us at 8 / 16 / 24 / 32 tokens: wide 69 / 117 / 161 / 177, narrow 72 / 119 /
-        // 151 / 179, the 32-column units in between or behind both).
+        // plus the full blocks.  A workgroup takes 64, 32 or 16 columns (one workgroup per compute unit at a
+        // time).  The widest units that fill a single round of workgroups reasonably (at least two thirds of the
+        // compute units, at most a tenth over); beyond a round, the wide units where their last round is three
+        // quarters full or there are four rounds and more, else the narrowest, whose last round costs least.
+        // DeepSeek-V3 layer, same routing, us with 16 / 32 / 64 columns: 2 tokens 35.3 / 33.5 / 41.2, 3 tokens
+        // 38.6 / 36.2 / 42.8, 7 tokens 61.7 / 60.7 / 58.2, 12 tokens 83.9 / 85.1 / 92.1, 16 tokens 101.2 / 105.3 /
+        // 100.9, 28 tokens 142.6 / 141.7 / 147.5, 48 tokens 184.7 / 187.2 / 191.8, 80 tokens 219.7 / 219.7 / 215.4.
         const double pairs  = (double)a.M * a.topk;
         const double blocks = (double)a.experts * (1.0 - exp(-pairs / (double)a.experts)) + pairs / 32.0;
-        const double wide   = blocks * (a.inter / 64), rounds = wide / 256.0;
-        int          nt     = a.gate_tiles;
+        const double wide = blocks * (a.inter / 64), mid = blocks * (a.inter / 32), rounds = wide / 256.0;
+        int          nt   = a.gate_tiles;
         if(nt != 1 && nt != 2 && nt != 4)
-            nt = (wide >= 230.0 && (rounds <= 1.05 || rounds - floor(rounds) >= 0.4 || rounds >= 4.0)) ? 4 : 1;
+        {
+            if(wide >= 170.0 && rounds <= 1.1)
+                nt = 4;
+            else if(mid >= 130.0 && mid <= 260.0)
+                nt = 2;
+            else if(wide >= 230.0 && (rounds - floor(rounds) >= 0.75 || rounds >= 4.0))
+                nt = 4;
+            else
+                nt = 1;
+        }
         p.n_groups = a.inter / (16 * nt);
         const dim3 grid((unsigned)((size_t)a.max_blocks * p.n_groups));
         switch(nt)
