@@ -1016,7 +1016,11 @@ struct DownColsParams
     int32_t         walkers; // waves per K block: each walks every walkers-th unit into tables of its own
 };
 
-constexpr int kColsDepth     = 7;
+// units a wave has requested ahead of the one it multiplies.  With the weights read non-temporally three is the
+// measured optimum (DeepSeek-V3 layer, us at 1 / 32 / 128 / 256 tokens: depth 2 24.3 / 155.1 / 236.9 / 255.6, 3 24.3 /
+// 151.9 / 233.0 / 255.9, 4 25.1 / 152.2 / 234.0 / 256.2, 7 25.9 / 154.1 / 236.4 / 258.9, 8 26.4 / 155.8 / 237.5 / 258.3):
+// more requests in flight per compute unit only queue up
+constexpr int kColsDepth     = 3;
 constexpr int kColsTiles     = 2;    // 16-column tiles per workgroup, both multiplied by every wave
 constexpr int kColsMaxBlocks = 1024; // blocks the unit scan takes (16 per lane)
 constexpr size_t kColsTableBytes = (size_t)140 << 10; // LDS for the per-token tables; the unit list (16 KiB at most) comes on top
@@ -1060,11 +1064,11 @@ __device__ __forceinline__ void cols_load8_at16(u32x2& d, const void* p)
 }
 constexpr int kColsLoadsPerStage = 9; // loads the walk requests per unit, counted by cols_wait_oldest
 // the stage requested kColsDepth - 1 stages ago has arrived once at most (kColsDepth - 1) *
-// kColsLoadsPerStage = 54 younger loads are outstanding (loads return in order); the stage's
+// kColsLoadsPerStage = 18 younger loads are outstanding (loads return in order); the stage's
 // registers are operands so that nothing that reads them is moved above the wait
 __device__ __forceinline__ void cols_wait_oldest(ColsStage& s)
 {
-    asm volatile("s_waitcnt vmcnt(54)"
+    asm volatile("s_waitcnt vmcnt(18)"
                  : "+v"(s.wlo[0]), "+v"(s.whi[0]), "+v"(s.wlo[1]), "+v"(s.whi[1]), "+v"(s.xlo), "+v"(s.xhi), "+v"(s.xs),
                    "+v"(s.ws), "+v"(s.sw_tok)
                  :
@@ -1080,7 +1084,7 @@ __device__ __forceinline__ void cols_drain(ColsStage& s)
                  :
                  : "memory");
 }
-static_assert((kColsDepth - 1) * kColsLoadsPerStage == 54 && kColsTiles == 2, "cols_wait_oldest counts 54 younger loads");
+static_assert((kColsDepth - 1) * kColsLoadsPerStage == 18 && kColsTiles == 2, "cols_wait_oldest counts 18 younger loads");
 
 template <In16 DT>
 __global__ __launch_bounds__(256) void moe_down_cols_kernel(DownColsParams p)
