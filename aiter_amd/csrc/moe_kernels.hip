@@ -848,6 +848,18 @@ __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int g
             }
         }
     };
+    if constexpr(MT > 2)
+    {
+        // pairs of blocks: one pair of tiles at a time, nothing requested ahead (measured: 385 -> 380 us at
+        // 1024 tokens; with one block per pass the requests ahead are worth 1.5 us at 512 tokens)
+        i32x8 wa[2][KB];
+        for(int pair = 0; pair < pairs; ++pair)
+        {
+            fetch(pair, wa);
+            finish(pair, wa);
+        }
+        return;
+    }
     i32x8 wa[2][KB], wb[2][KB];
     fetch(0, wa);
     for(int pair = 0; pair < pairs; pair += 2)
