@@ -998,13 +998,14 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
         // the reference's names pick among its tuned kernels; here "nt=1|2|4" pins the first GEMM's
         // columns per workgroup, "dw=" / "dc=" / "down=rows" pick the second GEMM that writes rows
         // (and its shape), "down=cols" the one that sums per token in LDS, "pair=0|1" whether consecutive
-        // blocks of one expert are multiplied in pairs; several hints are joined by commas; anything else
+        // blocks of one expert are multiplied in pairs, "tail=0" keeps the first GEMM's last blocks as wide as the rest; several hints are joined by commas; anything else
         // means choose
         a.gate_tiles     = 0;
         a.down_waves     = 0;
         a.down_wave_cols = 0;
         a.down_mode      = 0;
         a.pair_blocks    = -1;
+        a.fine_tail      = -1;
         for(const char* hint = kernel_name; hint && *hint;)
         {
             const char*  end = strchr(hint, ',');
@@ -1029,6 +1030,8 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
                 a.down_mode = 2;
             else if(len > 5 && strncmp(hint, "pair=", 5) == 0)
                 a.pair_blocks = atoi(hint + 5) != 0 ? 1 : 0;
+            else if(is("tail=0"))
+                a.fine_tail = 0;
             hint = end ? end + 1 : nullptr;
         }
         a.device_id         = input->device_id;

@@ -24,6 +24,7 @@
 #include "gemm_common.h"
 #include "moe_launch.h"
 
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 
@@ -510,6 +511,7 @@ struct MoeGemmParams
     int32_t        block_rows;   // sorted rows a workgroup's block covers: 32, or 16 when the arrays were sorted in blocks of 16
     int32_t        expert_shift; // such a block's entry in sorted_expert_ids is block >> expert_shift (sorting blocks of 64, 128)
     int32_t        pair_blocks;  // two consecutive blocks of one expert are multiplied together (many rows per expert)
+    int32_t        fine_blocks;  // first GEMM, NT = 4: the blocks taken last that are cut into 16-column workgroups
     int64_t        lda;
 };
 
@@ -619,6 +621,7 @@ __device__ __forceinline__ PairOfBlocks pair_of_blocks(const MoeGemmParams& p, c
 // workgroup that has a compute unit to itself (the last units of a launch) should still stream at
 // the unit's share of HBM
 constexpr int kGateUpWaves = 8;
+constexpr int kChipCus     = 256;
 
 template <int MT, int NT, bool STREAM>
 __device__ __forceinline__ void gate_up_body(const MoeGemmParams& p, float* red, int blk, int grp, int expert)
@@ -720,8 +723,34 @@ __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmP
     // shared expert, which every token is routed to and which conventionally has the last id, has the
     // most blocks, each of two full row tiles and read with ordinary loads: started first, they are not
     // what the launch ends on.
-    const int at = blockIdx.x / p.n_groups, grp = blockIdx.x - at * p.n_groups;
-    const int blk = (p.num_valid[0] + p.block_rows - 1) / p.block_rows - 1 - at;
+    // Wide units (NT = 4) occupy a compute unit each, so they run in rounds of kChipCus, and a last round
+    // that is nearly empty still takes a unit's streaming time.  When the wide units of the valid blocks
+    // leave such a remainder -- at most fine_blocks blocks' worth, a quarter of a round -- the blocks of
+    // the remainder (the ones taken last) go out as narrow units of 16 columns instead, which the launch
+    // reserves workgroups for behind the wide ones: the launch then ends on one short round.  Decided
+    // here from the number of valid blocks, which the host does not know (DeepSeek-V3 layer, remainder
+    // of 2-16 % of a round: 5-9 us of 240-270; a remainder of 60 % and more treated the same way costs 2-5).
+    const int valid_blocks = (p.num_valid[0] + p.block_rows - 1) / p.block_rows;
+    int       at = blockIdx.x / p.n_groups, grp = blockIdx.x - at * p.n_groups;
+    bool      fine = false;
+    if constexpr(NT == 4 && !PAIRS)
+    {
+        const int left = (valid_blocks * p.n_groups) % kChipCus, left_blocks = (left + p.n_groups - 1) / p.n_groups;
+        const int tail = left_blocks <= p.fine_blocks && valid_blocks * p.n_groups > kChipCus ? left_blocks : 0;
+        const int wide = p.max_blocks * p.n_groups;
+        if((int)blockIdx.x >= wide)
+        {
+            const int j = (int)blockIdx.x - wide, narrow_groups = 4 * p.n_groups;
+            at          = valid_blocks - tail + j / narrow_groups;
+            grp         = j % narrow_groups;
+            fine        = true;
+            if(j / narrow_groups >= tail)
+                return;
+        }
+        else if(at >= valid_blocks - tail)
+            return;
+    }
+    const int blk = valid_blocks - 1 - at;
     if(blk < 0)
         return;
     const int expert = p.sorted_expert_ids[blk >> p.expert_shift];
@@ -772,6 +801,17 @@ __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmP
     }
     else
         once = only_block_of_its_expert(p, blk, expert);
+    if constexpr(NT == 4 && !PAIRS)
+    {
+        if(fine)
+        {
+            if(second_half)
+                once ? gate_up_body<2, 1, true>(p, red_dyn, blk, grp, expert) : gate_up_body<2, 1, false>(p, red_dyn, blk, grp, expert);
+            else
+                once ? gate_up_body<1, 1, true>(p, red_dyn, blk, grp, expert) : gate_up_body<1, 1, false>(p, red_dyn, blk, grp, expert);
+            return;
+        }
+    }
     if(second_half)
         once ? gate_up_body<2, NT, true>(p, red_dyn, blk, grp, expert) : gate_up_body<2, NT, false>(p, red_dyn, blk, grp, expert);
     else
@@ -1683,7 +1723,10 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
                 nt = 1;
         }
         p.n_groups = a.inter / (16 * nt);
-        const dim3 grid((unsigned)((size_t)a.max_blocks * p.n_groups));
+        // wide units: workgroups for up to a quarter of a round of blocks cut into narrow units are launched
+        // behind them (the kernel uses them when the valid blocks leave such a remainder)
+        p.fine_blocks = (nt == 4 && !p.pair_blocks && a.fine_tail != 0) ? std::min(a.max_blocks, kChipCus / 4 / p.n_groups) : 0;
+        const dim3 grid((unsigned)((size_t)a.max_blocks * p.n_groups + (size_t)p.fine_blocks * 4 * p.n_groups));
         switch(nt)
         {
         case 4:
