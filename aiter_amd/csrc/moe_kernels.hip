@@ -565,11 +565,12 @@ struct RunOfBlocks
     // the only block of its expert: its weights are read once
     __device__ bool alone() const { return before == 0 && !next; }
 };
-__device__ __forceinline__ RunOfBlocks run_of_blocks(const MoeGemmParams& p, int blk, int expert)
+// (blocks below `lo` do not count: they are multiplied on their own)
+__device__ __forceinline__ RunOfBlocks run_of_blocks(const MoeGemmParams& p, int blk, int expert, int lo = 0)
 {
     const int      lane  = threadIdx.x & 63, valid = p.num_valid[0];
     const int      b0    = lane < 2 ? blk + 1 + lane : blk + 1 - lane;
-    const bool     in0   = lane < 2 ? b0 * p.block_rows < valid : b0 >= 0;
+    const bool     in0   = lane < 2 ? b0 * p.block_rows < valid : b0 >= lo;
     const bool     same0 = in0 && p.sorted_expert_ids[(in0 ? b0 : blk) >> p.expert_shift] == expert;
     const uint64_t m0    = __ballot(same0);
     RunOfBlocks    r{0, (m0 & 1) != 0, (m0 & 3) == 3};
@@ -579,7 +580,7 @@ __device__ __forceinline__ RunOfBlocks run_of_blocks(const MoeGemmParams& p, int
     while(more)
     {
         const int      b    = blk - 1 - r.before - lane;
-        const bool     same = b >= 0 && p.sorted_expert_ids[(b >= 0 ? b : 0) >> p.expert_shift] == expert;
+        const bool     same = b >= lo && p.sorted_expert_ids[(b >= lo ? b : lo) >> p.expert_shift] == expert;
         const uint64_t m    = __ballot(same);
         const int      run  = m == ~(uint64_t)0 ? 64 : __builtin_ctzll(~m);
         r.before += run;
@@ -733,10 +734,11 @@ __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmP
     const int valid_blocks = (p.num_valid[0] + p.block_rows - 1) / p.block_rows;
     int       at = blockIdx.x / p.n_groups, grp = blockIdx.x - at * p.n_groups;
     bool      fine = false;
-    if constexpr(NT == 4 && !PAIRS)
+    int       tail = 0; // blocks 0 .. tail - 1 are the remainder
+    if constexpr(NT == 4)
     {
         const int left = (valid_blocks * p.n_groups) % kChipCus, left_blocks = (left + p.n_groups - 1) / p.n_groups;
-        const int tail = left_blocks <= p.fine_blocks && valid_blocks * p.n_groups > kChipCus ? left_blocks : 0;
+        tail           = left_blocks <= p.fine_blocks && valid_blocks * p.n_groups > kChipCus ? left_blocks : 0;
         const int wide = p.max_blocks * p.n_groups;
         if((int)blockIdx.x >= wide)
         {
@@ -781,9 +783,10 @@ __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmP
     bool once;
     if constexpr(PAIRS && NT == 4)
     {
-        const RunOfBlocks  run = run_of_blocks(p, blk, expert);
+        // (the blocks of the remainder stay out of the pairs: they are multiplied as narrow units)
+        const RunOfBlocks  run = run_of_blocks(p, blk, expert, fine ? 0 : tail);
         const PairOfBlocks pr  = pair_of_blocks(p, run, blk);
-        if(pr.paired)
+        if(pr.paired && !fine)
         {
             // half as many columns (two gate tiles and their up tiles), the rows of both blocks; the second
             // block's second half only if it holds real rows (the first block of a pair is full)
@@ -801,7 +804,7 @@ __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmP
     }
     else
         once = only_block_of_its_expert(p, blk, expert);
-    if constexpr(NT == 4 && !PAIRS)
+    if constexpr(NT == 4)
     {
         if(fine)
         {
@@ -1725,7 +1728,7 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
         p.n_groups = a.inter / (16 * nt);
         // wide units: workgroups for up to a quarter of a round of blocks cut into narrow units are launched
         // behind them (the kernel uses them when the valid blocks leave such a remainder)
-        p.fine_blocks = (nt == 4 && !p.pair_blocks && a.fine_tail != 0) ? std::min(a.max_blocks, kChipCus / 4 / p.n_groups) : 0;
+        p.fine_blocks = (nt == 4 && a.fine_tail != 0) ? std::min(a.max_blocks, kChipCus / 4 / p.n_groups) : 0;
         const dim3 grid((unsigned)((size_t)a.max_blocks * p.n_groups + (size_t)p.fine_blocks * 4 * p.n_groups));
         switch(nt)
         {

@@ -345,6 +345,23 @@ def test_fmoe_pairs_of_blocks_give_the_same_bits(tokens, dim, inter, experts, to
         assert torch.equal(run_moe(p).view(torch.int16), run_moe(p, kernel_name="pair=1").view(torch.int16))
 
 
+@pytest.mark.parametrize("tokens", [2100, 2150, 2200, 2250, 2300])
+def test_fmoe_narrow_remainder_of_the_first_gemm_gives_the_same_bits(tokens):
+    # 66 .. 74 blocks of rows on 4 experts: their wide workgroups fill one round of 256 and leave 8 .. 40 more, a
+    # remainder that the first GEMM cuts into narrow workgroups when it is at most a quarter of a round (some of
+    # these token counts are, some are not); with and without pairs of blocks, which must leave the
+    # remainder's blocks alone.  Every product is summed in the same order either way.
+    p = make_moe(tokens, 512, 256, 4, 1, seed=tokens)
+    base = run_moe(p, kernel_name="tail=0,pair=0")
+    for hint in ("pair=0", "tail=0,pair=1", "pair=1", ""):
+        assert torch.equal(base.view(torch.int16), run_moe(p, kernel_name=hint).view(torch.int16)), hint
+    rows = torch.cat([torch.arange(0, 24), torch.arange(tokens - 24, tokens)])
+    q = dict(p, aq=p["aq"][rows], asc=p["asc"][rows], tw=p["tw"][rows], ti=p["ti"][rows])
+    quantised, _ = reference(q)
+    o = base[rows.to(DEV)].float().cpu()
+    assert ((o - quantised).norm() / quantised.norm()).item() < 8e-3
+
+
 @pytest.mark.parametrize("block", [64, 128])
 def test_fmoe_pairs_of_blocks_in_arrays_sorted_in_larger_blocks(block):
     # sorted in blocks of 64 or 128 rows, the kernels' 32-row blocks of one sorted block share an expert id:
