@@ -1693,11 +1693,11 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
     p.max_blocks        = a.max_blocks;
     p.block_rows        = a.block_rows;
     p.expert_shift      = a.expert_shift;
-    // pairs of blocks where the average expert has a block's worth of rows or more (DeepSeek-V3 layer,
-    // 1024 tokens: 407 -> 386 us with the first GEMM's pairs; at 256 and 512 tokens, where only the
-    // shared expert has runs of blocks, the gathered rows of a pair cost more than its weights save:
-    // 258 -> 263 and 286 -> 292 us)
-    p.pair_blocks       = a.pair_blocks >= 0 ? a.pair_blocks : ((double)a.M * a.topk >= 32.0 * a.experts ? 1 : 0);
+    // pairs of blocks from 28 rows per expert on average (DeepSeek-V3 layer, us block by block / in pairs:
+    // 704 tokens 304.7 / 311.1, 768: 317.8 / 319.4, 832: 330.4 / 325.4, 896: 363.7 / 345.4, 1024: 412.7 / 381.1;
+    // at 256 and 512 tokens, where only the shared expert has runs of blocks, the gathered rows of a pair
+    // cost more than its weights save)
+    p.pair_blocks       = a.pair_blocks >= 0 ? a.pair_blocks : ((double)a.M * a.topk >= 28.0 * a.experts ? 1 : 0);
     p.experts           = a.experts;
     p.activation        = a.activation;
     p.lda               = a.x16 ? a.dim : a.lda;
