@@ -302,6 +302,8 @@ __global__ __launch_bounds__(kQuantBlock) void group_quant_kernel(QuantKernelPar
     const uint32_t n_groups = rows * p.groups_per_row;
     const uint32_t lig      = threadIdx.x % LPG;
     const uint32_t g0       = blockIdx.x * (GPB * UNITS) + threadIdx.x / LPG;
+    __shared__ float block_scales[UNITS * GPB];
+    const bool     contiguous_scales = !p.transpose_scale && p.scale_row_stride == 0; // uniform
 
     u32x4 c[UNITS][2];
 #pragma unroll
@@ -328,7 +330,9 @@ __global__ __launch_bounds__(kQuantBlock) void group_quant_kernel(QuantKernelPar
             float s;
             quant16<DT, LPG>(c[u][0], c[u][1], v, codes, s);
             __builtin_nontemporal_store(codes, p.y + (size_t)g * (GS / 16) + lig);
-            if(lig == 0)
+            if(lig == 0 && contiguous_scales)
+                block_scales[u * GPB + threadIdx.x / LPG] = s;
+            else if(lig == 0)
             {
                 size_t idx = g;
                 if(p.transpose_scale)
@@ -345,6 +349,22 @@ __global__ __launch_bounds__(kQuantBlock) void group_quant_kernel(QuantKernelPar
                 }
                 p.scale[idx] = s;
             }
+        }
+    }
+    // Contiguous scales leave as whole lines: the block's GPB scales per unit go through LDS and GPB
+    // neighbouring lanes store them (4 bytes each, 128 bytes for 1x128 groups).  Stored by the lanes that
+    // computed them, every wave wrote 32 bytes of the line on its own, and those partial writes cost the
+    // memory system far more than their bytes (16384 x 7168: 58.8 us; without any scale store 56.85; whole
+    // lines 57.97, whole lines stored non-temporally 57.35).
+    if(contiguous_scales)
+    {
+        __syncthreads();
+#pragma unroll
+        for(int u = 0; u < UNITS; ++u)
+        {
+            const uint32_t g = blockIdx.x * (GPB * UNITS) + u * GPB + threadIdx.x;
+            if(threadIdx.x < GPB && g < n_groups)
+                __builtin_nontemporal_store(block_scales[u * GPB + threadIdx.x], p.scale + g);
         }
     }
 }
