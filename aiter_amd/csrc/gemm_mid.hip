@@ -55,18 +55,30 @@ struct MidShape
     // compute unit.  PAIR: six stages, filled in pairs every other iteration.
     static constexpr int kStages = PAIR ? 6 : 4;
     static constexpr int kSmem = kStages * kStageBytes;
-    static constexpr int kOccupancy = kSmem <= 72 * 1024 ? 2 : 1;
+    // Row-major x_scale in windows of four K blocks (16 bytes per row and load instead of 4: a wave's load of
+    // one scale per row touches as many lines as the rows it covers, and fetched per K block these loads are a
+    // third of the kernel's line requests).  A ring of four windows behind the stages: the stages in flight
+    // and the one being multiplied (at most seven consecutive K blocks) never span more than three.
+    static constexpr int kWindowBytes = BM * 16, kWindows = 4;
+    static constexpr int kSmemWindows = kSmem + kWindows * kWindowBytes;
+    static constexpr int kOccupancy = kSmemWindows <= 72 * 1024 ? 2 : 1;
     static_assert(NQ % 4 == 0, "the product rotation below assumes a multiple of four tiles");
 };
 
-// waits until at most `ahead` stages' worth of this wave's loads are still in flight
+// waits until at most `ahead` stages' worth of this wave's loads (and `extra` single loads: 0 or 1)
+// are still in flight
 template <int A, int LPS>
-__device__ __forceinline__ void wait_ahead(int ahead)
+__device__ __forceinline__ void wait_ahead(int ahead, int extra = 0)
 {
     if(ahead >= A)
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(A * LPS));
+    {
+        if(extra)
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(A * LPS + 1));
+        else
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(A * LPS));
+    }
     else if constexpr(A > 0)
-        wait_ahead<A - 1, LPS>(ahead);
+        wait_ahead<A - 1, LPS>(ahead, extra);
 }
 
 // The two instruction forms of the multiply stream, as non-template functions: inside the kernel
@@ -92,13 +104,17 @@ __device__ __forceinline__ void store_through(float* dst, const f32x4& v)
     asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
 }
 
-template <int BM, int BN, bool SHUF, int OCC, bool PAIR>
+// XS4: x_scale is row-major with 16-byte aligned rows and comes in windows of four K blocks.
+template <int BM, int BN, bool SHUF, int OCC, bool PAIR, bool XS4>
 __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
 {
     using S = MidShape<BM, BN, PAIR>;
     constexpr int TI = S::TI, TJ = S::TJ, NQ = S::NQ;
     constexpr int kWBytes = S::kWBytes, kXBytes = S::kXBytes, kStageBytes = S::kStageBytes;
-    constexpr int kLoadsPerStage = S::kLoadsPerStage, kStages = S::kStages;
+    // XS4: a stage's loads are its slab units, plus the window's load in front of them when the stage opens a
+    // window; the waits count the windows opened by the younger stages on top of their slab units.
+    constexpr int kLoadsPerStage = XS4 ? S::kLoadsPerStage - 1 : S::kLoadsPerStage, kStages = S::kStages;
+    constexpr uint32_t kWindowsAt = (uint32_t)S::kSmem;
 
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     const GemmKernelParams& g = p.g;
@@ -189,6 +205,14 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
     auto fill_stage = [&](int stage, int kb) {
         const uint32_t base = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)stage * kStageBytes);
         const size_t   koff = (size_t)kb * 128, koff_w = SHUF ? (size_t)kb * 2048 : koff;
+        if constexpr(XS4)
+        {
+            // the first stage of a window (or of the K range) brings the window, ahead of its own slabs
+            if(((kb & 3) == 0 || kb == kb_lo) && lane < kXsLanes)
+                dma16(__builtin_amdgcn_readfirstlane(lds0 + kWindowsAt + (uint32_t)((kb >> 2) & 3) * S::kWindowBytes +
+                                                     (uint32_t)wave * (uint32_t)kXsLanes * 16u),
+                      xs_goff + (uint32_t)(kb & ~3) * 4u, (const uint8_t*)g.xs);
+        }
 #pragma unroll
         for(int i = 0; i < S::kWUnits; ++i)
             dma16(__builtin_amdgcn_readfirstlane(base + (4u * i + wave) * 1024u), goff_w[i], g.wq + koff_w);
@@ -196,7 +220,7 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
         for(int i = 0; i < S::kXUnits; ++i)
             dma16(__builtin_amdgcn_readfirstlane(base + (uint32_t)kWBytes + (4u * i + wave) * 1024u), goff_x[i],
                   g.xq + koff);
-        if(lane < kXsLanes) // every wave issues the same number of loads per stage: the waits count them
+        if(!XS4 && lane < kXsLanes) // every wave issues the same number of loads per stage: the waits count them
             dma4(__builtin_amdgcn_readfirstlane(base + (uint32_t)(kWBytes + kXBytes) +
                                                 (uint32_t)wave * (uint32_t)kXsLanes * 4u),
                  xs_goff + (uint32_t)kb * (uint32_t)g.xs_k * 4u, g.xs);
@@ -227,7 +251,9 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
     const uint32_t whi_off = SHUF ? wlo_off + 256u : hi_off;
     const uint32_t w_base  = (uint32_t)wn * (uint32_t)(BN / 2) * 128u;
     const uint32_t x_base  = (uint32_t)kWBytes + (uint32_t)wm * (uint32_t)(BM / 2) * 128u;
-    const uint32_t xs_lds  = (uint32_t)(kWBytes + kXBytes) + ((uint32_t)wm * (uint32_t)(BM / 2) + (uint32_t)l16) * 4u;
+    // (XS4: this lane's row in window 0, first K block of the window)
+    const uint32_t xs_lds  = XS4 ? kWindowsAt + ((uint32_t)wm * (uint32_t)(BM / 2) + (uint32_t)l16) * 16u
+                                 : (uint32_t)(kWBytes + kXBytes) + ((uint32_t)wm * (uint32_t)(BM / 2) + (uint32_t)l16) * 4u;
 
     float acc[TI][TJ][4]; // plain floats: the FMAs below name single elements as asm operands
 #pragma unroll
@@ -252,6 +278,14 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
     // landed (loads return in order, so that is a count of the younger ones still allowed in
     // flight), barrier (every wave's share has landed, and every wave is done with the stage read
     // in the previous iteration), refill that previous stage, multiply.
+    // XS4: where this lane's x_scale of K block kb lies (window (kb / 4) & 3, block kb & 3 of its row).  The
+    // address of the next K block is worked out behind the multiply stream, not between the barrier and the
+    // first reads of the next iteration.
+    auto xs_window_addr = [&](int kb) -> uint32_t {
+        return (uint32_t)(((kb >> 2) & 3) * S::kWindowBytes + (kb & 3) * 4) + xs_lds;
+    };
+    uint32_t xs_addr = XS4 ? xs_window_addr(kb_lo) : 0u;
+
     const int nkb = kb_hi - kb_lo;
     constexpr int kAhead = PAIR ? 4 : kStages - 2; // most stages in flight behind the one waited for
     if(fetches)
@@ -267,8 +301,10 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
         const int kb    = kb_lo + it;
         // younger stages already requested
         const int ahead = min(nkb - 1 - it, PAIR ? ((it & 1) ? 4 : 3) : kStages - 2);
+        // (XS4: a K block among the `ahead` younger ones that is a multiple of four came with a window's load;
+        // there is at most one, as ahead <= 4)
         if(fetches)
-            wait_ahead<kAhead, kLoadsPerStage>(ahead);
+            wait_ahead<kAhead, kLoadsPerStage>(ahead, XS4 ? ((kb & 3) + ahead) >> 2 : 0);
         __syncthreads();
         if(fetches)
         {
@@ -312,7 +348,9 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
             const i32x4 lo = *(lds_vvec_ptr)(smem3 + stage + x_base + j * 2048 + lo_off);
             const i32x4 hi = *(lds_vvec_ptr)(smem3 + stage + x_base + j * 2048 + hi_off);
             bx[j]          = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            sc[j]          = *(lds_f32_ptr)(smem3 + stage + xs_lds + j * 64) * wsc;
+            sc[j]          = (XS4 ? *(lds_f32_ptr)(smem3 + xs_addr + j * 256)
+                                  : *(lds_f32_ptr)(smem3 + stage + xs_lds + j * 64)) *
+                             wsc;
         }
         // Tile q = (i, j) = (q / TJ, q % TJ).  The product of tile q is folded in behind the MFMA
         // of tile q + 2: it has been written back by then (two MFMAs of 8 passes each), so no
@@ -332,6 +370,11 @@ __global__ __launch_bounds__(kThreads, OCC) void gemm_mid_kernel(MidParams p)
 #pragma unroll
         for(int j = 0; j < TJ; ++j)
             scp[j] = sc[j];
+        if constexpr(XS4)
+        {
+            xs_addr = xs_window_addr(kb + 1);
+            asm volatile("" : "+v"(xs_addr)); // here, behind the last MFMA
+        }
     }
     // One K range, 16-byte aligned output rows: the tile goes through LDS so that all eight waves
     // store whole 128-byte (or longer) row segments, 16 bytes per lane; otherwise the waves that
@@ -491,19 +534,28 @@ hipError_t launch_shape(MidParams& p, int split_k_log2, int want_splits, const L
         p.partial = (float*)partial;
     }
 
-    auto        kernel = g.w_shuffled ? gemm_mid_kernel<BM, BN, true, S::kOccupancy, PAIR>
-                                      : gemm_mid_kernel<BM, BN, false, S::kOccupancy, PAIR>;
-    static std::atomic<bool> raised[2][64]; // dynamic LDS above the default limit needs opting in, once
-    const int   which = g.w_shuffled ? 1 : 0;
+    // x_scale in windows of four K blocks: row-major, whole windows, 16-byte aligned rows.  With the weights
+    // coming from HBM: 1024 x 2112 x 7168 44.8 -> 39.2 us, 512 x 4608 x 7168 44.9 -> 39.5, 128 x 16384 x 4096
+    // 25.9 -> 22.9, 96 x 36864 x 7168 86.6 -> 79.3; loops of 8 to 16 K blocks gain 0 to 5 %.  (With weights
+    // that a benchmark loop leaves in the last-level cache a single round of workgroups measures 0 to 7 %
+    // slower with windows; that is not the case the kernel is built for.)
+    const bool  xs4    = !g.w_shuffled && g.xs_k == 1 && g.xs_m == g.kblocks && (g.kblocks & 3) == 0 &&
+                         ((uintptr_t)g.xs & 15) == 0;
+    auto        kernel = g.w_shuffled ? gemm_mid_kernel<BM, BN, true, S::kOccupancy, PAIR, false>
+                         : xs4        ? gemm_mid_kernel<BM, BN, false, S::kOccupancy, PAIR, true>
+                                      : gemm_mid_kernel<BM, BN, false, S::kOccupancy, PAIR, false>;
+    const int   smem   = xs4 ? S::kSmemWindows : S::kSmem;
+    static std::atomic<bool> raised[3][64]; // dynamic LDS above the default limit needs opting in, once
+    const int   which = g.w_shuffled ? 1 : xs4 ? 2 : 0;
     if(device_id >= 0 && device_id < 64 && !raised[which][device_id])
     {
         hipError_t e =
-            hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, S::kSmem);
+            hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if(e != hipSuccess)
             return e;
         raised[which][device_id] = true;
     }
-    hipLaunchKernelGGL(kernel, dim3(tiles * splits), dim3(kThreads), S::kSmem, stream, p);
+    hipLaunchKernelGGL(kernel, dim3(tiles * splits), dim3(kThreads), smem, stream, p);
     hipError_t e = hipGetLastError();
     if(e != hipSuccess || splits == 1)
         return e;

@@ -29,6 +29,13 @@ constexpr int tile_n(int nw) { return nw * 32; }
 constexpr int slab_bytes(int nw) { return (kBM + tile_n(nw)) * 128; } // weight rows, then 256 activation rows
 constexpr int stage_bytes(int nw) { return slab_bytes(nw) + kBM * 4; } // + this K block's x_scale for the 256 rows
 constexpr uint32_t epi_pitch(int nw) { return (uint32_t)nw * 32u + 16u; } // bytes per row of a wave's 64 x NW*16 output block in LDS
+// Row-major x_scale ([M][K/128]): a lane's scale of one K block is 4 bytes of a line that holds 32 K
+// blocks of its row, and a wave's load of 64 such scales touches 64 lines.  Fetched per K block these
+// loads are a third of all line requests of the kernel for 1.5 % of its bytes (8192 x 36864 x 7168:
+// 1865 us, against 1775 us with the same scales stored column-major).  Where the rows allow 16-byte
+// loads the scales therefore come four K blocks at a time: a quarter of the requests, into two
+// windows of 16 bytes per row behind the stages.
+constexpr int kWindowBytes = kBM * 16;
 
 // 16-byte chunk c of stage row r is stored at chunk c ^ lds_swizzle(r): every group of 16 lanes
 // that the LDS serves together in a fragment read then falls on 16 different 16-byte bank groups.
@@ -44,7 +51,8 @@ __device__ __forceinline__ i32x8 read_frag(const uint8_t* base, uint32_t row, ui
 // SHUF: weights pre-shuffled (16,16).  A 16-row tile's K block is then 2 KiB of contiguous global
 // memory already in fragment order; the weight slab in LDS is a straight copy of it (tile after
 // tile), and a lane's fragment halves sit at kg*512 + l16*16 and 256 bytes further.
-template <In16 DT, bool SHUF, int NW>
+// XS4: x_scale is row-major with 16-byte aligned rows and comes in windows of four K blocks.
+template <In16 DT, bool SHUF, int NW, bool XS4>
 __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams p, int tiles_m,
                                                                 int tiles_n, int splits,
                                                                 int kb_per_split, float* partial,
@@ -56,6 +64,7 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
     constexpr uint32_t kEpiPitch = epi_pitch(NW);
     constexpr int      kLoads    = (kBM + kBN) / 64; // slab loads per wave and stage: 8 rows each, weights first
     constexpr int      kWLoads   = kBN / 64;
+    constexpr uint32_t kWindows  = (uint32_t)(kStages * kStageBytes); // the two x_scale windows (XS4)
 
     typedef const volatile i32x4 __attribute__((address_space(3)))* lds_vec_ptr;
     typedef uint8_t __attribute__((address_space(3)))*              lds_byte_ptr;
@@ -229,14 +238,20 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
         for(int i = 0; i < kLoads; ++i)
             dma16(dst0 + i * 8192, goff[i],
                   i < kWLoads ? p.wq + (size_t)kb_lo * (SHUF ? 2048 : 128) : p.xq + (size_t)kb_lo * 128);
-        if(wave < 4)
+        if(wave < 4 && XS4) // the window that holds K block kb_lo: lane l's 16 bytes are row 64 w + l's
+            dma16(__builtin_amdgcn_readfirstlane(
+                      (uint32_t)(uintptr_t)(smem3 + kWindows + ((kb_lo >> 2) & 1) * kWindowBytes + wave * 1024)),
+                  xs_goff + (uint32_t)(kb_lo & ~3) * 4u, (const uint8_t*)p.xs);
+        else if(wave < 4)
             dma4(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(smem3 + kSlabBytes + wave * 256)),
                  xs_goff + (uint32_t)kb_lo * (uint32_t)p.xs_k * 4u, p.xs);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wave's LDS-direct loads have landed
     __syncthreads();
     // LDS address of this lane's x_scale for m tile 0 (tile j sits 64 bytes further)
-    const uint32_t xs_lds = (uint32_t)kSlabBytes + ((uint32_t)wm * 64u + (uint32_t)l16) * 4u;
+    // (XS4: of this lane's row in window 0, K block 0 of the window; tile j sits 256 bytes further)
+    const uint32_t xs_lds = XS4 ? kWindows + ((uint32_t)wm * 64u + (uint32_t)l16) * 16u
+                                : (uint32_t)kSlabBytes + ((uint32_t)wm * 64u + (uint32_t)l16) * 4u;
 
     // ---- the K loop, skewed by a quarter of a K block.
     // Issue order of one iteration (4 NW MFMA slots; the numbers are those of NW = 8):
@@ -287,6 +302,14 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
 
     typedef const volatile float __attribute__((address_space(3)))* lds_f32_ptr;
 
+    // XS4: where this lane's x_scale of K block kb lies (window (kb / 4) & 1, block kb & 3 of its row).  The
+    // address of the next K block is worked out in the middle of the multiply stream, not between the barrier
+    // and the first reads of the next iteration.
+    auto xs_window_addr = [&](int kb) -> uint32_t {
+        return (uint32_t)(((kb >> 2) & 1) * kWindowBytes + (kb & 3) * 4) + xs_lds;
+    };
+    uint32_t xs_addr = XS4 ? xs_window_addr(kb_lo) : 0u;
+
     for(int kb = kb_lo; kb < kb_hi; ++kb)
     {
         const int      cur      = (kb - kb_lo) & 1;
@@ -317,7 +340,8 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
 #pragma unroll
         for(int j = 0; j < 4; ++j)
         {
-            const float xsv = *(lds_f32_ptr)(smem3 + stage + xs_lds + j * 64);
+            const float xsv = XS4 ? *(lds_f32_ptr)(smem3 + xs_addr + j * 256)
+                                  : *(lds_f32_ptr)(smem3 + stage + xs_lds + j * 64);
 #pragma unroll
             for(int g = 0; g < kScaleGroups; ++g)
                 sc[g][j] = xsv * wsc[g];
@@ -351,8 +375,25 @@ __global__ __launch_bounds__(kThreads) void gemm_prefill_kernel(GemmKernelParams
                 dma16(dma_dst + u * 8192, goff[u], u < kWLoads ? p.wq + dma_koff_w : p.xq + dma_koff);
             }
             if(q == 2 * kLoads && wave < 4)
-                dma4(__builtin_amdgcn_readfirstlane(dma_dst - wave * 1024 + kSlabBytes + wave * 256),
-                     xs_goff + (uint32_t)kn * (uint32_t)p.xs_k * 4u, p.xs);
+            {
+                if constexpr(XS4)
+                {
+                    // the next K block opens a window: into the one that was last read four K blocks ago
+                    if((kn & 3) == 0 && kn != kb)
+                        dma16(__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(
+                                  smem3 + kWindows + ((kn >> 2) & 1) * kWindowBytes + wave * 1024)),
+                              xs_goff + (uint32_t)kn * 4u, (const uint8_t*)p.xs);
+                }
+                else
+                    dma4(__builtin_amdgcn_readfirstlane(dma_dst - wave * 1024 + kSlabBytes + wave * 256),
+                         xs_goff + (uint32_t)kn * (uint32_t)p.xs_k * 4u, p.xs);
+            }
+
+            if(XS4 && q == 2 * NW)
+            {
+                xs_addr = xs_window_addr(kb + 1);
+                asm volatile("" : "+v"(xs_addr)); // here, between two slots
+            }
 
             // fold in the product issued two slots ago
             if(q == 0)
@@ -605,15 +646,20 @@ static hipError_t launch_prefill_nw(const GemmKernelParams& p, In16 out_dtype, c
     const hipStream_t stream = ctx.stream;
     const int    tiles_m = (p.M + kBM - 1) / kBM, tiles_n = (p.N + kBN - 1) / kBN;
     // the two stages, or the eight waves' output blocks of the epilogue, whichever is larger
-    const size_t smem    = std::max((size_t)kStages * stage_bytes(NW), (size_t)8 * 64 * epi_pitch(NW));
+    // x_scale in windows of four K blocks: row-major, whole windows, 16-byte aligned rows
+    const bool   xs4     = !p.w_shuffled && p.xs_k == 1 && p.xs_m == p.kblocks && (p.kblocks & 3) == 0 &&
+                           ((uintptr_t)p.xs & 15) == 0;
+    const size_t smem    = std::max((size_t)kStages * stage_bytes(NW) + (xs4 ? 2 * kWindowBytes : 0),
+                                    (size_t)8 * 64 * epi_pitch(NW));
     const bool   bf      = out_dtype == In16::bf16;
-    auto         kernel  = p.w_shuffled ? (bf ? gemm_prefill_kernel<In16::bf16, true, NW> : gemm_prefill_kernel<In16::fp16, true, NW>)
-                                        : (bf ? gemm_prefill_kernel<In16::bf16, false, NW> : gemm_prefill_kernel<In16::fp16, false, NW>);
+    auto         kernel  = p.w_shuffled ? (bf ? gemm_prefill_kernel<In16::bf16, true, NW, false> : gemm_prefill_kernel<In16::fp16, true, NW, false>)
+                           : xs4        ? (bf ? gemm_prefill_kernel<In16::bf16, false, NW, true> : gemm_prefill_kernel<In16::fp16, false, NW, true>)
+                                        : (bf ? gemm_prefill_kernel<In16::bf16, false, NW, false> : gemm_prefill_kernel<In16::fp16, false, NW, false>);
     // Per device and instantiation, once: the opt-in to more than 64 KiB of LDS.  (Racing first
     // calls repeat the same idempotent set-up.)
     constexpr int kMaxDevices = 64;
-    static std::atomic<bool> ready[kMaxDevices][4];
-    const int inst = (p.w_shuffled ? 2 : 0) + (bf ? 0 : 1);
+    static std::atomic<bool> ready[kMaxDevices][6];
+    const int inst = (p.w_shuffled ? 2 : xs4 ? 4 : 0) + (bf ? 0 : 1);
     hipError_t e;
     if(device < 0 || device >= kMaxDevices || !ready[device][inst])
     {

@@ -479,6 +479,36 @@ def test_config4_full_size(layout):
     _check_rows_against_f64(out, xq, wq, xs, ws, rows, f"config 4 {layout}")
 
 
+@pytest.mark.parametrize("name", ["prefill_256x256", "prefill_256x192", "prefill_256x128", "prefill_256x256:s=3",
+                                  "mid_128x128", "mid_64x128", "mid_64x64", "mid_128x128:s=3", "mid_64x64:s=3"])
+@pytest.mark.parametrize("k", [2560, 1152])  # 20 K blocks (x_scale fetched four blocks at a time), 9 (one at a time)
+def test_x_scale_in_windows_and_rows_not_16_byte_aligned(k, name):
+    # Row-major x_scale reaches the mid_* and prefill_* kernels four K blocks per load where its rows are
+    # 16-byte aligned.  The same values at an address 4 bytes past a 16-byte boundary must take the loads of
+    # one block each and give the same bits; with three K ranges of 20 blocks (7 + 7 + 6) the ranges start
+    # inside a window.
+    m, n = 600, 1000
+    xq, wq, xs, ws = _gpu_problem(m, n, k, seed=k, outliers=True)
+    flat = torch.empty(xs.numel() + 1, dtype=torch.float32, device=DEV)
+    shifted = flat[1:].view(xs.shape)
+    shifted.copy_(xs)
+    assert shifted.data_ptr() % 16 == 4 and shifted.is_contiguous()
+    a = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    b = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, xs, ws, a, kernelName=name)
+    aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, shifted, ws, b, kernelName=name)
+    tile = torch.empty_like(a)
+    aiter_amd.gemm_a8w8_blockscale_ck(xq, wq, xs, ws, tile, kernelName="tile_128x128")
+    torch.cuda.synchronize()
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    if ":s=" in name:  # K ranges regroup the fp32 additions
+        assert (a.view(torch.int16) != tile.view(torch.int16)).float().mean().item() < 0.02
+        rows = torch.tensor([0, 1, 255, 300, m - 1], device=DEV)
+        _check_rows_against_f64(a, xq, wq, xs, ws, rows, f"{name} {m}x{n}x{k}")
+    else:
+        assert torch.equal(a.view(torch.int16), tile.view(torch.int16))
+
+
 @pytest.mark.parametrize("m,n,k,name", [
     (512, 768, 2048, "prefill_256x256:s=2"),   # 6 tiles x 2 ranges of 8 K blocks
     (300, 1000, 1408, "prefill_256x256:s=3"),  # ragged tiles, 11 K blocks as 4 + 4 + 3
@@ -487,6 +517,7 @@ def test_config4_full_size(layout):
     (300, 1000, 1408, "prefill_256x128:s=3"),
     (512, 2112, 2048, "prefill_256x192:s=2"),  # eleven full 192-wide tiles per row of tiles, two scale blocks per wave
     (300, 1000, 1408, "prefill_256x192:s=3"),
+    (512, 768, 2560, "prefill_256x256:s=3"),   # 20 K blocks as 7 + 7 + 6: the ranges start inside a window of four x_scale blocks
     (2048, 4096, 7168, ""),                    # benchmark config 5's GEMM: the library's own choice (2 ranges)
 ])
 def test_prefill_kernel_k_ranges_across_workgroups(m, n, k, name):
