@@ -503,6 +503,7 @@ struct MoeGemmParams
     int32_t        topk;
     int32_t        waves;   // second GEMM only: waves per workgroup
     int32_t        wave_cols; // second GEMM only: columns per wave (64 or 128)
+    int32_t        out_staged; // second GEMM only: 16-bit rows leave through LDS as whole 128-byte lines
     int32_t*       where;   // first GEMM only: [M][topk] sorted position of each (token, slot) pair
     uint32_t*      block_mask; // first GEMM only: [blocks] bit r set = row r of the block is a real pair
     float*         row_info;   // first GEMM only: [slots][kRowInfo] records, see below (null: not wanted)
@@ -825,13 +826,28 @@ __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmP
 // 8 weight tiles walked two at a time with the next two already requested; the block's
 // activation rows (K = inter_dim, at most 4 K blocks on this path) stay in registers.
 // `half` 0 / 1 with `halves` 2: a wave takes the first / second half of its columns only (pairs of blocks)
+//
+// The rows it writes.  A lane holds 4 consecutive columns of one row per tile, so stored from there one
+// instruction writes 16 rows x 32 bytes: quarter lines, which the memory system pays for far beyond their
+// bytes (the 59 / 117 MB of 16-bit rows at 512 / 1024 tokens cost 28 / 41 us of the layer that way).  With
+// `out_staged` a wave parks two pairs of tiles (64 columns = one 128-byte line per row) in an LDS region of
+// its own, rows 144 bytes apart, and stores them 8 rows x 128 bytes per instruction.
+constexpr int kDownStagePitch = 144;
+constexpr int down_stage_bytes(int waves, int mt) { return waves * mt * 16 * kDownStagePitch; }
+
 template <int MT, int KB, bool STREAM>
-__device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int grp, int expert, int half = 0, int halves = 1)
+__device__ __forceinline__ void down_body(const MoeGemmParams& p, uint8_t* stage_lds, int blk, int grp, int expert, int half = 0,
+                                          int halves = 1)
 {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
     const int n0 = (grp * p.waves + wave) * p.wave_cols + half * (p.wave_cols / halves);
     if(n0 >= p.N)
         return;
+    const bool     staged = p.out_staged != 0; // uniform
+    uint8_t* const stage  = stage_lds + wave * (MT * 16 * kDownStagePitch);
+    // bit r: row r of the block (or pair of blocks) is a real row
+    const uint64_t real_rows =
+        __ballot(lane < MT * 16 && (p.sorted_ids[(size_t)blk * p.block_rows + (lane < MT * 16 ? lane : 0)] & 0xffffff) < p.M);
     i32x8 x[MT][KB];
     float xs[MT][KB];
     bool  real[MT]; // padding rows are multiplied along but not stored
@@ -881,6 +897,12 @@ __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int g
                 }
                 const size_t slot = (size_t)blk * p.block_rows + j * 16 + l16;
                 const int    col  = n + kg * 4;
+                if(staged)
+                {
+                    *(u32x2*)(stage + (j * 16 + l16) * kDownStagePitch + ((pair & 1) * 32 + i * 16 + kg * 4) * 2) =
+                        u32x2{pack2<In16::bf16>(acc[0], acc[1]), pack2<In16::bf16>(acc[2], acc[3])};
+                    continue;
+                }
                 if(!real[j])
                     continue;
                 if(p.out_f32)
@@ -888,6 +910,22 @@ __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int g
                 else
                     *(u32x2*)(p.out + slot * p.N + col) =
                         u32x2{pack2<In16::bf16>(acc[0], acc[1]), pack2<In16::bf16>(acc[2], acc[3])};
+            }
+        }
+        // every second pair (and the last one): the parked columns leave, a lane per 16 bytes, 8 rows per
+        // instruction.  The wave's LDS operations complete in the order they were issued.
+        if(staged && ((pair & 1) || pair + 1 == pairs))
+        {
+            const int first_col = n0 + (pair & ~1) * 32;
+            const int chunks    = (pair & 1) ? 8 : 4; // 16-byte pieces per row that hold columns
+            const int c         = lane & 7;
+#pragma unroll
+            for(int r0 = 0; r0 < MT * 16; r0 += 8)
+            {
+                const int   row = r0 + (lane >> 3);
+                const u32x4 v   = *(const u32x4*)(stage + row * kDownStagePitch + c * 16);
+                if(c < chunks && ((real_rows >> row) & 1))
+                    *(u32x4*)(p.out + ((size_t)blk * p.block_rows + row) * p.N + first_col + c * 8) = v;
             }
         }
     };
@@ -923,6 +961,7 @@ __device__ __forceinline__ void down_body(const MoeGemmParams& p, int blk, int g
 template <int KB, bool PAIRS>
 __global__ __launch_bounds__(512) void moe_down_kernel(MoeGemmParams p)
 {
+    extern __shared__ __attribute__((aligned(16))) uint8_t down_stage[]; // down_stage_bytes(waves, 4 or 2) when rows are staged
     const int blk = blockIdx.x / p.n_groups, grp = blockIdx.x - blk * p.n_groups;
     if(blk * p.block_rows >= p.num_valid[0])
         return;
@@ -939,11 +978,11 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeGemmParams p)
         {
             const bool full = (p.sorted_ids[(pr.first + 1) * 32 + 16] & 0xffffff) < p.M;
             if(full)
-                pr.once ? down_body<4, KB, true>(p, pr.first, grp, expert, pr.half, 2)
-                        : down_body<4, KB, false>(p, pr.first, grp, expert, pr.half, 2);
+                pr.once ? down_body<4, KB, true>(p, down_stage, pr.first, grp, expert, pr.half, 2)
+                        : down_body<4, KB, false>(p, down_stage, pr.first, grp, expert, pr.half, 2);
             else
-                pr.once ? down_body<3, KB, true>(p, pr.first, grp, expert, pr.half, 2)
-                        : down_body<3, KB, false>(p, pr.first, grp, expert, pr.half, 2);
+                pr.once ? down_body<3, KB, true>(p, down_stage, pr.first, grp, expert, pr.half, 2)
+                        : down_body<3, KB, false>(p, down_stage, pr.first, grp, expert, pr.half, 2);
             return;
         }
         once = run.alone();
@@ -951,9 +990,9 @@ __global__ __launch_bounds__(512) void moe_down_kernel(MoeGemmParams p)
     else
         once = only_block_of_its_expert(p, blk, expert);
     if(second_half)
-        once ? down_body<2, KB, true>(p, blk, grp, expert) : down_body<2, KB, false>(p, blk, grp, expert);
+        once ? down_body<2, KB, true>(p, down_stage, blk, grp, expert) : down_body<2, KB, false>(p, down_stage, blk, grp, expert);
     else
-        once ? down_body<1, KB, true>(p, blk, grp, expert) : down_body<1, KB, false>(p, blk, grp, expert);
+        once ? down_body<1, KB, true>(p, down_stage, blk, grp, expert) : down_body<1, KB, false>(p, down_stage, blk, grp, expert);
 }
 
 // The same for any K: workgroup = (block, 256 columns), wave = 64 columns, K blocks walked in turn.
@@ -1820,22 +1859,29 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
         d.wave_cols     = a.down_wave_cols == 64 ? 64 : 128;
         d.n_groups      = (a.dim + d.wave_cols * d.waves - 1) / (d.wave_cols * d.waves);
         const dim3 grid((unsigned)((size_t)a.max_blocks * d.n_groups));
+        // 16-bit rows leave through LDS as whole lines where a wave's pairs of tiles start on line boundaries
+        // and the staging region of the widest body (four row tiles with pairs of blocks, else two) stays
+        // within the LDS a launch gets without asking for more
+        const bool   pairs_inst = d.pair_blocks && d.kblocks <= 2;
+        const size_t stage      = (size_t)down_stage_bytes(d.waves, pairs_inst ? 4 : 2);
+        d.out_staged = (!y32 && a.down_staged != 0 && (a.dim & 63) == 0 && ((uintptr_t)y & 127) == 0 && stage <= 65536) ? 1 : 0;
+        const size_t lds = d.out_staged ? stage : 0;
         switch(d.kblocks)
         {
         case 1:
             if(d.pair_blocks)
-                hipLaunchKernelGGL((moe_down_kernel<1, true>), grid, dim3(64 * d.waves), 0, stream, d);
+                hipLaunchKernelGGL((moe_down_kernel<1, true>), grid, dim3(64 * d.waves), lds, stream, d);
             else
-                hipLaunchKernelGGL((moe_down_kernel<1, false>), grid, dim3(64 * d.waves), 0, stream, d);
+                hipLaunchKernelGGL((moe_down_kernel<1, false>), grid, dim3(64 * d.waves), lds, stream, d);
             break;
         case 2:
             if(d.pair_blocks)
-                hipLaunchKernelGGL((moe_down_kernel<2, true>), grid, dim3(64 * d.waves), 0, stream, d);
+                hipLaunchKernelGGL((moe_down_kernel<2, true>), grid, dim3(64 * d.waves), lds, stream, d);
             else
-                hipLaunchKernelGGL((moe_down_kernel<2, false>), grid, dim3(64 * d.waves), 0, stream, d);
+                hipLaunchKernelGGL((moe_down_kernel<2, false>), grid, dim3(64 * d.waves), lds, stream, d);
             break;
-        case 3: hipLaunchKernelGGL((moe_down_kernel<3, false>), grid, dim3(64 * d.waves), 0, stream, d); break;
-        default: hipLaunchKernelGGL((moe_down_kernel<4, false>), grid, dim3(64 * d.waves), 0, stream, d); break;
+        case 3: hipLaunchKernelGGL((moe_down_kernel<3, false>), grid, dim3(64 * d.waves), lds, stream, d); break;
+        default: hipLaunchKernelGGL((moe_down_kernel<4, false>), grid, dim3(64 * d.waves), lds, stream, d); break;
         }
     }
     else

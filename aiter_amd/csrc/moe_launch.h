@@ -67,6 +67,7 @@ struct MoeArgs
     int32_t        down_mode;      // second GEMM: 1 = rows through memory + separate sum, 2 = per-token sum in LDS
     int32_t        pair_blocks;    // consecutive blocks of one expert multiplied in pairs: 1 / 0, -1 = choose
     int32_t        fine_tail;      // first GEMM: 0 = no narrow workgroups at the end of the launch, else choose
+    int32_t        down_staged;    // second GEMM: 0 = 16-bit rows stored straight from the lanes, else through LDS as whole lines
                                    // (where its tables fit); 0 = choose
     int64_t        lda, out_stride;
     int            device_id;

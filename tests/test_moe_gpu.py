@@ -362,6 +362,22 @@ def test_fmoe_narrow_remainder_of_the_first_gemm_gives_the_same_bits(tokens):
     assert ((o - quantised).norm() / quantised.norm()).item() < 8e-3
 
 
+@pytest.mark.parametrize("tokens,dim,inter,experts,topk", [(200, 7168, 256, 32, 8), (1200, 1024, 256, 8, 8),
+                                                           (1000, 1280, 128, 6, 8), (530, 2304, 512, 16, 8)])
+def test_fmoe_rows_through_lds_give_the_same_bits(tokens, dim, inter, experts, topk):
+    # The second GEMM's 16-bit rows (written where tokens x topk x dim x 4 bytes exceed 32 MiB) leave through LDS
+    # as whole 128-byte lines; "stage=0" stores them straight from the lanes that hold them.  Same values
+    # either way: widths of 128 and 64 columns per wave (the latter with pairs of blocks is one pair of
+    # tiles per flush: half lines), a last group of columns that is partly outside the matrix, K of 1, 2, 4 blocks.
+    assert tokens * topk * dim * 4 > 32 << 20
+    p = make_moe(tokens, dim, inter, experts, topk, seed=tokens + dim)
+    for hint in ("down=rows", "down=rows,pair=1", "down=rows,pair=0", "dc=4", "dc=4,pair=1", "dw=8,pair=1", "dw=2"):
+        staged = run_moe(p, kernel_name=hint)
+        direct = run_moe(p, kernel_name=hint + ",stage=0")
+        assert torch.equal(staged.view(torch.int16), direct.view(torch.int16)), hint
+    assert_close(run_moe(p, kernel_name="down=rows"), reference(p), "rows through LDS")
+
+
 @pytest.mark.parametrize("block", [64, 128])
 def test_fmoe_pairs_of_blocks_in_arrays_sorted_in_larger_blocks(block):
     # sorted in blocks of 64 or 128 rows, the kernels' 32-row blocks of one sorted block share an expert id:
