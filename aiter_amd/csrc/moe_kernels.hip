@@ -1468,7 +1468,7 @@ __global__ __launch_bounds__(256) void moe_combine8_kernel(const uint16_t* __res
         return;
     const int32_t valid = num_valid[0] < max_padded ? num_valid[0] : max_padded;
     float         acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    constexpr int kChunk = 8;
+    constexpr int kChunk = 10; // top-8 and a shared expert in one pass
     for(int k0 = 0; k0 < topk; k0 += kChunk)
     {
         u32x4 v[kChunk];
