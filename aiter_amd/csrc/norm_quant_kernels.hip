@@ -369,6 +369,65 @@ __global__ __launch_bounds__(kQuantBlock) void group_quant_kernel(QuantKernelPar
     }
 }
 
+// Transposed scales ([groups per row][rows]) for 1x128 groups.  In the kernel above a wave's eight scales are
+// eight 4-byte stores a column apart, and the 32 rows that share a 128-byte line of a scale column are
+// quantised by workgroups that run at different times on different XCDs: every line is written in 32 pieces
+// (16384 x 7168 in a replayed graph: 67.4 us per launch against 57.4 with row-major scales).  Here a workgroup of
+// 512 lanes takes a tile of 32 rows x 4 groups, two rows per lane group (a wave: 2 rows x 1 KiB), parks the 128
+// scales in LDS and stores each column's 32 scales as one line: 62.1 us.  Of the 4.7 us that remain, 4 are the
+// tiles' strided reads (61.4 us without any scale store; tiles of 32 x 2 groups measure the same).  Same
+// arithmetic, same results.
+constexpr int kQuantTileRows = 32, kQuantTileCols = 4, kQuantTileUnits = 2;
+constexpr int kQuantTileBlock = kQuantTileRows / kQuantTileUnits * kQuantTileCols * 8;
+template <In16 DT>
+__global__ __launch_bounds__(kQuantTileBlock) void group_quant_tiles_kernel(QuantKernelParams p, uint32_t col_tiles)
+{
+    constexpr int  LPG  = 8;
+    constexpr int  kRowsPerUnit = kQuantTileRows / kQuantTileUnits;
+    const uint32_t band = blockIdx.x / col_tiles, ct = blockIdx.x - band * col_tiles;
+    const uint32_t pair = threadIdx.x / LPG, lig = threadIdx.x % LPG;
+    const uint32_t col  = ct * kQuantTileCols + pair % kQuantTileCols;
+    __shared__ float tile_scales[kQuantTileCols][kQuantTileRows];
+    u32x4 c[kQuantTileUnits][2];
+#pragma unroll
+    for(int u = 0; u < kQuantTileUnits; ++u)
+    {
+        const uint32_t row = band * kQuantTileRows + u * kRowsPerUnit + pair / kQuantTileCols;
+        if(row < p.rows && col < p.groups_per_row) // uniform over the 8 lanes of a group
+        {
+            const u32x4* src = p.x + ((size_t)row * p.groups_per_row + col) * 16 + lig * 2;
+            c[u][0]          = __builtin_nontemporal_load(src);
+            c[u][1]          = __builtin_nontemporal_load(src + 1);
+        }
+    }
+#pragma unroll
+    for(int u = 0; u < kQuantTileUnits; ++u)
+    {
+        const uint32_t r   = u * kRowsPerUnit + pair / kQuantTileCols;
+        const uint32_t row = band * kQuantTileRows + r;
+        if(row < p.rows && col < p.groups_per_row)
+        {
+            float v[16];
+            unpack8<DT>(c[u][0], v);
+            unpack8<DT>(c[u][1], v + 8);
+            u32x4 codes;
+            float s;
+            quant16<DT, LPG>(c[u][0], c[u][1], v, codes, s);
+            __builtin_nontemporal_store(codes, p.y + ((size_t)row * p.groups_per_row + col) * 8 + lig);
+            if(lig == 0)
+                tile_scales[pair % kQuantTileCols][r] = s;
+        }
+    }
+    __syncthreads();
+    if(threadIdx.x < kQuantTileCols * kQuantTileRows)
+    {
+        const uint32_t cc = threadIdx.x / kQuantTileRows, r = threadIdx.x % kQuantTileRows;
+        const uint32_t orow = band * kQuantTileRows + r, ocol = ct * kQuantTileCols + cc;
+        if(orow < p.rows && ocol < p.groups_per_row)
+            __builtin_nontemporal_store(tile_scales[cc][r], p.scale + (size_t)ocol * p.rows + orow);
+    }
+}
+
 template <In16 DT, int GS>
 static hipError_t launch_group_quant_t(const QuantArgs& a, hipStream_t stream)
 {
@@ -388,6 +447,18 @@ static hipError_t launch_group_quant_t(const QuantArgs& a, hipStream_t stream)
     const uint64_t n_groups = (uint64_t)a.rows * (uint64_t)a.groups_per_row;
     if(n_groups == 0)
         return hipSuccess;
+    if constexpr(GS == 128)
+    {
+        // transposed scales of a whole matrix (no row count on the device): by tiles of 32 rows
+        const uint64_t col_tiles = ((uint64_t)a.groups_per_row + kQuantTileCols - 1) / kQuantTileCols;
+        const uint64_t tiles     = (((uint64_t)a.rows + kQuantTileRows - 1) / kQuantTileRows) * col_tiles;
+        if(a.transpose_scale && a.num_rows == nullptr && a.rows >= kQuantTileRows && tiles < (1ull << 31))
+        {
+            hipLaunchKernelGGL((group_quant_tiles_kernel<DT>), dim3((uint32_t)tiles), dim3(kQuantTileBlock), 0, stream, p,
+                               (uint32_t)col_tiles);
+            return hipGetLastError();
+        }
+    }
     const uint32_t grid = (uint32_t)((n_groups + GPB - 1) / GPB);
     hipLaunchKernelGGL((group_quant_kernel<DT, GS, UNITS>), dim3(grid), dim3(kQuantBlock), 0, stream, p);
     return hipGetLastError();

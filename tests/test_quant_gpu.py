@@ -156,14 +156,26 @@ def test_other_group_sizes(group):
     assert_quant_bit_exact(y, s, x, group=group, what=f"group {group}")
 
 
-def test_transposed_scale_layout():
-    # csrc/kernels/quant_kernels.cu:141-148: scale[g] goes to index col*rows + row
-    x = tr.make_activation(48, 1024, seed=5)
+@pytest.mark.parametrize("rows,cols", [(48, 1024), (31, 1024), (32, 128), (33, 384), (100, 896), (257, 7168), (2048, 640)])
+def test_transposed_scale_layout(rows, cols):
+    # csrc/kernels/quant_kernels.cu:141-148: scale[g] goes to index col*rows + row.  From 32 rows on the
+    # library quantises by tiles of 32 rows x 2 groups so that a scale column's 32 rows leave as one line:
+    # ragged last bands of rows, an odd number of groups per row, fewer than 32 rows (the other kernel).
+    x = tr.make_activation(rows, cols, seed=rows + cols)
     y, s = hip_quant(x.to(DEV))
     yt, st = hip_quant(x.to(DEV), transpose_scale=True)
     assert st.shape == s.shape
     assert np.array_equal(codes8(y), codes8(yt))
-    assert np.array_equal(bits32(st).reshape(8, 48), bits32(s).T)
+    assert np.array_equal(bits32(st).reshape(cols // 128, rows), bits32(s).T)
+    assert_quant_bit_exact(y, s, x, group=128, what=f"{rows}x{cols}")
+
+
+def test_transposed_scale_layout_fp16():
+    x = tr.make_activation(70, 640, seed=3).half()
+    y, s = hip_quant(x.to(DEV))
+    yt, st = hip_quant(x.to(DEV), transpose_scale=True)
+    assert np.array_equal(codes8(y), codes8(yt))
+    assert np.array_equal(bits32(st).reshape(5, 70), bits32(s).T)
 
 
 def test_num_rows_limits_work_and_leaves_rest_untouched():
