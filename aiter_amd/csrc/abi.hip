@@ -998,7 +998,7 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
         // the reference's names pick among its tuned kernels; here "nt=1|2|4" pins the first GEMM's
         // columns per workgroup, "dw=" / "dc=" / "down=rows" pick the second GEMM that writes rows
         // (and its shape), "down=cols" the one that sums per token in LDS, "pair=0|1" whether consecutive
-        // blocks of one expert are multiplied in pairs, "tail=0" keeps the first GEMM's last blocks as wide as the rest, "stage=0" stores the second GEMM's 16-bit rows straight from the lanes instead of through LDS; several hints are joined by commas; anything else
+        // blocks of one expert are multiplied in pairs, "tail=0" keeps the first GEMM's last blocks as wide as the rest, "stage=0" stores the second GEMM's 16-bit rows straight from the lanes instead of through LDS, "ring=0" has the first GEMM's pairs of blocks request and wait for every K block in turn instead of keeping the weights two K blocks ahead; several hints are joined by commas; anything else
         // means choose
         a.gate_tiles     = 0;
         a.down_waves     = 0;
@@ -1007,6 +1007,7 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
         a.pair_blocks    = -1;
         a.fine_tail      = -1;
         a.down_staged    = -1;
+        a.gate_ring      = -1;
         for(const char* hint = kernel_name; hint && *hint;)
         {
             const char*  end = strchr(hint, ',');
@@ -1035,6 +1036,8 @@ int fmoe_fp8_blockscale_g1u1(aiter_tensor_t* out, aiter_tensor_t* input, aiter_t
                 a.fine_tail = 0;
             else if(is("stage=0"))
                 a.down_staged = 0;
+            else if(is("ring=0"))
+                a.gate_ring = 0;
             hint = end ? end + 1 : nullptr;
         }
         a.device_id         = input->device_id;

@@ -504,6 +504,7 @@ struct MoeGemmParams
     int32_t        waves;   // second GEMM only: waves per workgroup
     int32_t        wave_cols; // second GEMM only: columns per wave (64 or 128)
     int32_t        out_staged; // second GEMM only: 16-bit rows leave through LDS as whole 128-byte lines
+    int32_t        gate_ring;  // first GEMM, pairs of blocks: weights two K blocks ahead through LDS (gate_up_ring_body)
     int32_t*       where;   // first GEMM only: [M][topk] sorted position of each (token, slot) pair
     uint32_t*      block_mask; // first GEMM only: [blocks] bit r set = row r of the block is a real pair
     float*         row_info;   // first GEMM only: [slots][kRowInfo] records, see below (null: not wanted)
@@ -625,6 +626,43 @@ __device__ __forceinline__ PairOfBlocks pair_of_blocks(const MoeGemmParams& p, c
 constexpr int kGateUpWaves = 8;
 constexpr int kChipCus     = 256;
 
+// The eight waves' sums of a block meet in LDS (red[wave][n tile][lane][c], one m tile at a time); wave i adds
+// them in wave order, applies the activation to the pair (gate tile i, up tile NT + i) and stores the product.
+template <int MT, int NT>
+__device__ __forceinline__ void gate_up_finish(const MoeGemmParams& p, float* red, const f32x4 (&acc)[MT][2 * NT], int blk, int grp)
+{
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
+#pragma unroll
+    for(int j = 0; j < MT; ++j)
+    {
+        if(j > 0)
+            __syncthreads();
+#pragma unroll
+        for(int i = 0; i < 2 * NT; ++i)
+            *(f32x4*)(red + (((size_t)wave * (2 * NT) + i) * 64 + lane) * 4) = acc[j][i];
+        __syncthreads();
+        if(wave < NT) // wave i finishes the pair (gate tile i, up tile NT + i)
+        {
+            const int i = wave;
+            f32x4     g = f32x4{0.f, 0.f, 0.f, 0.f}, u = g;
+#pragma unroll
+            for(int w = 0; w < kGateUpWaves; ++w) // wave order: the sum does not depend on timing
+            {
+                g += *(const f32x4*)(red + (((size_t)w * (2 * NT) + i) * 64 + lane) * 4);
+                u += *(const f32x4*)(red + (((size_t)w * (2 * NT) + NT + i) * 64 + lane) * 4);
+            }
+            float h[4];
+#pragma unroll
+            for(int c = 0; c < 4; ++c)
+                h[c] = activate(g[c], p.activation) * u[c];
+            const int slot = blk * p.block_rows + j * 16 + l16;
+            const int col  = (grp * NT + i) * 16 + kg * 4;
+            *(u32x2*)(p.out + (size_t)slot * p.inter + col) =
+                u32x2{pack2<In16::bf16>(h[0], h[1]), pack2<In16::bf16>(h[2], h[3])};
+        }
+    }
+}
+
 template <int MT, int NT, bool STREAM>
 __device__ __forceinline__ void gate_up_body(const MoeGemmParams& p, float* red, int blk, int grp, int expert)
 {
@@ -683,35 +721,237 @@ __device__ __forceinline__ void gate_up_body(const MoeGemmParams& p, float* red,
             }
     }
 
-    // red[wave][n tile][lane][c], one m tile at a time
+    gate_up_finish<MT, NT>(p, red, acc, blk, grp);
+}
+
+// The first GEMM for a pair of blocks (NT = 2: two gate tiles and their up tiles, MT = 3 or 4 row tiles), with
+// the weights two K blocks ahead.
+//
+// In gate_up_body a wave asks for a K block, waits, multiplies, and has nothing in flight while it multiplies.
+// With 16 MFMAs and 64 FMAs per 8 KiB of weights and eight waves per compute unit (the registers allow no more)
+// that launch is bound by the latency of its loads: 4.9 TB/s at 1024 tokens where the narrower bodies, with
+// twice the bytes per request, stream at 6.3.  Requesting the next K block into a second set of registers does
+// not fit (256 registers and 407 spilled).  Here the weights travel through LDS instead: every wave owns two
+// stages of 8 KiB that direct global->LDS loads fill (global_load_lds_dwordx4: no registers while in flight),
+// so the weights of K blocks i + 1 and i + 2 are on their way while block i is multiplied; the token rows and
+// their scales of block i + 1 are requested into a second set of registers.
+//
+// Loads return in order, so the order of issue decides what a wait can leave in flight:
+//   ids W(0) W(1) X(0) | X(1) W(2) | X(2) W(3) | ...    (X: 3 MT register loads, W: 8 LDS-direct loads)
+// Iteration i > 0 needs X(i) and W(i); the only younger loads are W(i + 1)'s eight: s_waitcnt vmcnt(8) (0 when
+// there is no W(i + 1), and in iteration 0, whose X is the youngest).  It then copies W(i) from its stage into registers, which frees the stage for
+// W(i + 2).  All of these loads are issued from asm, invisible to the compiler's wait counts; the compiler
+// itself issues no vector memory loads inside the loop.  Products, scales and their order are those of
+// gate_up_body: same bits.
+// a pointer that is the same in every lane, said so to the compiler (asm operands that must be scalar registers)
+template <typename T>
+__device__ __forceinline__ const T* uniform_ptr(const T* ptr)
+{
+    const uint64_t v  = (uint64_t)(uintptr_t)ptr;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const T*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+
+constexpr int kRingStageBytes = 4 * 2048;                                  // four 16-row tiles of one K block
+constexpr int kRingLdsBytes   = kGateUpWaves * 2 * kRingStageBytes;        // two stages per wave: 128 KiB
+
+template <int MT, bool STREAM>
+__device__ __forceinline__ void gate_up_ring_body(const MoeGemmParams& p, uint8_t* lds, int blk, int grp, int expert)
+{
+    constexpr int NT = 2;
+    const int t = threadIdx.x, lane = t & 63, l16 = lane & 15, kg = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6); // scalar: K blocks, stages and scale addresses derive from it
+    typedef uint8_t __attribute__((address_space(3)))*              lds_byte_ptr;
+    typedef const volatile i32x4 __attribute__((address_space(3)))* lds_vec_ptr;
+    const lds_byte_ptr lds3 = (lds_byte_ptr)lds;
+
+    // The rows' token ids are asked for first (from asm as well: a load the compiler knows of would make it
+    // wait for everything issued before its use), so that the first weights can be requested while they travel.
+    int      row_id[MT];
+    uint32_t xoff[MT], xsoff[MT]; // per-lane byte offsets of the token rows and of their scales, once the ids are here
+    {
+        const int32_t* ids = uniform_ptr(p.sorted_ids);
+#pragma unroll
+        for(int j = 0; j < MT; ++j)
+        {
+            const uint32_t at = (uint32_t)(blk * p.block_rows + j * 16 + l16) * 4u;
+            asm volatile("global_load_dword %0, %1, %2" : "=v"(row_id[j]) : "v"(at), "s"(ids) : "memory");
+        }
+    }
+    const size_t   tile_stride = (size_t)16 * (size_t)p.K;
+    const size_t   wexp = (size_t)expert * (size_t)p.N * (size_t)p.K;
+    const uint8_t* wt[2 * NT]; // uniform: the wave's four tiles (gate, gate, up, up)
+#pragma unroll
+    for(int i = 0; i < NT; ++i)
+    {
+        wt[i]      = p.w + wexp + (size_t)(grp * NT + i) * tile_stride;
+        wt[NT + i] = p.w + wexp + (size_t)((p.inter >> 4) + grp * NT + i) * tile_stride;
+    }
+    // (read through the constant address space at scalar addresses, i.e. with scalar loads: a vector load here
+    // would make the compiler wait for every load in flight)
+    typedef const float __attribute__((address_space(4)))* const_f32_ptr;
+    const const_f32_ptr ws_gate = (const_f32_ptr)(uintptr_t)uniform_ptr(p.wsc + ((size_t)expert * (p.N / 128) + (grp * NT * 16) / 128) * p.kblocks);
+    const const_f32_ptr ws_up   = (const_f32_ptr)(uintptr_t)uniform_ptr(p.wsc + ((size_t)expert * (p.N / 128) + (p.inter + grp * NT * 16) / 128) * p.kblocks);
+
+    const uint32_t stage0   = (uint32_t)(uintptr_t)(lds3 + wave * (2 * kRingStageBytes));
+    const uint32_t lane16   = (uint32_t)lane * 16u, lane16b = lane16 + 1024u;
+    const uint32_t frag_off = (uint32_t)kg * 512u + (uint32_t)l16 * 16u;
+
+    // W(kb) -> stage: per tile two loads of 1 KiB (lane l's 16 bytes land at M0 + 16 l)
+    auto issue_w = [&](int kb, int stage) {
+#pragma unroll
+        for(int i = 0; i < 2 * NT; ++i)
+        {
+            const uint8_t* base = uniform_ptr(wt[i] + (size_t)kb * 2048);
+            const uint32_t dst  = __builtin_amdgcn_readfirstlane(stage0 + (uint32_t)stage * kRingStageBytes + (uint32_t)i * 2048u);
+            if constexpr(STREAM)
+            {
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(lane16), "s"(base) : "memory");
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst + 1024u), "v"(lane16b), "s"(base) : "memory");
+            }
+            else
+            {
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane16), "s"(base) : "memory");
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst + 1024u), "v"(lane16b), "s"(base) : "memory");
+            }
+        }
+    };
+    struct Rows
+    {
+        i32x4 lo[MT], hi[MT];
+        float xs[MT];
+    };
+    // X(kb) -> registers (not valid before the wait that names them)
+    auto issue_x = [&](int kb, Rows& r) {
+        const uint8_t* xbase  = uniform_ptr(p.xq + (size_t)kb * 128);
+        const float*   xsbase = uniform_ptr(p.xs + (size_t)kb * p.M);
+#pragma unroll
+        for(int j = 0; j < MT; ++j)
+        {
+            asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r.lo[j]) : "v"(xoff[j]), "s"(xbase) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, %2 offset:16" : "=v"(r.hi[j]) : "v"(xoff[j]), "s"(xbase) : "memory");
+            asm volatile("global_load_dword %0, %1, %2" : "=v"(r.xs[j]) : "v"(xsoff[j]), "s"(xsbase) : "memory");
+        }
+    };
+    // the wait of an iteration: everything but the eight youngest loads (W of the next K block) has arrived
+    auto arrived = [&](Rows& r, bool next_w_in_flight) {
+        if(next_w_in_flight)
+            asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for(int j = 0; j < MT; ++j)
+            asm volatile("" : "+v"(r.lo[j]), "+v"(r.hi[j]), "+v"(r.xs[j]));
+    };
+
+    f32x4 acc[MT][2 * NT];
+#pragma unroll
+    for(int j = 0; j < MT; ++j)
+#pragma unroll
+        for(int i = 0; i < 2 * NT; ++i)
+            acc[j][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int n = wave < p.kblocks ? (p.kblocks - wave + kGateUpWaves - 1) / kGateUpWaves : 0; // this wave's K blocks
+    auto kb_of = [&](int i) { return wave + i * kGateUpWaves; };
+
+    auto step = [&](int i, Rows& cur, Rows& nxt) {
+        arrived(cur, i > 0 && i + 1 < n);
+        i32x8 w[2 * NT];
+#pragma unroll
+        for(int q = 0; q < 2 * NT; ++q)
+        {
+            const uint32_t at = (uint32_t)(wave * (2 * kRingStageBytes) + (i & 1) * kRingStageBytes + q * 2048) + frag_off;
+            const i32x4    lo = *(lds_vec_ptr)(lds3 + at);
+            const i32x4    hi = *(lds_vec_ptr)(lds3 + at + 256);
+            w[q]              = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+        // the fragments are in registers (the compiler waits for its LDS reads here): the stage is free
+#pragma unroll
+        for(int q = 0; q < 2 * NT; ++q)
+            asm volatile("" : "+v"(w[q]));
+        if(i + 1 < n)
+            issue_x(kb_of(i + 1), nxt);
+        if(i + 2 < n)
+            issue_w(kb_of(i + 2), i & 1);
+        const int   kb = kb_of(i);
+        const float sg = ws_gate[kb], su = ws_up[kb];
+#pragma unroll
+        for(int j = 0; j < MT; ++j)
+        {
+            const i32x8 x = i32x8{cur.lo[j][0], cur.lo[j][1], cur.lo[j][2], cur.lo[j][3],
+                                  cur.hi[j][0], cur.hi[j][1], cur.hi[j][2], cur.hi[j][3]};
+#pragma unroll
+            for(int q = 0; q < 2 * NT; ++q)
+            {
+                const f32x4 prod = mfma_16x16x128_fp8(w[q], x, f32x4{0.f, 0.f, 0.f, 0.f});
+                const float sc   = cur.xs[j] * (q < NT ? sg : su);
+#pragma unroll
+                for(int c = 0; c < 4; ++c)
+                    acc[j][q][c] = __builtin_fmaf(prod[c], sc, acc[j][q][c]);
+            }
+        }
+    };
+
+    // ids | W(0) W(1) | wait for the ids | X(0): the first iteration waits for everything
+    Rows ra, rb;
+    if(n > 0)
+        issue_w(kb_of(0), 0);
+    if(n > 1)
+        issue_w(kb_of(1), 1);
+    if(n > 1)
+        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else if(n > 0)
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // the token rows: 32 bytes of every K block per lane
 #pragma unroll
     for(int j = 0; j < MT; ++j)
     {
-        if(j > 0)
-            __syncthreads();
+        asm volatile("" : "+v"(row_id[j]));
+        const int id  = row_id[j] & 0xffffff;
+        const int tok = id < p.M ? id : 0; // padding rows compute on token 0 and are never read
+        xoff[j]       = (uint32_t)tok * (uint32_t)p.lda + (uint32_t)kg * 32u;
+        xsoff[j]      = (uint32_t)tok * 4u;
+    }
+    if(n > 0)
+        issue_x(kb_of(0), ra);
+    for(int i = 0; i < n; i += 2)
+    {
+        step(i, ra, rb);
+        if(i + 1 < n)
+            step(i + 1, rb, ra);
+    }
+    // The sums meet where the stages were (every wave must be done with its stages first), all MT row tiles at
+    // once: red[row tile][wave][n tile][lane][c] is MT x 32 KiB, and wave 2 j + i adds up the pair (gate tile i,
+    // up tile NT + i) of row tile j in wave order, as gate_up_finish does one row tile after the other with two
+    // of the eight waves (a compute unit holds one such workgroup and requests nothing while it finishes).
+    __syncthreads();
+    float* const red = (float*)lds;
 #pragma unroll
-        for(int i = 0; i < 2 * NT; ++i)
-            *(f32x4*)(red + (((size_t)wave * (2 * NT) + i) * 64 + lane) * 4) = acc[j][i];
-        __syncthreads();
-        if(wave < NT) // wave i finishes the pair (gate tile i, up tile NT + i)
+    for(int j = 0; j < MT; ++j)
+#pragma unroll
+        for(int q = 0; q < 2 * NT; ++q)
+            *(f32x4*)(red + ((((size_t)j * kGateUpWaves + wave) * (2 * NT) + q) * 64 + lane) * 4) = acc[j][q];
+    __syncthreads();
+    const int j = wave / NT, i = wave % NT;
+    if(j < MT)
+    {
+        f32x4 g = f32x4{0.f, 0.f, 0.f, 0.f}, u = g;
+#pragma unroll
+        for(int w = 0; w < kGateUpWaves; ++w) // wave order: the sum does not depend on timing
         {
-            const int i = wave;
-            f32x4     g = f32x4{0.f, 0.f, 0.f, 0.f}, u = g;
-#pragma unroll
-            for(int w = 0; w < kGateUpWaves; ++w) // wave order: the sum does not depend on timing
-            {
-                g += *(const f32x4*)(red + (((size_t)w * (2 * NT) + i) * 64 + lane) * 4);
-                u += *(const f32x4*)(red + (((size_t)w * (2 * NT) + NT + i) * 64 + lane) * 4);
-            }
-            float h[4];
-#pragma unroll
-            for(int c = 0; c < 4; ++c)
-                h[c] = activate(g[c], p.activation) * u[c];
-            const int slot = blk * p.block_rows + j * 16 + l16;
-            const int col  = (grp * NT + i) * 16 + kg * 4;
-            *(u32x2*)(p.out + (size_t)slot * p.inter + col) =
-                u32x2{pack2<In16::bf16>(h[0], h[1]), pack2<In16::bf16>(h[2], h[3])};
+            g += *(const f32x4*)(red + ((((size_t)j * kGateUpWaves + w) * (2 * NT) + i) * 64 + lane) * 4);
+            u += *(const f32x4*)(red + ((((size_t)j * kGateUpWaves + w) * (2 * NT) + NT + i) * 64 + lane) * 4);
         }
+        float h[4];
+#pragma unroll
+        for(int c = 0; c < 4; ++c)
+            h[c] = activate(g[c], p.activation) * u[c];
+        const int slot = blk * p.block_rows + j * 16 + l16;
+        const int col  = (grp * NT + i) * 16 + kg * 4;
+        *(u32x2*)(p.out + (size_t)slot * p.inter + col) =
+            u32x2{pack2<In16::bf16>(h[0], h[1]), pack2<In16::bf16>(h[2], h[3])};
     }
 }
 
@@ -720,7 +960,11 @@ __device__ __forceinline__ void gate_up_body(const MoeGemmParams& p, float* red,
 template <int NT, bool PAIRS>
 __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmParams p)
 {
-    __shared__ __attribute__((aligned(16))) float red_dyn[kGateUpWaves * 2 * NT * 64 * 4];
+    // the pairs instance is launched with kRingLdsBytes of dynamic LDS: the ring of gate_up_ring_body, and
+    // every body's reduction buffer in its first 64 KiB
+    extern __shared__ __attribute__((aligned(1024))) uint8_t gate_up_lds[];
+    __shared__ __attribute__((aligned(16))) float red_static[PAIRS ? 4 : kGateUpWaves * 2 * NT * 64 * 4];
+    float* const red_dyn = PAIRS ? (float*)gate_up_lds : red_static;
     // Blocks are taken from the last valid one down: the experts with the highest ids come first.  A
     // shared expert, which every token is routed to and which conventionally has the last id, has the
     // most blocks, each of two full row tiles and read with ordinary loads: started first, they are not
@@ -804,6 +1048,16 @@ __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmP
             // block's second half only if it holds real rows (the first block of a pair is full)
             const int  group = pr.half * p.n_groups + grp;
             const bool full  = (p.sorted_ids[(pr.first + 1) * 32 + 16] & 0xffffff) < p.M;
+            if(p.gate_ring)
+            {
+                if(full)
+                    pr.once ? gate_up_ring_body<4, true>(p, gate_up_lds, pr.first, group, expert)
+                            : gate_up_ring_body<4, false>(p, gate_up_lds, pr.first, group, expert);
+                else
+                    pr.once ? gate_up_ring_body<3, true>(p, gate_up_lds, pr.first, group, expert)
+                            : gate_up_ring_body<3, false>(p, gate_up_lds, pr.first, group, expert);
+                return;
+            }
             if(full)
                 pr.once ? gate_up_body<4, 2, true>(p, red_dyn, pr.first, group, expert)
                         : gate_up_body<4, 2, false>(p, red_dyn, pr.first, group, expert);
@@ -1785,7 +2039,22 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
         {
         case 4:
             if(p.pair_blocks)
-                hipLaunchKernelGGL((moe_gate_up_kernel<4, true>), grid, dim3(64 * kGateUpWaves), 0, stream, p);
+            {
+                // the pairs instance keeps its LDS (ring and reduction buffer) in the dynamic segment: opt in once
+                static std::atomic<bool> raised[64];
+                if(a.device_id < 0 || a.device_id >= 64 || !raised[a.device_id])
+                {
+                    e = hipFuncSetAttribute((const void*)moe_gate_up_kernel<4, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            kRingLdsBytes);
+                    if(e != hipSuccess)
+                        return e;
+                    if(a.device_id >= 0 && a.device_id < 64)
+                        raised[a.device_id] = true;
+                }
+                // 32-bit byte offsets of the token rows in the ring body
+                p.gate_ring = (a.gate_ring != 0 && (uint64_t)a.M * (uint64_t)a.lda < (1ull << 32) && (uint64_t)a.M * 4 < (1ull << 32)) ? 1 : 0;
+                hipLaunchKernelGGL((moe_gate_up_kernel<4, true>), grid, dim3(64 * kGateUpWaves), kRingLdsBytes, stream, p);
+            }
             else
                 hipLaunchKernelGGL((moe_gate_up_kernel<4, false>), grid, dim3(64 * kGateUpWaves), 0, stream, p);
             break;

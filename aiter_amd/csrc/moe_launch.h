@@ -68,6 +68,7 @@ struct MoeArgs
     int32_t        pair_blocks;    // consecutive blocks of one expert multiplied in pairs: 1 / 0, -1 = choose
     int32_t        fine_tail;      // first GEMM: 0 = no narrow workgroups at the end of the launch, else choose
     int32_t        down_staged;    // second GEMM: 0 = 16-bit rows stored straight from the lanes, else through LDS as whole lines
+    int32_t        gate_ring;      // first GEMM, pairs of blocks: 0 = every K block requested and waited for in turn, else weights two K blocks ahead through LDS
                                    // (where its tables fit); 0 = choose
     int64_t        lda, out_stride;
     int            device_id;
