@@ -626,40 +626,41 @@ __device__ __forceinline__ PairOfBlocks pair_of_blocks(const MoeGemmParams& p, c
 constexpr int kGateUpWaves = 8;
 constexpr int kChipCus     = 256;
 
-// The eight waves' sums of a block meet in LDS (red[wave][n tile][lane][c], one m tile at a time); wave i adds
-// them in wave order, applies the activation to the pair (gate tile i, up tile NT + i) and stores the product.
+// The eight waves' sums of a block meet in LDS, all MT row tiles at once: red[row tile][wave][n tile][lane][c]
+// (MT x NT x 16 KiB), and wave NT j + i adds up the pair (gate tile i, up tile NT + i) of row tile j in wave
+// order (the sum does not depend on timing), applies the activation and stores the product.  One row tile
+// after the other, with NT of the eight waves at work, a compute unit that holds a single workgroup requested
+// nothing for as many rounds as there are row tiles.
+constexpr size_t gate_up_red_bytes(int mt, int nt) { return (size_t)mt * kGateUpWaves * 2 * nt * 64 * 16; }
 template <int MT, int NT>
 __device__ __forceinline__ void gate_up_finish(const MoeGemmParams& p, float* red, const f32x4 (&acc)[MT][2 * NT], int blk, int grp)
 {
+    static_assert(MT * NT <= kGateUpWaves, "a wave per (row tile, column pair)");
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, l16 = lane & 15, kg = lane >> 4;
 #pragma unroll
     for(int j = 0; j < MT; ++j)
+#pragma unroll
+        for(int q = 0; q < 2 * NT; ++q)
+            *(f32x4*)(red + ((((size_t)j * kGateUpWaves + wave) * (2 * NT) + q) * 64 + lane) * 4) = acc[j][q];
+    __syncthreads();
+    const int j = wave / NT, i = wave % NT;
+    if(j < MT)
     {
-        if(j > 0)
-            __syncthreads();
+        f32x4 g = f32x4{0.f, 0.f, 0.f, 0.f}, u = g;
 #pragma unroll
-        for(int i = 0; i < 2 * NT; ++i)
-            *(f32x4*)(red + (((size_t)wave * (2 * NT) + i) * 64 + lane) * 4) = acc[j][i];
-        __syncthreads();
-        if(wave < NT) // wave i finishes the pair (gate tile i, up tile NT + i)
+        for(int w = 0; w < kGateUpWaves; ++w)
         {
-            const int i = wave;
-            f32x4     g = f32x4{0.f, 0.f, 0.f, 0.f}, u = g;
-#pragma unroll
-            for(int w = 0; w < kGateUpWaves; ++w) // wave order: the sum does not depend on timing
-            {
-                g += *(const f32x4*)(red + (((size_t)w * (2 * NT) + i) * 64 + lane) * 4);
-                u += *(const f32x4*)(red + (((size_t)w * (2 * NT) + NT + i) * 64 + lane) * 4);
-            }
-            float h[4];
-#pragma unroll
-            for(int c = 0; c < 4; ++c)
-                h[c] = activate(g[c], p.activation) * u[c];
-            const int slot = blk * p.block_rows + j * 16 + l16;
-            const int col  = (grp * NT + i) * 16 + kg * 4;
-            *(u32x2*)(p.out + (size_t)slot * p.inter + col) =
-                u32x2{pack2<In16::bf16>(h[0], h[1]), pack2<In16::bf16>(h[2], h[3])};
+            g += *(const f32x4*)(red + ((((size_t)j * kGateUpWaves + w) * (2 * NT) + i) * 64 + lane) * 4);
+            u += *(const f32x4*)(red + ((((size_t)j * kGateUpWaves + w) * (2 * NT) + NT + i) * 64 + lane) * 4);
         }
+        float h[4];
+#pragma unroll
+        for(int c = 0; c < 4; ++c)
+            h[c] = activate(g[c], p.activation) * u[c];
+        const int slot = blk * p.block_rows + j * 16 + l16;
+        const int col  = (grp * NT + i) * 16 + kg * 4;
+        *(u32x2*)(p.out + (size_t)slot * p.inter + col) =
+            u32x2{pack2<In16::bf16>(h[0], h[1]), pack2<In16::bf16>(h[2], h[3])};
     }
 }
 
@@ -922,37 +923,15 @@ __device__ __forceinline__ void gate_up_ring_body(const MoeGemmParams& p, uint8_
         if(i + 1 < n)
             step(i + 1, rb, ra);
     }
-    // The sums meet where the stages were (every wave must be done with its stages first), all MT row tiles at
-    // once: red[row tile][wave][n tile][lane][c] is MT x 32 KiB, and wave 2 j + i adds up the pair (gate tile i,
-    // up tile NT + i) of row tile j in wave order, as gate_up_finish does one row tile after the other with two
-    // of the eight waves (a compute unit holds one such workgroup and requests nothing while it finishes).
+    // the sums meet where the stages were: every wave must be done with its stages first
     __syncthreads();
-    float* const red = (float*)lds;
-#pragma unroll
-    for(int j = 0; j < MT; ++j)
-#pragma unroll
-        for(int q = 0; q < 2 * NT; ++q)
-            *(f32x4*)(red + ((((size_t)j * kGateUpWaves + wave) * (2 * NT) + q) * 64 + lane) * 4) = acc[j][q];
-    __syncthreads();
-    const int j = wave / NT, i = wave % NT;
-    if(j < MT)
-    {
-        f32x4 g = f32x4{0.f, 0.f, 0.f, 0.f}, u = g;
-#pragma unroll
-        for(int w = 0; w < kGateUpWaves; ++w) // wave order: the sum does not depend on timing
-        {
-            g += *(const f32x4*)(red + ((((size_t)j * kGateUpWaves + w) * (2 * NT) + i) * 64 + lane) * 4);
-            u += *(const f32x4*)(red + ((((size_t)j * kGateUpWaves + w) * (2 * NT) + NT + i) * 64 + lane) * 4);
-        }
-        float h[4];
-#pragma unroll
-        for(int c = 0; c < 4; ++c)
-            h[c] = activate(g[c], p.activation) * u[c];
-        const int slot = blk * p.block_rows + j * 16 + l16;
-        const int col  = (grp * NT + i) * 16 + kg * 4;
-        *(u32x2*)(p.out + (size_t)slot * p.inter + col) =
-            u32x2{pack2<In16::bf16>(h[0], h[1]), pack2<In16::bf16>(h[2], h[3])};
-    }
+    gate_up_finish<MT, NT>(p, (float*)lds, acc, blk, grp);
+}
+
+// LDS of an instance: two row tiles of its own width, or (pairs) four of half the width, which is the ring's size
+constexpr size_t gate_up_lds_bytes(int nt, bool pairs)
+{
+    return pairs ? (gate_up_red_bytes(4, 2) > (size_t)kRingLdsBytes ? gate_up_red_bytes(4, 2) : (size_t)kRingLdsBytes) : gate_up_red_bytes(2, nt);
 }
 
 // PAIRS: the instance that can multiply pairs of blocks, kept apart from the usual one (which needs
@@ -960,11 +939,10 @@ __device__ __forceinline__ void gate_up_ring_body(const MoeGemmParams& p, uint8_
 template <int NT, bool PAIRS>
 __global__ __launch_bounds__(64 * kGateUpWaves) void moe_gate_up_kernel(MoeGemmParams p)
 {
-    // the pairs instance is launched with kRingLdsBytes of dynamic LDS: the ring of gate_up_ring_body, and
-    // every body's reduction buffer in its first 64 KiB
+    // dynamic LDS: the reduction buffer of the widest body of the instance (gate_up_lds_bytes), which in the
+    // pairs instance is also the ring of gate_up_ring_body
     extern __shared__ __attribute__((aligned(1024))) uint8_t gate_up_lds[];
-    __shared__ __attribute__((aligned(16))) float red_static[PAIRS ? 4 : kGateUpWaves * 2 * NT * 64 * 4];
-    float* const red_dyn = PAIRS ? (float*)gate_up_lds : red_static;
+    float* const red_dyn = (float*)gate_up_lds;
     // Blocks are taken from the last valid one down: the experts with the highest ids come first.  A
     // shared expert, which every token is routed to and which conventionally has the last id, has the
     // most blocks, each of two full row tiles and read with ordinary loads: started first, they are not
@@ -2035,32 +2013,27 @@ hipError_t launch_fmoe_blockscale(const MoeArgs& a, hipStream_t stream, const ch
         p.fine_blocks = (nt == 4 && a.fine_tail != 0) ? std::min(a.max_blocks, kChipCus / 4 / p.n_groups) : 0;
         // (blocks rounded up to a multiple of 8: the kernel deals them out to the 8 XCDs)
         const dim3 grid((unsigned)((size_t)((a.max_blocks + 7) & ~7) * p.n_groups + (size_t)p.fine_blocks * 4 * p.n_groups));
-        switch(nt)
+        // every instance keeps its LDS (reduction buffer; ring of the pairs instance) in the dynamic segment:
+        // opt in to more than 64 KiB once per device and instance
+        const bool paired = nt == 4 && p.pair_blocks;
+        auto kernel = paired     ? moe_gate_up_kernel<4, true>
+                      : nt == 4 ? moe_gate_up_kernel<4, false>
+                      : nt == 2 ? moe_gate_up_kernel<2, false>
+                                : moe_gate_up_kernel<1, false>;
+        const size_t lds = gate_up_lds_bytes(nt, paired);
+        static std::atomic<bool> raised[64][4];
+        const int inst = paired ? 3 : nt == 4 ? 2 : nt == 2 ? 1 : 0;
+        if(lds > 65536 && (a.device_id < 0 || a.device_id >= 64 || !raised[a.device_id][inst]))
         {
-        case 4:
-            if(p.pair_blocks)
-            {
-                // the pairs instance keeps its LDS (ring and reduction buffer) in the dynamic segment: opt in once
-                static std::atomic<bool> raised[64];
-                if(a.device_id < 0 || a.device_id >= 64 || !raised[a.device_id])
-                {
-                    e = hipFuncSetAttribute((const void*)moe_gate_up_kernel<4, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                            kRingLdsBytes);
-                    if(e != hipSuccess)
-                        return e;
-                    if(a.device_id >= 0 && a.device_id < 64)
-                        raised[a.device_id] = true;
-                }
-                // 32-bit byte offsets of the token rows in the ring body
-                p.gate_ring = (a.gate_ring != 0 && (uint64_t)a.M * (uint64_t)a.lda < (1ull << 32) && (uint64_t)a.M * 4 < (1ull << 32)) ? 1 : 0;
-                hipLaunchKernelGGL((moe_gate_up_kernel<4, true>), grid, dim3(64 * kGateUpWaves), kRingLdsBytes, stream, p);
-            }
-            else
-                hipLaunchKernelGGL((moe_gate_up_kernel<4, false>), grid, dim3(64 * kGateUpWaves), 0, stream, p);
-            break;
-        case 2: hipLaunchKernelGGL((moe_gate_up_kernel<2, false>), grid, dim3(64 * kGateUpWaves), 0, stream, p); break;
-        default: hipLaunchKernelGGL((moe_gate_up_kernel<1, false>), grid, dim3(64 * kGateUpWaves), 0, stream, p); break;
+            e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if(e != hipSuccess)
+                return e;
+            if(a.device_id >= 0 && a.device_id < 64)
+                raised[a.device_id][inst] = true;
         }
+        // (32-bit byte offsets of the token rows in the ring body)
+        p.gate_ring = (paired && a.gate_ring != 0 && (uint64_t)a.M * (uint64_t)a.lda < (1ull << 32) && (uint64_t)a.M * 4 < (1ull << 32)) ? 1 : 0;
+        hipLaunchKernelGGL(kernel, grid, dim3(64 * kGateUpWaves), lds, stream, p);
     }
 
     QuantArgs qa{};
