@@ -328,7 +328,9 @@ def test_fmoe_tuning_hints_do_not_change_the_result(hint):
 
 
 @pytest.mark.parametrize("tokens,dim,inter,experts,topk", [(300, 512, 256, 4, 2), (200, 7168, 256, 32, 8),
-                                                           (70, 1024, 128, 3, 2), (330, 512, 256, 5, 1)])
+                                                           (70, 1024, 128, 3, 2), (330, 512, 256, 5, 1),
+                                                           (260, 2048, 256, 4, 2), (260, 1536, 256, 3, 2),
+                                                           (190, 3328, 512, 3, 2)])
 def test_fmoe_pairs_of_blocks_give_the_same_bits(tokens, dim, inter, experts, topk):
     # Where the average expert has 32 rows or more the library multiplies two consecutive blocks of an expert
     # together (their workgroups take half the columns each for the rows of both).  Every product is summed in
@@ -341,6 +343,10 @@ def test_fmoe_pairs_of_blocks_give_the_same_bits(tokens, dim, inter, experts, to
         paired = run_moe(p, kernel_name=f"pair=1,{down}")
         assert torch.equal(single.view(torch.int16), paired.view(torch.int16)), down
         assert_close(paired, refs, f"pairs of blocks, {down}")
+        # the first GEMM's pairs with the weights two K blocks ahead through LDS, and without: a wave has
+        # 0, 1, 2, 3 or 7 K blocks in these shapes (4, 8, 12, 16, 26 and 56 K blocks over eight waves)
+        plain = run_moe(p, kernel_name=f"pair=1,ring=0,{down}")
+        assert torch.equal(plain.view(torch.int16), paired.view(torch.int16)), f"ring, {down}"
     if tokens * topk >= 28 * experts:  # the library's own choice is then the paired form
         assert torch.equal(run_moe(p).view(torch.int16), run_moe(p, kernel_name="pair=1").view(torch.int16))
 
