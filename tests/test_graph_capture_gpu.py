@@ -96,3 +96,34 @@ def test_moe_under_graph_replay_with_changing_routing():
         return [tw, ti, out]
 
     replay_and_compare(build, refill, run)
+
+
+def test_moe_with_many_rows_per_expert_under_graph_replay():
+    # 200 rows per expert: pairs of blocks (the first GEMM's LDS ring, 128 KiB of dynamic LDS), the second GEMM
+    # by rows (16-bit rows through LDS) and the separate per-token sum, with the routing redrawn per replay
+    tokens, dim, inter, experts, topk = 400, 7168, 256, 4, 2
+    g = torch.Generator(device=DEV).manual_seed(6)
+    w1 = (torch.randn(experts * 2 * inter, dim, generator=g, device=DEV) * 0.1).bfloat16()
+    w2 = (torch.randn(experts * dim, inter, generator=g, device=DEV) * 0.1).bfloat16()
+    w1q, w1s = aiter_amd.weight_per_128x128_quant(w1)
+    w2q, w2s = aiter_amd.weight_per_128x128_quant(w2)
+    w1q = aiter_amd.shuffle_weight(w1q.view(experts, 2 * inter, dim).view(torch.uint8)).view(dtypes.fp8)
+    w2q = aiter_amd.shuffle_weight(w2q.view(experts, dim, inter).view(torch.uint8)).view(dtypes.fp8)
+    w1s, w2s = w1s.view(experts, -1).contiguous(), w2s.view(experts, -1).contiguous()
+
+    def build():
+        return dict(x=torch.empty(tokens, dim, device=DEV, dtype=torch.bfloat16),
+                    score=torch.empty(tokens, experts, device=DEV))
+
+    def refill(t, i):
+        gg = torch.Generator(device=DEV).manual_seed(300 + i)
+        t["x"].copy_(torch.randn(tokens, dim, generator=gg, device=DEV).bfloat16())
+        t["score"].copy_(torch.randn(tokens, experts, generator=gg, device=DEV))
+
+    def run(t):
+        tw, ti = aiter_amd.fused_topk(t["x"], t["score"], topk, True)
+        out = aiter_amd.fused_moe(t["x"], w1q, w2q, tw, ti, quant_type=aiter_amd.QuantType.per_1x128,
+                                  w1_scale=w1s, w2_scale=w2s)
+        return [tw, ti, out]
+
+    replay_and_compare(build, refill, run)
