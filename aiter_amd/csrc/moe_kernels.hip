@@ -244,14 +244,14 @@ __global__ __launch_bounds__(1024) void moe_sort_scan_kernel(SortParams p)
     const int e   = threadIdx.x;
     int32_t   run = 0;
     if(e < p.experts)
-        for(int c0 = 0; c0 < p.chunks; c0 += 8) // eight counts requested together: one round trip, not eight
+        for(int c0 = 0; c0 < p.chunks; c0 += 32) // 32 counts requested together: one round trip, not 32
         {
-            int32_t n[8];
+            int32_t n[32];
 #pragma unroll
-            for(int i = 0; i < 8; ++i)
+            for(int i = 0; i < 32; ++i)
                 n[i] = c0 + i < p.chunks ? p.counts[(size_t)(c0 + i) * p.experts + e] : 0;
 #pragma unroll
-            for(int i = 0; i < 8; ++i)
+            for(int i = 0; i < 32; ++i)
                 if(c0 + i < p.chunks)
                 {
                     p.counts[(size_t)(c0 + i) * p.experts + e] = run; // position inside the expert's run
